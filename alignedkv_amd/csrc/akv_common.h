@@ -1,0 +1,94 @@
+// Shared device helpers of the AlignedKV HIP kernels (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/alignedkv.h"
+
+typedef uint32_t u32;
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+
+namespace akv {
+
+// ---- host-side error reporting -------------------------------------------------------------
+void set_error(const char *fmt, ...);
+int check_launch(const char *what);
+
+#define AKV_REQUIRE(cond, ...)            \
+    do {                                   \
+        if (!(cond)) {                     \
+            akv::set_error(__VA_ARGS__);   \
+            return AKV_ERR_INVALID;        \
+        }                                  \
+    } while (0)
+
+// ---- fp16 bit helpers ------------------------------------------------------------------------
+__device__ __forceinline__ float half_bits_to_float(u32 bits16) {
+    return __half2float(__ushort_as_half((unsigned short)bits16));
+}
+__device__ __forceinline__ float lo_half_to_float(u32 w) {
+    return __half2float(__ushort_as_half((unsigned short)(w & 0xffffu)));
+}
+__device__ __forceinline__ float hi_half_to_float(u32 w) {
+    return __half2float(__ushort_as_half((unsigned short)(w >> 16)));
+}
+__device__ __forceinline__ unsigned short float_to_half_bits(float f) {
+    return __half_as_ushort(__float2half_rn(f));
+}
+
+// ---- fetch levels ------------------------------------------------------------------------------
+// K: per (batch, head, channel); diff is computed in uint8 (reference: extension/csrc/K_cache.cu:211,249-250).
+__device__ __forceinline__ int k_level(unsigned char max_u8, unsigned char sum_u8) {
+    unsigned char diff = (unsigned char)(max_u8 - sum_u8);
+    return diff >= 8 ? 2 : (diff >= 4 ? 1 : 0);
+}
+// V: per (batch, head, token); `amin << 10` and the difference live in 16-bit signed integers
+// (reference: extension/csrc/V_cache.cu:195-197,211,250-251).
+__device__ __forceinline__ int v_level(unsigned char amin_u8, unsigned short s_bits) {
+    short a = (short)((unsigned short)((unsigned)amin_u8 << 10));
+    short diff = (short)((unsigned short)((unsigned short)a - s_bits));
+    return diff >= 0x0800 ? 2 : (diff >= 0x0400 ? 1 : 0);
+}
+
+// ---- 8 elements at a time ------------------------------------------------------------------------
+// Ha/Hb: high bytes of elements 0..3 / 4..7; M, L: the 4 mid / last bytes covering the same 8
+// elements (even element in the high nibble).  Skipped planes are passed as the substitution
+// bytes (M = 0x88888888, L = 0 for level 2; L = 0x88888888 for level 1), which reproduces
+// hi<<8|0x80 and hi<<8|mid<<4|0x8 (reference: extension/csrc/K_cache.cu:201-205,249-252).
+// acc[i] += value(element i) * x.
+__device__ __forceinline__ void fma8(float *acc, u32 Ha, u32 Hb, u32 M, u32 L, float x) {
+    u32 E = (M & 0xF0F0F0F0u) | ((L >> 4) & 0x0F0F0F0Fu);   // low bytes of elements 0,2,4,6
+    u32 O = ((M << 4) & 0xF0F0F0F0u) | (L & 0x0F0F0F0Fu);   // low bytes of elements 1,3,5,7
+    u32 w02 = __builtin_amdgcn_perm(Ha, E, 0x06010400u);
+    u32 w13 = __builtin_amdgcn_perm(Ha, O, 0x07010500u);
+    u32 w46 = __builtin_amdgcn_perm(Hb, E, 0x06030402u);
+    u32 w57 = __builtin_amdgcn_perm(Hb, O, 0x07030502u);
+    acc[0] = fmaf(lo_half_to_float(w02), x, acc[0]);
+    acc[2] = fmaf(hi_half_to_float(w02), x, acc[2]);
+    acc[1] = fmaf(lo_half_to_float(w13), x, acc[1]);
+    acc[3] = fmaf(hi_half_to_float(w13), x, acc[3]);
+    acc[4] = fmaf(lo_half_to_float(w46), x, acc[4]);
+    acc[6] = fmaf(hi_half_to_float(w46), x, acc[6]);
+    acc[5] = fmaf(lo_half_to_float(w57), x, acc[5]);
+    acc[7] = fmaf(hi_half_to_float(w57), x, acc[7]);
+}
+
+// Scalar reconstruction used by the generic (any-shape) kernels.
+__device__ __forceinline__ u32 rebuild_bits(u32 hi, u32 mid_nibble, u32 last_nibble, int level) {
+    u32 lo = level == 0 ? ((mid_nibble << 4) | last_nibble) : (level == 1 ? ((mid_nibble << 4) | 0x8u) : 0x80u);
+    return (hi << 8) | lo;
+}
+
+// ---- buffer resources: loads whose byte offset is >= num_records return 0 and fetch nothing ---
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, u32 num_bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)num_bytes, 0x00020000);
+}
+constexpr int kSkip = 0x7fffffff;   // an offset no plane slice reaches
+
+__device__ __forceinline__ float wave_xor_add(float v, int mask) { return v + __shfl_xor(v, mask, 64); }
+
+}  // namespace akv

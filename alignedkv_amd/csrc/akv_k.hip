@@ -1,0 +1,340 @@
+// K side of the AlignedKV hot path: plane writes (k_cache_save) and decode scores (k_cache_compute).
+//
+// Plane layout (reference: extension/k_cache_file.py:45-53): per (batch, head, block) a block of
+// d_block tokens is stored channel-major, first_8[d][slot] (d_block bytes per channel) and
+// mid_4/last_4[d][slot/2] (d_block/2 bytes per channel, even slot in the high nibble).
+//
+// Score kernel, tuned shape (d_block == 64, d_head in {64,128,256}): one wave owns one block.
+// A 16-byte load per lane covers 16 channels x 64 slots of first_8 (lane = 16 slots of one
+// channel), an 8-byte load per lane covers the same (channel, slots) of a nibble plane, so the
+// three planes of an element meet in one lane without any exchange.  The fetch level depends
+// only on the channel, i.e. on (load group, lane/4): nibble loads of skipped channels are issued
+// with an out-of-range buffer offset (they return 0 and fetch nothing) and OR-ed with the
+// substitution byte.  Each lane keeps 16 fp32 accumulators (its 16 slots); a reduce-scatter over
+// the 16 lanes that share the slots leaves one score per lane.
+#include "akv_common.h"
+
+namespace akv {
+
+// ------------------------------------------------------------------------------------------------
+// k_cache_save
+// ------------------------------------------------------------------------------------------------
+// grid (n_blocks * tiles_per_block, H, B), 256 threads; a workgroup transposes one tile of up to
+// 64 slots through LDS (dynamic LDS = tile_slots * (D + 2) halves) so that both the token-major
+// fp16 reads and the channel-major plane writes are coalesced.
+// reference: extension/csrc/K_cache.cu:19-58 (same destination bytes, written instead of accumulated).
+__global__ __launch_bounds__(256) void k_save_blocks_kernel(
+    uint8_t *__restrict__ first_8, uint8_t *__restrict__ mid_4, uint8_t *__restrict__ last_4,
+    const unsigned short *__restrict__ k_new, int n_max_blocks, int H, int D, int cb, int tile_slots,
+    int tiles_per_block, int start_block, int seqlen) {
+    extern __shared__ unsigned short tile[];   // [tile_slots][D + 2]
+    const int pitch = D + 2;
+    const int z = blockIdx.x / tiles_per_block, tile_id = blockIdx.x - z * tiles_per_block;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int slot0 = tile_id * tile_slots;                       // first slot of this tile in the block
+    const int t0 = z * cb + slot0;                                // first source token
+    const int nv = min(min(tile_slots, cb - slot0), seqlen - t0); // valid tokens of this tile
+    if (nv <= 0) return;
+    const int halfD = D >> 1;
+    const u32 *src32 = reinterpret_cast<const u32 *>(k_new);
+    for (int idx = threadIdx.x; idx < nv * halfD; idx += blockDim.x) {
+        int j = idx / halfD, dp = idx - j * halfD;
+        u32 w = src32[(((int64_t)b * seqlen + t0 + j) * H + h) * halfD + dp];
+        tile[j * pitch + 2 * dp] = (unsigned short)(w & 0xffffu);
+        tile[j * pitch + 2 * dp + 1] = (unsigned short)(w >> 16);
+    }
+    __syncthreads();
+    const int64_t blk_base = (((int64_t)b * H + h) * n_max_blocks + (start_block + z)) * (int64_t)D * (cb >> 1);
+    uint8_t *f8 = first_8 + blk_base * 2 + slot0;
+    uint8_t *m4 = mid_4 + blk_base + (slot0 >> 1);
+    uint8_t *l4 = last_4 + blk_base + (slot0 >> 1);
+    // first_8: 4 slots per thread
+    const int q4 = tile_slots >> 2;
+    for (int idx = threadIdx.x; idx < D * q4; idx += blockDim.x) {
+        int d = idx / q4, j = (idx - d * q4) * 4;
+        if (j + 3 < nv) {
+            u32 w = (u32)(tile[j * pitch + d] >> 8) | ((u32)(tile[(j + 1) * pitch + d] >> 8) << 8) |
+                    ((u32)(tile[(j + 2) * pitch + d] >> 8) << 16) | ((u32)(tile[(j + 3) * pitch + d] >> 8) << 24);
+            *reinterpret_cast<u32 *>(f8 + (int64_t)d * cb + j) = w;
+        } else {
+            for (int jj = j; jj < nv; ++jj) f8[(int64_t)d * cb + jj] = (uint8_t)(tile[jj * pitch + d] >> 8);
+        }
+    }
+    // nibble planes: 8 slots (4 bytes) per thread
+    const int q8 = tile_slots >> 3;
+    for (int idx = threadIdx.x; idx < D * q8; idx += blockDim.x) {
+        int d = idx / q8, j = (idx - d * q8) * 8;
+        if (j >= nv) continue;
+        u32 mw = 0, lw = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int je = j + 2 * i, jo = je + 1;
+            u32 le = je < nv ? (tile[je * pitch + d] & 0xffu) : 0u;
+            u32 lo = jo < nv ? (tile[jo * pitch + d] & 0xffu) : 0u;
+            mw |= ((le & 0xf0u) | (lo >> 4)) << (8 * i);
+            lw |= (((le & 0x0fu) << 4) | (lo & 0x0fu)) << (8 * i);
+        }
+        if (j + 7 < nv) {
+            *reinterpret_cast<u32 *>(m4 + (int64_t)d * (cb >> 1) + (j >> 1)) = mw;
+            *reinterpret_cast<u32 *>(l4 + (int64_t)d * (cb >> 1) + (j >> 1)) = lw;
+        } else {
+            int nbytes = (nv - j + 1) >> 1;
+            for (int i = 0; i < nbytes; ++i) {
+                m4[(int64_t)d * (cb >> 1) + (j >> 1) + i] = (uint8_t)(mw >> (8 * i));
+                l4[(int64_t)d * (cb >> 1) + (j >> 1) + i] = (uint8_t)(lw >> (8 * i));
+            }
+        }
+    }
+}
+
+// One token into slot `slot` of block `blk`: nibble insert (the other nibble of the byte is kept).
+// grid (H, B), D threads.  reference: extension/csrc/K_cache.cu:63-94.
+__global__ void k_save_token_kernel(uint8_t *__restrict__ first_8, uint8_t *__restrict__ mid_4,
+                                    uint8_t *__restrict__ last_4, const unsigned short *__restrict__ k_new,
+                                    int n_max_blocks, int H, int D, int cb, int blk, int slot) {
+    const int h = blockIdx.x, b = blockIdx.y;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        u32 bits = k_new[((int64_t)b * H + h) * D + d];
+        int64_t base = ((((int64_t)b * H + h) * n_max_blocks + blk) * D + d) * (int64_t)(cb >> 1);
+        first_8[base * 2 + slot] = (uint8_t)(bits >> 8);
+        uint8_t *pm = mid_4 + base + (slot >> 1);
+        uint8_t *pl = last_4 + base + (slot >> 1);
+        u32 mid = (bits >> 4) & 0xfu, last = bits & 0xfu;
+        if (slot & 1) {
+            *pm = (uint8_t)((*pm & 0xf0u) | mid);
+            *pl = (uint8_t)((*pl & 0xf0u) | last);
+        } else {
+            *pm = (uint8_t)((*pm & 0x0fu) | (mid << 4));
+            *pl = (uint8_t)((*pl & 0x0fu) | (last << 4));
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// k_cache_compute, tuned: d_block == 64
+// ------------------------------------------------------------------------------------------------
+template <int N>
+__device__ __forceinline__ void reduce_scatter_step(float *a, int lane_mask) {
+    const bool up = (threadIdx.x & lane_mask) != 0;
+#pragma unroll
+    for (int i = 0; i < N / 2; ++i) {
+        float send = up ? a[i] : a[i + N / 2];
+        float keep = up ? a[i + N / 2] : a[i];
+        a[i] = keep + __shfl_xor(send, lane_mask, 64);
+    }
+}
+
+// grid (ceil(n_blocks / (4*blocks_per_wave)), H, B), 256 threads (4 waves).
+template <int D, bool REF>
+__global__ __launch_bounds__(256) void k_compute_cb64_kernel(
+    const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
+    const uint8_t *__restrict__ sum_u8, const uint8_t *__restrict__ max_u8, const unsigned short *__restrict__ q,
+    unsigned short *__restrict__ s, uint8_t *__restrict__ levels_out, int n_blocks, int n_max_blocks, int H,
+    int blocks_per_wave, float scale) {
+    constexpr int CB = 64;
+    constexpr int NG = D / 16;            // load groups of 16 channels
+    constexpr int GC = NG < 8 ? NG : 8;   // groups in flight at a time
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int bh = b * H + h;
+    const int first_blk = (blockIdx.x * 4 + wave) * blocks_per_wave;
+    if (first_blk >= n_blocks) return;
+    const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
+
+    // per-lane channel data: channel of group g is g*16 + lane/4
+    float qf[NG];
+    u32 need_mid = 0, need_last = 0;
+    const unsigned char mx = REF ? 0 : max_u8[bh];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+        int c = g * 16 + (lane >> 2);
+        qf[g] = half_bits_to_float(q[(int64_t)bh * D + c]);
+        int lv = REF ? 0 : k_level(mx, sum_u8[(int64_t)bh * D + c]);
+        need_mid |= (lv < 2 ? 1u : 0u) << g;
+        need_last |= (lv == 0 ? 1u : 0u) << g;
+        if (levels_out != nullptr && blockIdx.x == 0 && wave == 0 && (lane & 3) == 0)
+            levels_out[(int64_t)bh * D + c] = (uint8_t)lv;
+    }
+
+    const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(first_8 + plane_off * 2, (u32)n_blocks * (D * CB));
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(mid_4 + plane_off, (u32)n_blocks * (D * CB / 2));
+    const __amdgpu_buffer_rsrc_t rL = make_rsrc(last_4 + plane_off, (u32)n_blocks * (D * CB / 2));
+    unsigned short *s_row = s + (int64_t)bh * ((int64_t)(n_blocks + 1) * CB);
+
+    for (int blk = first_blk; blk < end_blk; ++blk) {
+        float acc[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int g0 = 0; g0 < NG; g0 += GC) {
+            u32x4 hv[GC];
+            u32x2 mv[GC], lv[GC];
+#pragma unroll
+            for (int g = 0; g < GC; ++g) {
+                const int gg = g0 + g;
+                hv[g] = __builtin_amdgcn_raw_buffer_load_b128(rH, blk * (D * CB) + gg * 1024 + lane * 16, 0, 0);
+                int mo = ((need_mid >> gg) & 1u) ? blk * (D * CB / 2) + gg * 512 + lane * 8 : kSkip;
+                int lo = ((need_last >> gg) & 1u) ? blk * (D * CB / 2) + gg * 512 + lane * 8 : kSkip;
+                mv[g] = __builtin_amdgcn_raw_buffer_load_b64(rM, mo, 0, 0);
+                lv[g] = __builtin_amdgcn_raw_buffer_load_b64(rL, lo, 0, 0);
+            }
+#pragma unroll
+            for (int g = 0; g < GC; ++g) {
+                const int gg = g0 + g;
+                const u32 cm = ((need_mid >> gg) & 1u) ? 0u : 0x88888888u;                            // level 2
+                const u32 cl = (((need_mid >> gg) & 1u) && !((need_last >> gg) & 1u)) ? 0x88888888u : 0u;  // level 1
+                fma8(acc, hv[g].x, hv[g].y, mv[g].x | cm, lv[g].x | cl, qf[gg]);
+                fma8(acc + 8, hv[g].z, hv[g].w, mv[g].y | cm, lv[g].y | cl, qf[gg]);
+            }
+        }
+        // acc[i] is the partial score of slot (lane&3)*16 + i over this lane's channels
+        reduce_scatter_step<16>(acc, 32);
+        reduce_scatter_step<8>(acc, 16);
+        reduce_scatter_step<4>(acc, 8);
+        reduce_scatter_step<2>(acc, 4);
+        const int slot = (lane & 3) * 16 + ((lane & 32) ? 8 : 0) + ((lane & 16) ? 4 : 0) + ((lane & 8) ? 2 : 0) +
+                         ((lane & 4) ? 1 : 0);
+        s_row[blk * CB + slot] = float_to_half_bits(acc[0] * scale);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// k_cache_compute, any shape: one thread per slot pair, like the reference's launch
+// (extension/csrc/K_cache.cu:350-351) but with fp32 accumulation.
+// grid (n_blocks, H, B), d_block/2 threads.
+// ------------------------------------------------------------------------------------------------
+template <bool REF>
+__global__ void k_compute_generic_kernel(const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4,
+                                         const uint8_t *__restrict__ last_4, const uint8_t *__restrict__ sum_u8,
+                                         const uint8_t *__restrict__ max_u8, const unsigned short *__restrict__ q,
+                                         unsigned short *__restrict__ s, uint8_t *__restrict__ levels_out,
+                                         int n_blocks, int n_max_blocks, int H, int D, int cb, float scale) {
+    const int z = blockIdx.x, h = blockIdx.y, b = blockIdx.z, tx = threadIdx.x;
+    const int bh = b * H + h;
+    const unsigned char mx = REF ? 0 : max_u8[bh];
+    const int64_t base = ((int64_t)bh * n_max_blocks + z) * (int64_t)D * (cb >> 1);
+    float r1 = 0.f, r2 = 0.f;
+    for (int i = 0; i < D; ++i) {
+        int lv = REF ? 0 : k_level(mx, sum_u8[(int64_t)bh * D + i]);
+        if (levels_out != nullptr && z == 0 && tx == 0) levels_out[(int64_t)bh * D + i] = (uint8_t)lv;
+        int64_t row = base + (int64_t)i * (cb >> 1);
+        u32 h1 = first_8[row * 2 + 2 * tx], h2 = first_8[row * 2 + 2 * tx + 1];
+        u32 m = lv < 2 ? mid_4[row + tx] : 0u;
+        u32 l = lv == 0 ? last_4[row + tx] : 0u;
+        float qf = half_bits_to_float(q[(int64_t)bh * D + i]);
+        r1 = fmaf(half_bits_to_float(rebuild_bits(h1, m >> 4, l >> 4, lv)), qf, r1);
+        r2 = fmaf(half_bits_to_float(rebuild_bits(h2, m & 0xfu, l & 0xfu, lv)), qf, r2);
+    }
+    unsigned short *s_row = s + (int64_t)bh * ((int64_t)(n_blocks + 1) * cb);
+    s_row[z * cb + 2 * tx] = float_to_half_bits(r1 * scale);
+    s_row[z * cb + 2 * tx + 1] = float_to_half_bits(r2 * scale);
+}
+
+template <int D, bool REF>
+static void launch_k_cb64(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *sum_u8,
+                          const uint8_t *max_u8, const uint8_t *q, uint8_t *s, uint8_t *levels, int B, int H,
+                          int n_blocks, int n_max_blocks, float scale, hipStream_t st) {
+    // enough waves to fill 256 CUs several times over, a few blocks per wave to amortise set-up
+    int bpw = 1;
+    while (bpw < 4 && (int64_t)B * H * ((n_blocks + bpw * 2 - 1) / (bpw * 2)) >= 8192) bpw *= 2;
+    dim3 grid((n_blocks + 4 * bpw - 1) / (4 * bpw), H, B);
+    hipLaunchKernelGGL((k_compute_cb64_kernel<D, REF>), grid, dim3(256), 0, st, f8, m4, l4, sum_u8, max_u8,
+                       reinterpret_cast<const unsigned short *>(q), reinterpret_cast<unsigned short *>(s), levels,
+                       n_blocks, n_max_blocks, H, bpw, scale);
+}
+
+}  // namespace akv
+
+using namespace akv;
+
+extern "C" int akv_k_cache_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *k_new, int bsz,
+                                int n_kv_heads, int n_blocks, int n_max_blocks, int d_head, int d_block,
+                                int start_pos, int seqlen, akv_stream_t stream) {
+    AKV_REQUIRE(first_8 && mid_4 && last_4 && k_new, "k_cache_save: null pointer");
+    AKV_REQUIRE(bsz > 0 && n_kv_heads > 0 && d_head > 0 && d_block > 0 && n_max_blocks > 0,
+                "k_cache_save: non-positive dimension (bsz=%d heads=%d d_head=%d d_block=%d n_max_blocks=%d)", bsz,
+                n_kv_heads, d_head, d_block, n_max_blocks);
+    AKV_REQUIRE(d_block % 8 == 0 && d_head % 2 == 0, "k_cache_save: needs d_block %% 8 == 0 and even d_head (got %d, %d)",
+                d_block, d_head);
+    AKV_REQUIRE(start_pos >= 0 && seqlen >= 0 && n_blocks >= 0, "k_cache_save: negative start_pos/seqlen/n_blocks");
+    AKV_REQUIRE(bsz <= 65535 && n_kv_heads <= 65535, "k_cache_save: bsz/heads exceed the grid limit 65535");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (start_pos == 0 || seqlen % d_block == 0) {
+        if (n_blocks == 0) return AKV_OK;
+        const int start_block = start_pos / d_block;
+        AKV_REQUIRE((int64_t)(n_blocks - 1) * d_block < seqlen, "k_cache_save: n_blocks=%d needs more than seqlen=%d tokens",
+                    n_blocks, seqlen);
+        AKV_REQUIRE(start_block + n_blocks <= n_max_blocks, "k_cache_save: blocks %d..%d exceed n_max_blocks=%d",
+                    start_block, start_block + n_blocks, n_max_blocks);
+        const int tile_slots = d_block < 64 ? d_block : 64;
+        const int tiles_per_block = (d_block + tile_slots - 1) / tile_slots;
+        size_t lds = (size_t)tile_slots * (d_head + 2) * sizeof(unsigned short);
+        AKV_REQUIRE(lds <= 64 * 1024, "k_cache_save: d_head=%d too large for the staging tile (%zu bytes)", d_head, lds);
+        hipLaunchKernelGGL(k_save_blocks_kernel, dim3(n_blocks * tiles_per_block, n_kv_heads, bsz), dim3(256), lds, st,
+                           first_8, mid_4, last_4, reinterpret_cast<const unsigned short *>(k_new), n_max_blocks,
+                           n_kv_heads, d_head, d_block, tile_slots, tiles_per_block, start_block, seqlen);
+        return check_launch("k_cache_save");
+    }
+    if (seqlen == 1) {
+        const int blk = start_pos / d_block;
+        AKV_REQUIRE(blk < n_max_blocks, "k_cache_save: start_pos=%d beyond n_max_blocks=%d", start_pos, n_max_blocks);
+        hipLaunchKernelGGL(k_save_token_kernel, dim3(n_kv_heads, bsz), dim3(d_head < 256 ? d_head : 256), 0, st,
+                           first_8, mid_4, last_4, reinterpret_cast<const unsigned short *>(k_new), n_max_blocks,
+                           n_kv_heads, d_head, d_block, blk, start_pos - blk * d_block);
+        return check_launch("k_cache_save(token)");
+    }
+    // the reference launches nothing for this combination (extension/csrc/K_cache.cu:120,142)
+    return AKV_OK;
+}
+
+extern "C" int akv_k_cache_compute(const uint8_t *first_8, const uint8_t *mid_4, const uint8_t *last_4,
+                                   const uint8_t *sum_u8, const uint8_t *max_u8, const uint8_t *q, uint8_t *s_out,
+                                   uint8_t *levels_out, int bsz, int n_kv_heads, int n_blocks, int n_max_blocks,
+                                   int d_head, int d_block, int seqlen, float sqrt_dim, int reference,
+                                   akv_stream_t stream) {
+    (void)seqlen;
+    AKV_REQUIRE(first_8 && mid_4 && last_4 && q && s_out, "k_cache_compute: null pointer");
+    AKV_REQUIRE(reference || (sum_u8 && max_u8), "k_cache_compute: null exponent-sum pointer");
+    AKV_REQUIRE(bsz > 0 && n_kv_heads > 0 && d_head > 0 && d_block > 0 && n_max_blocks > 0 && n_blocks >= 0,
+                "k_cache_compute: bad dimension (bsz=%d heads=%d d_head=%d d_block=%d n_blocks=%d n_max_blocks=%d)", bsz,
+                n_kv_heads, d_head, d_block, n_blocks, n_max_blocks);
+    AKV_REQUIRE(n_blocks <= n_max_blocks, "k_cache_compute: n_blocks=%d > n_max_blocks=%d", n_blocks, n_max_blocks);
+    AKV_REQUIRE(d_block % 2 == 0 && d_block / 2 <= 1024, "k_cache_compute: d_block must be even and <= 2048");
+    AKV_REQUIRE(bsz <= 65535 && n_kv_heads <= 65535, "k_cache_compute: bsz/heads exceed the grid limit 65535");
+    AKV_REQUIRE((int64_t)n_max_blocks * d_head * d_block < (int64_t)1 << 31,
+                "k_cache_compute: one (batch, head) slice of first_8 must stay below 2 GiB");
+    if (n_blocks == 0) return AKV_OK;   // reference returns the uninitialised tensor, K_cache.cu:331-333
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // the reference multiplies by __float2half2_rn(sqrt_dim): the scale is rounded to fp16
+    const float scale = __half2float(__float2half_rn(sqrt_dim));
+    const bool ref = reference != 0;
+#define AKV_K_TUNED(DD)                                                                                          \
+    if (ref)                                                                                                     \
+        launch_k_cb64<DD, true>(first_8, mid_4, last_4, sum_u8, max_u8, q, s_out, levels_out, bsz, n_kv_heads,   \
+                                n_blocks, n_max_blocks, scale, st);                                              \
+    else                                                                                                         \
+        launch_k_cb64<DD, false>(first_8, mid_4, last_4, sum_u8, max_u8, q, s_out, levels_out, bsz, n_kv_heads,  \
+                                 n_blocks, n_max_blocks, scale, st);
+    if (d_block == 64 && d_head == 128) {
+        AKV_K_TUNED(128)
+    } else if (d_block == 64 && d_head == 64) {
+        AKV_K_TUNED(64)
+    } else if (d_block == 64 && d_head == 256) {
+        AKV_K_TUNED(256)
+    } else {
+        dim3 grid(n_blocks, n_kv_heads, bsz), block(d_block / 2);
+        if (ref)
+            hipLaunchKernelGGL(k_compute_generic_kernel<true>, grid, block, 0, st, first_8, mid_4, last_4, sum_u8,
+                               max_u8, reinterpret_cast<const unsigned short *>(q),
+                               reinterpret_cast<unsigned short *>(s_out), levels_out, n_blocks, n_max_blocks,
+                               n_kv_heads, d_head, d_block, scale);
+        else
+            hipLaunchKernelGGL(k_compute_generic_kernel<false>, grid, block, 0, st, first_8, mid_4, last_4, sum_u8,
+                               max_u8, reinterpret_cast<const unsigned short *>(q),
+                               reinterpret_cast<unsigned short *>(s_out), levels_out, n_blocks, n_max_blocks,
+                               n_kv_heads, d_head, d_block, scale);
+    }
+#undef AKV_K_TUNED
+    return check_launch("k_cache_compute");
+}

@@ -1,0 +1,162 @@
+"""Drop-in for the reference's extension/KV_cache_cpp_extention.py: exposes `cuda_module` with the
+five ops k_cache_save, k_cache_compute, v_cache_save, v_cache_test_compute, v_cache_compute
+(reference binding: extension/csrc/KV_cache_ops.cpp:69-75), same positional signatures and the
+same "every tensor crosses as torch.uint8" convention.
+
+Here the ops are thin marshalling over the C ABI of libalignedkv_hip.so (include/alignedkv.h):
+torch supplies device memory and the current stream, the arithmetic is in the HIP library.
+Nothing is compiled at import time and there is no fallback implementation.
+"""
+from __future__ import annotations
+
+import torch
+
+from .._lib import check, load_library
+
+
+def _stream_ptr(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _require(name: str, t: torch.Tensor, min_bytes: int, device=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name}: expected a torch.Tensor, got {type(t).__name__}")
+    if t.dtype != torch.uint8:
+        raise RuntimeError(f"{name}: expected dtype torch.uint8 (pass .view(torch.uint8)), got {t.dtype}")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name}: expected a tensor on the GPU, got device {t.device}")
+    if device is not None and t.device != device:
+        raise RuntimeError(f"{name}: on {t.device}, other arguments on {device}")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name}: must be contiguous")
+    if t.numel() < min_bytes:
+        raise RuntimeError(f"{name}: holds {t.numel()} bytes, the scalar arguments imply {min_bytes}")
+
+
+class _AlignedKVModule:
+    """The object bound to the name `cuda_module`."""
+
+    def __init__(self):
+        self._workspaces = {}
+
+    def _workspace(self, device, nbytes: int) -> torch.Tensor:
+        # one scratch buffer per (device, stream): calls on one stream are ordered, so they can share it
+        key = (device, torch.cuda.current_stream(device).cuda_stream)
+        ws = self._workspaces.get(key)
+        if ws is None or ws.numel() < nbytes:
+            ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+            self._workspaces[key] = ws
+        return ws
+
+    # ---- K ---------------------------------------------------------------------------------
+    def k_cache_save(self, k_cache_first_8, k_cache_mid_4, k_cache_last_4, k_new, bsz, n_kv_heads, n_blocks,
+                     n_max_blocks, d_head, d_block, start_pos, seqlen):
+        lib = load_library()
+        dev = k_new.device if isinstance(k_new, torch.Tensor) else None
+        plane = bsz * n_kv_heads * n_max_blocks * d_head * d_block
+        _require("k_cache_first_8", k_cache_first_8, plane, dev)
+        _require("k_cache_mid_4", k_cache_mid_4, plane // 2, dev)
+        _require("k_cache_last_4", k_cache_last_4, plane // 2, dev)
+        _require("k_new", k_new, bsz * seqlen * n_kv_heads * d_head * 2, dev)
+        with torch.cuda.device(dev):
+            check(lib.akv_k_cache_save(_ptr(k_cache_first_8), _ptr(k_cache_mid_4), _ptr(k_cache_last_4), _ptr(k_new),
+                                       bsz, n_kv_heads, n_blocks, n_max_blocks, d_head, d_block, start_pos, seqlen,
+                                       _stream_ptr(dev)), lib)
+
+    def k_cache_compute(self, k_cache_first_8, k_cache_mid_4, k_cache_last_4, k_column_max_multiply_q,
+                        k_column_max_multiply_q_max, q, bsz, n_kv_heads, n_blocks, n_max_blocks, d_head, d_block,
+                        seqlen, sqrt_dim, reference, levels_out=None):
+        lib = load_library()
+        dev = q.device if isinstance(q, torch.Tensor) else None
+        plane = bsz * n_kv_heads * n_max_blocks * d_head * d_block
+        _require("k_cache_first_8", k_cache_first_8, plane, dev)
+        _require("k_cache_mid_4", k_cache_mid_4, plane // 2, dev)
+        _require("k_cache_last_4", k_cache_last_4, plane // 2, dev)
+        _require("k_column_max_multiply_q", k_column_max_multiply_q, bsz * n_kv_heads * d_head, dev)
+        _require("k_column_max_multiply_q_max", k_column_max_multiply_q_max, bsz * n_kv_heads, dev)
+        _require("q", q, bsz * n_kv_heads * d_head * 2, dev)
+        if levels_out is not None:
+            _require("levels_out", levels_out, bsz * n_kv_heads * d_head, dev)
+        s = torch.empty((bsz, n_kv_heads, 1, (n_blocks + 1) * d_block * 2), dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            check(lib.akv_k_cache_compute(_ptr(k_cache_first_8), _ptr(k_cache_mid_4), _ptr(k_cache_last_4),
+                                          _ptr(k_column_max_multiply_q), _ptr(k_column_max_multiply_q_max), _ptr(q),
+                                          _ptr(s), _ptr(levels_out), bsz, n_kv_heads, n_blocks, n_max_blocks, d_head,
+                                          d_block, seqlen, float(sqrt_dim), int(bool(reference)), _stream_ptr(dev)),
+                  lib)
+        return s
+
+    # ---- V ---------------------------------------------------------------------------------
+    def v_cache_save(self, v_cache_first_8, v_cache_mid_4, v_cache_last_4, v_new, bsz, n_local_kv_heads, max_seq_len,
+                     head_dim, start_pos, seq_len):
+        lib = load_library()
+        if not isinstance(v_new, torch.Tensor) or v_new.dim() != 4:
+            raise RuntimeError("v_new: expected a 4-d uint8 view [bsz, seqlen, heads, head_dim*2]")
+        dev = v_new.device
+        plane = bsz * n_local_kv_heads * max_seq_len * head_dim
+        v_new_seq = v_new.size(1)
+        _require("v_cache_first_8", v_cache_first_8, plane, dev)
+        _require("v_cache_mid_4", v_cache_mid_4, plane // 2, dev)
+        _require("v_cache_last_4", v_cache_last_4, plane // 2, dev)
+        _require("v_new", v_new, bsz * v_new_seq * n_local_kv_heads * head_dim * 2, dev)
+        with torch.cuda.device(dev):
+            check(lib.akv_v_cache_save(_ptr(v_cache_first_8), _ptr(v_cache_mid_4), _ptr(v_cache_last_4), _ptr(v_new),
+                                       bsz, n_local_kv_heads, max_seq_len, head_dim, start_pos, seq_len, v_new_seq,
+                                       _stream_ptr(dev)), lib)
+
+    def v_cache_test_compute(self, v_cache_first_8, v_cache_mid_4, v_cache_last_4, test_s_value, test_s_index, bsz,
+                             n_local_kv_heads, max_seq_len, head_dim, top_max_k):
+        lib = load_library()
+        dev = test_s_value.device if isinstance(test_s_value, torch.Tensor) else None
+        plane = bsz * n_local_kv_heads * max_seq_len * head_dim
+        _require("v_cache_first_8", v_cache_first_8, plane, dev)
+        _require("test_s_value", test_s_value, bsz * n_local_kv_heads * top_max_k * 2, dev)
+        _require("test_s_index", test_s_index, bsz * n_local_kv_heads * top_max_k * 4, dev)
+        test_o = torch.empty((bsz, n_local_kv_heads, 1, head_dim * 2), dtype=torch.uint8, device=dev)
+        with torch.cuda.device(dev):
+            check(lib.akv_v_cache_test_compute(_ptr(v_cache_first_8), _ptr(v_cache_mid_4), _ptr(v_cache_last_4),
+                                               _ptr(test_s_value), _ptr(test_s_index), _ptr(test_o), bsz,
+                                               n_local_kv_heads, max_seq_len, head_dim, top_max_k, _stream_ptr(dev)),
+                  lib)
+        return test_o
+
+    def v_cache_compute(self, v_cache_first_8, v_cache_mid_4, v_cache_last_4, s, s_exp_expect_alignment_min, bsz,
+                        n_local_kv_heads, max_seq_len, head_dim, s_last_dim, start_pos_add_seqlen, reference,
+                        levels_out=None):
+        lib = load_library()
+        dev = v_cache_first_8.device if isinstance(v_cache_first_8, torch.Tensor) else None
+        plane = bsz * n_local_kv_heads * max_seq_len * head_dim
+        n_tok = start_pos_add_seqlen
+        _require("v_cache_first_8", v_cache_first_8, plane, dev)
+        _require("v_cache_mid_4", v_cache_mid_4, plane // 2, dev)
+        _require("v_cache_last_4", v_cache_last_4, plane // 2, dev)
+        # `s` may be a sliced view (row stride s_last_dim, reference: extension/v_cache_file.py:150,184):
+        # only its base pointer and the stride argument are used, like in the reference op
+        if not isinstance(s, torch.Tensor) or s.dtype != torch.uint8 or not s.is_cuda:
+            raise RuntimeError("s: expected a uint8 view of the fp16 probabilities on the GPU")
+        if n_tok > 0:
+            if s.stride(-1) != 1:
+                raise RuntimeError("s: innermost dimension must be dense")
+            span = ((bsz * n_local_kv_heads - 1) * s_last_dim + n_tok) * 2
+            avail = s.untyped_storage().nbytes() - s.storage_offset()
+            if span > avail:
+                raise RuntimeError(f"s: rows of stride {s_last_dim} halves need {span} bytes, storage has {avail}")
+        _require("s_exp_expect_alignment_min", s_exp_expect_alignment_min, bsz * n_local_kv_heads, dev)
+        if levels_out is not None:
+            _require("levels_out", levels_out, bsz * n_local_kv_heads * n_tok, dev)
+        o = torch.empty((bsz, n_local_kv_heads, 1, head_dim * 2), dtype=torch.uint8, device=dev)
+        need = lib.akv_v_cache_compute_workspace_bytes(bsz, n_local_kv_heads, head_dim, n_tok)
+        ws = self._workspace(dev, need)
+        with torch.cuda.device(dev):
+            check(lib.akv_v_cache_compute(_ptr(v_cache_first_8), _ptr(v_cache_mid_4), _ptr(v_cache_last_4), _ptr(s),
+                                          _ptr(s_exp_expect_alignment_min), _ptr(o), _ptr(levels_out), _ptr(ws),
+                                          ws.numel(), bsz, n_local_kv_heads, max_seq_len, head_dim, s_last_dim,
+                                          n_tok, int(bool(reference)), _stream_ptr(dev)), lib)
+        return o
+
+
+cuda_module = _AlignedKVModule()

@@ -1,0 +1,123 @@
+/*
+ * alignedkv.h -- C ABI of the MI355X (gfx950) AlignedKV library, libalignedkv_hip.so.
+ *
+ * The five akv_* ops below are what the reference's Python layer binds through pybind11 as
+ * `cuda_module` (reference: extension/csrc/KV_cache_ops.cpp:69-75, loaded by
+ * extension/KV_cache_cpp_extention.py:6-9).  Every argument that the reference passes as a
+ * torch.uint8 tensor is a plain device pointer here; outputs the reference allocates with
+ * torch::empty are caller-allocated.  Scalar arguments keep the reference's names, order and meaning.
+ *
+ * Conventions
+ *   - all pointers are device pointers on the current HIP device; `stream` is a hipStream_t
+ *     (NULL = the default stream); every call is asynchronous on that stream;
+ *   - fp16 tensors are passed as bytes (little endian halves), as in the reference;
+ *   - return value 0 = launched; non-zero = rejected, nothing was launched and
+ *     akv_last_error() returns a description (thread local);
+ *   - plane layouts (extension/k_cache_file.py:45-53, extension/v_cache_file.py:46-54):
+ *       K first_8 [bsz, n_kv_heads, n_max_blocks, d_head, d_block]      uint8
+ *       K mid_4 / last_4 [bsz, n_kv_heads, n_max_blocks, d_head, d_block/2]  two slots per byte,
+ *                                                                      even slot in the high nibble
+ *       V first_8 [bsz, n_kv_heads, max_seq_len, head_dim]             uint8
+ *       V mid_4 / last_4 [bsz, n_kv_heads, max_seq_len, head_dim/2]    even channel in the high nibble
+ *   - fetch levels: 0 = all planes, 1 = last_4 not fetched (replaced by 0x8), 2 = mid_4 and
+ *     last_4 not fetched (low byte replaced by 0x80).
+ */
+#ifndef ALIGNEDKV_H
+#define ALIGNEDKV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *akv_stream_t; /* hipStream_t */
+
+#if defined(__GNUC__)
+#define AKV_API __attribute__((visibility("default")))
+#else
+#define AKV_API
+#endif
+
+#define AKV_OK 0
+#define AKV_ERR_INVALID 1     /* bad argument (null pointer, unsupported shape, size mismatch) */
+#define AKV_ERR_LAUNCH 2      /* the HIP runtime refused the launch */
+
+/* Library version (major*100 + minor). */
+AKV_API int akv_version(void);
+
+/* Description of the last non-zero return on this thread ("" if none). */
+AKV_API const char *akv_last_error(void);
+
+/*
+ * Replaces k_cache_save (reference: extension/csrc/KV_cache_ops.cpp:5-16, extension/csrc/K_cache.cu:97-164).
+ * k_new: fp16 [bsz, seqlen, n_kv_heads, d_head] contiguous.
+ * start_pos == 0 or seqlen % d_block == 0: writes blocks start_pos/d_block .. +n_blocks from tokens
+ * 0 .. min(n_blocks*d_block, seqlen) of k_new.  Otherwise, seqlen == 1: inserts one token at slot
+ * start_pos % d_block of block start_pos / d_block.  Nibble bytes are written, not accumulated
+ * (identical to the reference's `+=` on zero-initialised planes).  Needs d_block % 8 == 0, d_head % 2 == 0.
+ */
+AKV_API int akv_k_cache_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *k_new,
+                     int bsz, int n_kv_heads, int n_blocks, int n_max_blocks, int d_head, int d_block,
+                     int start_pos, int seqlen, akv_stream_t stream);
+
+/*
+ * Replaces k_cache_compute (reference: extension/csrc/KV_cache_ops.cpp:18-32, extension/csrc/K_cache.cu:314-395).
+ * k_column_max_multiply_q: uint8 [bsz, 1, n_kv_heads, d_head]; k_column_max_multiply_q_max: uint8
+ * [bsz, 1, n_kv_heads, 1]; q: fp16 [bsz, 1, n_kv_heads, d_head].
+ * s_out: fp16 [bsz, n_kv_heads, 1, (n_blocks+1)*d_block] (the tensor the reference returns); entries
+ * < n_blocks*d_block are written, the last d_block entries of every row are left untouched.
+ * s[b,h,t] = fp16( (sum_d khat[t,d]*q[d]) * half(sqrt_dim) ), fp32 accumulation.  `sqrt_dim` is the
+ * reciprocal 1/sqrt(d_head) as in the reference.  `seqlen` is accepted for signature parity and unused.
+ * levels_out (optional, may be NULL): uint8 [bsz, n_kv_heads, d_head], the fetch level each channel used.
+ */
+AKV_API int akv_k_cache_compute(const uint8_t *first_8, const uint8_t *mid_4, const uint8_t *last_4,
+                        const uint8_t *k_column_max_multiply_q, const uint8_t *k_column_max_multiply_q_max,
+                        const uint8_t *q, uint8_t *s_out, uint8_t *levels_out,
+                        int bsz, int n_kv_heads, int n_blocks, int n_max_blocks, int d_head, int d_block,
+                        int seqlen, float sqrt_dim, int reference, akv_stream_t stream);
+
+/*
+ * Replaces v_cache_save (reference: extension/csrc/KV_cache_ops.cpp:34-43, extension/csrc/V_cache.cu:44-80).
+ * v_new: fp16 [bsz, v_new_seq, n_local_kv_heads, head_dim] contiguous (v_new_seq = v_new.size(1) in the
+ * reference); its first seq_len tokens are stored at rows start_pos .. start_pos+seq_len.
+ */
+AKV_API int akv_v_cache_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *v_new,
+                     int bsz, int n_local_kv_heads, int max_seq_len, int head_dim, int start_pos,
+                     int seq_len, int v_new_seq, akv_stream_t stream);
+
+/*
+ * Replaces v_cache_test_compute (reference: extension/csrc/KV_cache_ops.cpp:45-54, extension/csrc/V_cache.cu:125-168).
+ * test_s_value: fp16 [bsz, heads, 1, top_max_k]; test_s_index: int32 [bsz, heads, 1, top_max_k];
+ * test_o_out: fp16 [bsz, heads, 1, head_dim].
+ * test_o[b,h,d] = fp16( sum_i s_i * |fp16(first_8[b,h,idx_i*top_max_k+i,d]<<8 | 0x80)| ).
+ * Token indices must lie in [0, max_seq_len).
+ */
+AKV_API int akv_v_cache_test_compute(const uint8_t *first_8, const uint8_t *mid_4, const uint8_t *last_4,
+                             const uint8_t *test_s_value, const uint8_t *test_s_index, uint8_t *test_o_out,
+                             int bsz, int n_local_kv_heads, int max_seq_len, int head_dim, int top_max_k,
+                             akv_stream_t stream);
+
+/* Bytes of device scratch akv_v_cache_compute needs for this shape (split-sequence partial sums). */
+AKV_API size_t akv_v_cache_compute_workspace_bytes(int bsz, int n_local_kv_heads, int head_dim, int n_tokens);
+
+/*
+ * Replaces v_cache_compute (reference: extension/csrc/KV_cache_ops.cpp:56-67, extension/csrc/V_cache.cu:310-374).
+ * s: fp16, row (b,h) starts at element (b*heads + h)*s_last_dim; s_exp_expect_alignment_min: uint8, entry
+ * b*heads + h is used; o_out: fp16 [bsz, heads, 1, head_dim].
+ * o[b,h,d] = fp16( sum_{t < start_pos_add_seqlen} vhat[t,d]*s[t] ), fp32 accumulation.
+ * levels_out (optional): uint8 [bsz, heads, start_pos_add_seqlen], the fetch level each token used.
+ * workspace: >= akv_v_cache_compute_workspace_bytes(...) bytes, 256-byte aligned, private to this call
+ * until the stream has passed it.
+ */
+AKV_API int akv_v_cache_compute(const uint8_t *first_8, const uint8_t *mid_4, const uint8_t *last_4,
+                        const uint8_t *s, const uint8_t *s_exp_expect_alignment_min, uint8_t *o_out,
+                        uint8_t *levels_out, void *workspace, size_t workspace_bytes,
+                        int bsz, int n_local_kv_heads, int max_seq_len, int head_dim, int s_last_dim,
+                        int start_pos_add_seqlen, int reference, akv_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ALIGNEDKV_H */
