@@ -25,3 +25,14 @@ def ulp_diff_fp16(a, b):
         u = np.asarray(x, np.float16).view(np.uint16).astype(np.int32)
         return np.where(u & 0x8000, -(u & 0x7FFF), u)
     return np.abs(key(a) - key(b))
+
+
+def assert_close_fp16(got, want, abs_floor):
+    """|got - want| <= one fp16 spacing at |want| + abs_floor.  The floor covers the fp32
+    accumulation-order noise of a dot product whose result is much smaller than its terms."""
+    g = np.asarray(got, np.float16).astype(np.float64)
+    w = np.asarray(want, np.float16).astype(np.float64)
+    spacing = np.abs(np.spacing(np.asarray(want, np.float16))).astype(np.float64)
+    err = np.abs(g - w)
+    bad = err > spacing + abs_floor
+    assert not bad.any(), f"max err {err.max():.3e} (allowed {float((spacing + abs_floor)[err.argmax()]):.3e}) at {int(bad.sum())} entries"
