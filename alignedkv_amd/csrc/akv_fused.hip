@@ -1,0 +1,486 @@
+// Fused AlignedKV decode step: append one token per sequence and attend over the whole cache in
+// four launches (K pass, middle, V pass, combine) instead of the reference's three custom launches
+// plus ~25 small framework kernels per layer (reference: model/KVCache_AlignedKV.py:101-124,
+// extension/k_cache_file.py:97-118,132-159, extension/v_cache_file.py:97-116,119-190).
+//
+//   K pass   scores of the flushed blocks; the fetch level of every channel is derived in the
+//            kernel from q, the column-max exponents and the new key (k_cache_file.py:98-99,136-138)
+//   middle   one workgroup per (batch, head): appends the token to the fp16 rest buffers and
+//            updates the column maxima, scores of the unflushed tail, mask, fp32 softmax -> fp16
+//            probabilities, arg-max of every residue class mod top_max_k, the output-magnitude
+//            probe, and the tail's share of the output
+//   V pass   split over the sequence; the alignment threshold of the (batch, head) is derived in
+//            the kernel from the probe exponents and the V column maxima (v_cache_file.py:156-160)
+//   combine  adds the chunk partials in a fixed order, rounds to fp16 and adds the fp16 tail part
+// On a step that fills the rest buffer (64 tokens) a persist kernel and the two plane-write kernels
+// run first, exactly as the reference flushes before it computes.
+#include "akv_cores.h"
+
+namespace akv {
+
+// defined in akv_k.hip / akv_v.hip
+int launch_k_save_blocks(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *k_new, int bsz, int heads,
+                         int n_blocks, int n_max_blocks, int d_head, int d_block, int start_pos, int seqlen,
+                         hipStream_t st);
+int launch_v_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *v_new, int bsz, int heads,
+                  int max_seq_len, int head_dim, int start_pos, int seq_len, int v_new_seq, hipStream_t st);
+
+__device__ __forceinline__ u32 exp_field(u32 half_bits) { return (half_bits >> 10) & 0x1fu; }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------------
+// persist (flush steps only): token -> rest buffers, column maxima.  grid (B*H), D threads.
+// ------------------------------------------------------------------------------------------------
+__global__ void fused_persist_kernel(const unsigned short *__restrict__ k_new, const unsigned short *__restrict__ v_new,
+                                     unsigned short *__restrict__ restk, unsigned short *__restrict__ restv,
+                                     uint8_t *__restrict__ kcm, uint8_t *__restrict__ vcm, int H, int D, int cb, int slot) {
+    const int bh = blockIdx.x, b = bh / H, h = bh - b * H;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        u32 kb = k_new[(int64_t)bh * D + d], vb = v_new[(int64_t)bh * D + d];
+        int64_t at = (((int64_t)b * cb + slot) * H + h) * D + d;
+        restk[at] = (unsigned short)kb;
+        restv[at] = (unsigned short)vb;
+        kcm[(int64_t)bh * D + d] = (uint8_t)max((u32)kcm[(int64_t)bh * D + d], exp_field(kb));
+        vcm[(int64_t)bh * D + d] = (uint8_t)max((u32)vcm[(int64_t)bh * D + d], exp_field(vb));
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// K pass.  grid (ceil(n_blocks / (4*blocks_per_wave)), H, B), 256 threads.
+// ------------------------------------------------------------------------------------------------
+template <int D, bool REF>
+__global__ __launch_bounds__(256) void fused_k_pass_kernel(
+    const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
+    const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
+    unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, int n_blocks, int n_max_blocks, int H,
+    int row_stride, int blocks_per_wave, float scale) {
+    constexpr int CB = 64;
+    constexpr int NG = D / 16;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int bh = b * H + h;
+    const int first_blk = (blockIdx.x * 4 + wave) * blocks_per_wave;
+    if (first_blk >= n_blocks) return;
+    const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
+
+    float qf[NG];
+    u32 esum[NG];
+    u32 mx = 0;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+        const int c = g * 16 + (lane >> 2);
+        const u32 qb = q[(int64_t)bh * D + c];
+        qf[g] = half_bits_to_float(qb);
+        // column max including the token appended by this step
+        const u32 cm = max((u32)kcm[(int64_t)bh * D + c], exp_field(k_new[(int64_t)bh * D + c]));
+        esum[g] = (exp_field(qb) + cm) & 0xffu;
+        mx = max(mx, esum[g]);
+    }
+#pragma unroll
+    for (int m = 4; m <= 32; m <<= 1) mx = max(mx, (u32)__shfl_xor((int)mx, m, 64));
+    u32 need_mid = 0, need_last = 0;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+        const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)esum[g]);
+        need_mid |= (lv < 2 ? 1u : 0u) << g;
+        need_last |= (lv == 0 ? 1u : 0u) << g;
+        if (levels_out != nullptr && blockIdx.x == 0 && wave == 0 && (lane & 3) == 0)
+            levels_out[(int64_t)bh * D + g * 16 + (lane >> 2)] = (uint8_t)lv;
+    }
+    const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
+    k_score_blocks<D>(first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
+                      need_mid, need_last, scores + (int64_t)bh * row_stride, scale);
+}
+
+// ------------------------------------------------------------------------------------------------
+// middle.  grid (B*H), 256 threads.
+// ------------------------------------------------------------------------------------------------
+struct MiddleArgs {
+    const unsigned short *q, *k_new, *v_new, *mask;
+    unsigned short *restk, *restv, *scores, *probs, *otail;
+    uint8_t *kcm, *vcm, *toe;
+    const uint8_t *v_first_8;
+    int H, cb, max_seq_len, row_stride, mask_stride;
+    int R;        // flushed tokens (multiple of cb)
+    int nrest;    // tokens in the rest buffer including the one of this step (0 on a flush step)
+    int top_k;
+    int persist;  // this kernel appends the token (no flush happened in this step)
+};
+
+__device__ __forceinline__ float block_reduce(float v, bool is_max, float *red) {
+    v = is_max ? wave_max(v) : wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return is_max ? fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])) : ((red[0] + red[1]) + (red[2] + red[3]));
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
+    __shared__ float red[4];
+    __shared__ unsigned short tail_s[64];     // fp16 scores of the tail (mask not yet added)
+    __shared__ float tail_p[64];              // probabilities of the tail
+    __shared__ float cand_v[64][33];
+    __shared__ int cand_t[64][33];
+    __shared__ float probe_p[64];
+    __shared__ int probe_t[64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bh = blockIdx.x, b = bh / a.H, h = bh - b * a.H;
+    const int R = a.R, nrest = a.nrest, newest = nrest - 1;
+    const unsigned short *qrow = a.q + (int64_t)bh * D;
+    const unsigned short *knew = a.k_new + (int64_t)bh * D;
+    const unsigned short *vnew = a.v_new + (int64_t)bh * D;
+    unsigned short *srow = a.scores + (int64_t)bh * a.row_stride;
+    unsigned short *prow = a.probs + (int64_t)bh * a.row_stride;
+    const unsigned short *mrow = a.mask ? a.mask + (int64_t)b * a.mask_stride : nullptr;
+
+    // (a) append the token: rest buffers and column maxima (extension/k_cache_file.py:98-101)
+    if (a.persist) {
+        for (int d = tid; d < D; d += 256) {
+            const u32 kb = knew[d], vb = vnew[d];
+            const int64_t at = (((int64_t)b * a.cb + newest) * a.H + h) * D + d;
+            a.restk[at] = (unsigned short)kb;
+            a.restv[at] = (unsigned short)vb;
+            a.kcm[(int64_t)bh * D + d] = (uint8_t)max((u32)a.kcm[(int64_t)bh * D + d], exp_field(kb));
+            a.vcm[(int64_t)bh * D + d] = (uint8_t)max((u32)a.vcm[(int64_t)bh * D + d], exp_field(vb));
+        }
+    }
+    // (b) scores of the tail: fp16(fp16(q.k) / sqrt(D)), the two roundings of an fp16 matmul followed by
+    //     an fp16 division (extension/k_cache_file.py:156)
+    const float sqrt_d = sqrtf((float)D);
+    for (int r = wave; r < nrest; r += 4) {
+        const unsigned short *krow = (r == newest && a.persist) ? knew : a.restk + (((int64_t)b * a.cb + r) * a.H + h) * D;
+        float part = 0.f;
+        for (int c = lane; c < D; c += 64) part = fmaf(half_bits_to_float(krow[c]), half_bits_to_float(qrow[c]), part);
+        part = wave_sum(part);
+        if (lane == 0) {
+            const float dot16 = half_bits_to_float(float_to_half_bits(part));
+            const unsigned short sc = float_to_half_bits(dot16 / sqrt_d);
+            tail_s[r] = sc;
+            srow[R + r] = sc;
+        }
+    }
+    __syncthreads();
+
+    // (c) softmax over [0, L): scores + mask in fp16, softmax in fp32, probabilities in fp16
+    //     (model/KVCache_AlignedKV.py:119-121).  Flushed part 8 tokens per thread and iteration.
+    auto masked = [&](u32 sbits, int t) -> float {
+        if (mrow == nullptr) return half_bits_to_float(sbits);
+        return half_bits_to_float(float_to_half_bits(half_bits_to_float(sbits) + half_bits_to_float(mrow[t])));
+    };
+    const int nvec = R >> 3;
+    float m = -INFINITY;
+    for (int i = tid; i < nvec; i += 256) {
+        const u32x4 w = *reinterpret_cast<const u32x4 *>(srow + i * 8);
+        const u32 ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            m = fmaxf(m, masked(ww[j] & 0xffffu, i * 8 + 2 * j));
+            m = fmaxf(m, masked(ww[j] >> 16, i * 8 + 2 * j + 1));
+        }
+    }
+    if (tid < nrest) m = fmaxf(m, masked(tail_s[tid], R + tid));
+    m = block_reduce(m, true, red);
+    float sum = 0.f;
+    for (int i = tid; i < nvec; i += 256) {
+        const u32x4 w = *reinterpret_cast<const u32x4 *>(srow + i * 8);
+        const u32 ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            sum += expf(masked(ww[j] & 0xffffu, i * 8 + 2 * j) - m);
+            sum += expf(masked(ww[j] >> 16, i * 8 + 2 * j + 1) - m);
+        }
+    }
+    if (tid < nrest) sum += expf(masked(tail_s[tid], R + tid) - m);
+    sum = block_reduce(sum, false, red);
+
+    // probabilities + running arg-max of the 8 residue classes this thread sees: token i*8+j has residue
+    // (8*(tid&3) + j) mod 32 when 32 | top_k ... the general residue is (i*8+j) % top_k, tracked per j
+    const int top_k = a.top_k;
+    float best_v[8];
+    int best_t[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        best_v[j] = -1.f;
+        best_t[j] = 0x7fffffff;
+    }
+    for (int i = tid; i < nvec; i += 256) {
+        const u32x4 w = *reinterpret_cast<const u32x4 *>(srow + i * 8);
+        const u32 ww[4] = {w.x, w.y, w.z, w.w};
+        u32 out[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const u32 p0 = float_to_half_bits(expf(masked(ww[j] & 0xffffu, i * 8 + 2 * j) - m) / sum);
+            const u32 p1 = float_to_half_bits(expf(masked(ww[j] >> 16, i * 8 + 2 * j + 1) - m) / sum);
+            out[j] = p0 | (p1 << 16);
+            const float f0 = half_bits_to_float(p0), f1 = half_bits_to_float(p1);
+            if (f0 > best_v[2 * j]) { best_v[2 * j] = f0; best_t[2 * j] = i * 8 + 2 * j; }
+            if (f1 > best_v[2 * j + 1]) { best_v[2 * j + 1] = f1; best_t[2 * j + 1] = i * 8 + 2 * j + 1; }
+        }
+        u32x4 o = {out[0], out[1], out[2], out[3]};
+        *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
+    }
+    if (tid < nrest) {
+        const unsigned short p = float_to_half_bits(expf(masked(tail_s[tid], R + tid) - m) / sum);
+        prow[R + tid] = p;
+        tail_p[tid] = half_bits_to_float(p);
+    }
+    __syncthreads();
+
+    // (d)+(e) probe over the flushed part (extension/v_cache_file.py:119-143): needs top_k == 32 and
+    //     256 % top_k == 0 so that a thread's 8 tokens keep their residues from iteration to iteration
+    if (R > 0) {
+        // thread tid covers residues 8*(tid&3)+j; 64 threads share each residue
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            cand_v[tid >> 2][8 * (tid & 3) + j] = best_v[j];
+            cand_t[tid >> 2][8 * (tid & 3) + j] = best_t[j];
+        }
+        __syncthreads();
+        if (tid < top_k) {
+            float bv = -1.f;
+            int bt = 0x7fffffff;
+            for (int k = 0; k < 64; ++k) {
+                const float v = cand_v[k][tid];
+                const int t = cand_t[k][tid];
+                if (v > bv || (v == bv && t < bt)) { bv = v; bt = t; }
+            }
+            probe_p[tid] = bv;
+            probe_t[tid] = bt;
+        }
+        __syncthreads();
+        for (int d = tid; d < D; d += 256) {
+            float acc = 0.f;
+            for (int i = 0; i < top_k; ++i) {
+                const u32 hi = a.v_first_8[((int64_t)bh * a.max_seq_len + probe_t[i]) * D + d];
+                acc = fmaf(half_bits_to_float(((hi << 8) | 0x80u) & 0x7fffu), probe_p[i], acc);
+            }
+            // exponent with the lowest bit cleared (`& 0x1F - 1`, extension/v_cache_file.py:142)
+            a.toe[(int64_t)bh * D + d] = (uint8_t)(exp_field(float_to_half_bits(acc)) & 0x1eu);
+        }
+    }
+    // (f) the tail's share of the output, an fp16 matmul result (extension/v_cache_file.py:189)
+    for (int d = tid; d < D; d += 256) {
+        float acc = 0.f;
+        for (int r = 0; r < nrest; ++r) {
+            const unsigned short *vrow = (r == newest && a.persist) ? vnew : a.restv + (((int64_t)b * a.cb + r) * a.H + h) * D;
+            acc = fmaf(half_bits_to_float(vrow[d]), tail_p[r], acc);
+        }
+        a.otail[(int64_t)bh * D + d] = float_to_half_bits(acc);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// V pass.  grid (n_chunks, H, B), 256 threads.
+// ------------------------------------------------------------------------------------------------
+template <int D, bool REF>
+__global__ __launch_bounds__(256) void fused_v_pass_kernel(
+    const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
+    const unsigned short *__restrict__ probs, const uint8_t *__restrict__ toe, const uint8_t *__restrict__ vcm,
+    float *__restrict__ partial, uint8_t *__restrict__ levels_out, uint8_t *__restrict__ amin_out, int H,
+    int max_seq_len, int row_stride, int n_tokens, int tokens_per_wave, int n_chunks, int literal_broadcast) {
+    __shared__ float wave_part[4][D];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    const int bh = b * H + h;
+    // alignment threshold: min over channels of probe exponent + 15 - column max, wrapping uint8
+    // (extension/v_cache_file.py:156-160).  literal_broadcast pairs entry b*H+h with the probe of
+    // (b / H, b % H) and the column maxima of (b / H, h), which is what the reference expression reads.
+    unsigned char amin = 0;
+    if (!REF) {
+        const int probe_bh = literal_broadcast ? (b / H) * H + (b % H) : bh;
+        const int cm_bh = literal_broadcast ? (b / H) * H + h : bh;
+        u32 mn = 0xffu;
+        for (int c = lane; c < D; c += 64)
+            mn = min(mn, ((u32)toe[(int64_t)probe_bh * D + c] + 15u - (u32)vcm[(int64_t)cm_bh * D + c]) & 0xffu);
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) mn = min(mn, (u32)__shfl_xor((int)mn, m, 64));
+        amin = (unsigned char)mn;
+        if (amin_out != nullptr && chunk == 0 && threadIdx.x == 0) amin_out[bh] = amin;
+    }
+    const int t_begin = (chunk * 4 + wave) * tokens_per_wave;
+    const int t_end = min(t_begin + tokens_per_wave, n_tokens);
+    const int64_t row0 = (int64_t)bh * max_seq_len;
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    v_accumulate<D, REF>(first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
+                         probs + (int64_t)bh * row_stride, amin, t_begin, t_end, acc,
+                         levels_out != nullptr ? levels_out + (int64_t)bh * n_tokens : nullptr);
+    v_fold_workgroup<D>(acc, wave_part, partial + ((int64_t)bh * n_chunks + chunk) * D);
+}
+
+// grid (B*H), D threads: out = fp16(fp16(sum of partials) + tail), the fp16 `o += tail` of the reference.
+__global__ void fused_combine_kernel(const float *__restrict__ partial, const unsigned short *__restrict__ otail,
+                                     unsigned short *__restrict__ out, int D, int n_chunks) {
+    const int bh = blockIdx.x;
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float acc = 0.f;
+        for (int c = 0; c < n_chunks; ++c) acc += partial[((int64_t)bh * n_chunks + c) * D + d];
+        const float o16 = half_bits_to_float(float_to_half_bits(acc));
+        out[(int64_t)bh * D + d] = float_to_half_bits(o16 + half_bits_to_float(otail[(int64_t)bh * D + d]));
+    }
+}
+
+struct StepLayout {
+    size_t toe, otail, partial, total;
+};
+
+static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
+    StepLayout l;
+    auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
+    const VPlan p = v_plan(B, H, D, max_seq_len);
+    // the plan for fewer tokens never has more chunks than the plan for max_seq_len has at its finest split
+    size_t max_chunks = (size_t)(max_seq_len + 4 * (D == 256 ? 32 : 64) - 1) / (4 * (D == 256 ? 32 : 64));
+    (void)p;
+    l.toe = 0;
+    l.otail = up((size_t)B * H * D);
+    l.partial = l.otail + up((size_t)B * H * D * 2);
+    l.total = l.partial + up((size_t)B * H * max_chunks * D * sizeof(float));
+    return l;
+}
+
+template <int D>
+static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint8_t *vm4, uint8_t *vl4, uint8_t *kcm,
+                    uint8_t *vcm, uint8_t *restk, uint8_t *restv, const uint8_t *q, const uint8_t *k_new,
+                    const uint8_t *v_new, const uint8_t *mask, int mask_stride, uint8_t *out, uint8_t *scores,
+                    uint8_t *probs, int row_stride, uint8_t *ws, uint8_t *k_levels_out, uint8_t *v_levels_out,
+                    uint8_t *amin_out, int B, int H, int n_max_blocks, int max_seq_len, int cb, int top_k, int cur_len,
+                    int rest_start, int rest_len, bool ref, int literal_broadcast, hipStream_t st) {
+    const StepLayout lay = step_layout(B, H, D, max_seq_len);
+    uint8_t *toe = ws + lay.toe;
+    unsigned short *otail = reinterpret_cast<unsigned short *>(ws + lay.otail);
+    float *partial = reinterpret_cast<float *>(ws + lay.partial);
+    const unsigned short *q16 = reinterpret_cast<const unsigned short *>(q);
+    const unsigned short *k16 = reinterpret_cast<const unsigned short *>(k_new);
+    const unsigned short *v16 = reinterpret_cast<const unsigned short *>(v_new);
+    unsigned short *s16 = reinterpret_cast<unsigned short *>(scores);
+    unsigned short *p16 = reinterpret_cast<unsigned short *>(probs);
+
+    int R = rest_start, nrest = rest_len + 1, persist = 1;
+    if (nrest == cb) {   // the token fills the rest buffer: flush it into the planes before computing
+        hipLaunchKernelGGL(fused_persist_kernel, dim3(B * H), dim3(D < 256 ? D : 256), 0, st, k16, v16,
+                           reinterpret_cast<unsigned short *>(restk), reinterpret_cast<unsigned short *>(restv), kcm,
+                           vcm, H, D, cb, rest_len);
+        int rc = check_launch("decode_step(persist)");
+        if (rc != AKV_OK) return rc;
+        rc = launch_k_save_blocks(kf8, km4, kl4, restk, B, H, 1, n_max_blocks, D, cb, rest_start, cb, st);
+        if (rc != AKV_OK) return rc;
+        rc = launch_v_save(vf8, vm4, vl4, restv, B, H, max_seq_len, D, rest_start, cb, cb, st);
+        if (rc != AKV_OK) return rc;
+        R = rest_start + cb;
+        nrest = 0;
+        persist = 0;
+    }
+    const int n_blocks = R / cb;
+    // the kernel multiplies by the fp16-rounded scale (extension/csrc/K_cache.cu:306)
+    const float scale = __half2float(__float2half_rn(1.0f / sqrtf((float)D)));
+    if (n_blocks > 0) {
+        const int bpw = k_blocks_per_wave(B, H, n_blocks);
+        dim3 grid((n_blocks + 4 * bpw - 1) / (4 * bpw), H, B);
+        if (ref)
+            hipLaunchKernelGGL((fused_k_pass_kernel<D, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
+                               k_levels_out, n_blocks, n_max_blocks, H, row_stride, bpw, scale);
+        else
+            hipLaunchKernelGGL((fused_k_pass_kernel<D, false>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
+                               k_levels_out, n_blocks, n_max_blocks, H, row_stride, bpw, scale);
+        int rc = check_launch("decode_step(k_pass)");
+        if (rc != AKV_OK) return rc;
+    }
+    MiddleArgs ma;
+    ma.q = q16; ma.k_new = k16; ma.v_new = v16;
+    ma.mask = reinterpret_cast<const unsigned short *>(mask);
+    ma.restk = reinterpret_cast<unsigned short *>(restk);
+    ma.restv = reinterpret_cast<unsigned short *>(restv);
+    ma.scores = s16; ma.probs = p16; ma.otail = otail;
+    ma.kcm = kcm; ma.vcm = vcm; ma.toe = toe; ma.v_first_8 = vf8;
+    ma.H = H; ma.cb = cb; ma.max_seq_len = max_seq_len; ma.row_stride = row_stride; ma.mask_stride = mask_stride;
+    ma.R = R; ma.nrest = nrest; ma.top_k = top_k; ma.persist = persist;
+    hipLaunchKernelGGL((fused_middle_kernel<D>), dim3(B * H), dim3(256), 0, st, ma);
+    int rc = check_launch("decode_step(middle)");
+    if (rc != AKV_OK) return rc;
+    const VPlan p = v_plan(B, H, D, R);
+    if (p.n_chunks > 0) {
+        dim3 grid(p.n_chunks, H, B);
+        if (ref)
+            hipLaunchKernelGGL((fused_v_pass_kernel<D, true>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, toe, vcm,
+                               partial, v_levels_out, amin_out, H, max_seq_len, row_stride, R, p.tokens_per_wave,
+                               p.n_chunks, literal_broadcast);
+        else
+            hipLaunchKernelGGL((fused_v_pass_kernel<D, false>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, toe, vcm,
+                               partial, v_levels_out, amin_out, H, max_seq_len, row_stride, R, p.tokens_per_wave,
+                               p.n_chunks, literal_broadcast);
+        rc = check_launch("decode_step(v_pass)");
+        if (rc != AKV_OK) return rc;
+    }
+    hipLaunchKernelGGL(fused_combine_kernel, dim3(B * H), dim3(D < 256 ? D : 256), 0, st, partial, otail,
+                       reinterpret_cast<unsigned short *>(out), D, p.n_chunks);
+    (void)cur_len;
+    return check_launch("decode_step(combine)");
+}
+
+}  // namespace akv
+
+using namespace akv;
+
+extern "C" size_t akv_decode_step_workspace_bytes(int bsz, int n_kv_heads, int head_dim, int max_seq_len) {
+    if (bsz <= 0 || n_kv_heads <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
+    return step_layout(bsz, n_kv_heads, head_dim, max_seq_len).total;
+}
+
+extern "C" int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,
+                               uint8_t *v_mid_4, uint8_t *v_last_4, uint8_t *k_exp_column_max,
+                               uint8_t *v_exp_column_max, uint8_t *restk, uint8_t *restv, const uint8_t *q,
+                               const uint8_t *k_new, const uint8_t *v_new, const uint8_t *mask, int mask_stride,
+                               uint8_t *out, uint8_t *scores, uint8_t *probs, int row_stride, void *workspace,
+                               size_t workspace_bytes, uint8_t *k_levels_out, uint8_t *v_levels_out, uint8_t *amin_out,
+                               int bsz, int n_kv_heads, int n_max_blocks, int max_seq_len, int head_dim, int d_block,
+                               int top_max_k, int cur_len, int rest_start, int rest_len, int reference,
+                               int literal_broadcast, akv_stream_t stream) {
+    AKV_REQUIRE(k_first_8 && k_mid_4 && k_last_4 && v_first_8 && v_mid_4 && v_last_4 && k_exp_column_max &&
+                    v_exp_column_max && restk && restv && q && k_new && v_new && out && scores && probs && workspace,
+                "decode_step: null pointer");
+    AKV_REQUIRE(bsz > 0 && n_kv_heads > 0 && n_max_blocks > 0 && max_seq_len > 0, "decode_step: non-positive dimension");
+    AKV_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256,
+                "decode_step: head_dim %d not supported by the fused step (64, 128, 256); use the five ops", head_dim);
+    AKV_REQUIRE(d_block == 64, "decode_step: d_block %d not supported by the fused step (64); use the five ops", d_block);
+    AKV_REQUIRE(top_max_k == 32, "decode_step: top_max_k %d not supported by the fused step (32)", top_max_k);
+    AKV_REQUIRE(bsz <= 65535 && n_kv_heads <= 65535, "decode_step: bsz/heads exceed the grid limit 65535");
+    AKV_REQUIRE(cur_len >= 0 && rest_start >= 0 && rest_len >= 0 && rest_len < d_block && rest_start % d_block == 0 &&
+                    rest_start + rest_len == cur_len,
+                "decode_step: inconsistent state cur_len=%d rest_start=%d rest_len=%d", cur_len, rest_start, rest_len);
+    AKV_REQUIRE(cur_len + 1 <= max_seq_len, "decode_step: cache full (%d of %d tokens)", cur_len, max_seq_len);
+    AKV_REQUIRE((int64_t)n_max_blocks * d_block >= rest_start + (rest_len + 1 == d_block ? d_block : 0),
+                "decode_step: K planes hold %d blocks, %d tokens flushed", n_max_blocks, rest_start);
+    AKV_REQUIRE(row_stride % 8 == 0 && row_stride >= rest_start + d_block,
+                "decode_step: row_stride %d must be a multiple of 8 and >= %d", row_stride, rest_start + d_block);
+    AKV_REQUIRE(mask == nullptr || mask_stride == 0 || mask_stride >= cur_len + 1,
+                "decode_step: mask row stride %d shorter than %d (0 = one row for all sequences)", mask_stride, cur_len + 1);
+    AKV_REQUIRE((int64_t)max_seq_len * head_dim < (int64_t)1 << 31 && (int64_t)n_max_blocks * head_dim * d_block < (int64_t)1 << 31,
+                "decode_step: one (batch, head) slice of a high-byte plane must stay below 2 GiB");
+    const size_t need = akv_decode_step_workspace_bytes(bsz, n_kv_heads, head_dim, max_seq_len);
+    AKV_REQUIRE(workspace_bytes >= need, "decode_step: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+    AKV_REQUIRE(((uintptr_t)workspace & 255) == 0 && ((uintptr_t)scores & 15) == 0 && ((uintptr_t)probs & 15) == 0,
+                "decode_step: workspace must be 256-byte aligned, scores/probs 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    uint8_t *ws = static_cast<uint8_t *>(workspace);
+#define AKV_STEP(DD)                                                                                                  \
+    return run_step<DD>(k_first_8, k_mid_4, k_last_4, v_first_8, v_mid_4, v_last_4, k_exp_column_max, v_exp_column_max, \
+                        restk, restv, q, k_new, v_new, mask, mask_stride, out, scores, probs, row_stride, ws,          \
+                        k_levels_out, v_levels_out, amin_out, bsz, n_kv_heads, n_max_blocks, max_seq_len, d_block,     \
+                        top_max_k, cur_len, rest_start, rest_len, reference != 0, literal_broadcast, st);
+    if (head_dim == 64) { AKV_STEP(64) }
+    if (head_dim == 128) { AKV_STEP(128) }
+    AKV_STEP(256)
+#undef AKV_STEP
+}

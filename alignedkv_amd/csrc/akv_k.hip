@@ -12,7 +12,7 @@
 // with an out-of-range buffer offset (they return 0 and fetch nothing) and OR-ed with the
 // substitution byte.  Each lane keeps 16 fp32 accumulators (its 16 slots); a reduce-scatter over
 // the 16 lanes that share the slots leaves one score per lane.
-#include "akv_common.h"
+#include "akv_cores.h"
 
 namespace akv {
 
@@ -112,19 +112,8 @@ __global__ void k_save_token_kernel(uint8_t *__restrict__ first_8, uint8_t *__re
 
 // ------------------------------------------------------------------------------------------------
 // k_cache_compute, tuned: d_block == 64
-// ------------------------------------------------------------------------------------------------
-template <int N>
-__device__ __forceinline__ void reduce_scatter_step(float *a, int lane_mask) {
-    const bool up = (threadIdx.x & lane_mask) != 0;
-#pragma unroll
-    for (int i = 0; i < N / 2; ++i) {
-        float send = up ? a[i] : a[i + N / 2];
-        float keep = up ? a[i + N / 2] : a[i];
-        a[i] = keep + __shfl_xor(send, lane_mask, 64);
-    }
-}
-
 // grid (ceil(n_blocks / (4*blocks_per_wave)), H, B), 256 threads (4 waves).
+// ------------------------------------------------------------------------------------------------
 template <int D, bool REF>
 __global__ __launch_bounds__(256) void k_compute_cb64_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
@@ -132,8 +121,7 @@ __global__ __launch_bounds__(256) void k_compute_cb64_kernel(
     unsigned short *__restrict__ s, uint8_t *__restrict__ levels_out, int n_blocks, int n_max_blocks, int H,
     int blocks_per_wave, float scale) {
     constexpr int CB = 64;
-    constexpr int NG = D / 16;            // load groups of 16 channels
-    constexpr int GC = NG < 8 ? NG : 8;   // groups in flight at a time
+    constexpr int NG = D / 16;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = blockIdx.y, b = blockIdx.z;
     const int bh = b * H + h;
@@ -155,48 +143,9 @@ __global__ __launch_bounds__(256) void k_compute_cb64_kernel(
         if (levels_out != nullptr && blockIdx.x == 0 && wave == 0 && (lane & 3) == 0)
             levels_out[(int64_t)bh * D + c] = (uint8_t)lv;
     }
-
     const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
-    const __amdgpu_buffer_rsrc_t rH = make_rsrc(first_8 + plane_off * 2, (u32)n_blocks * (D * CB));
-    const __amdgpu_buffer_rsrc_t rM = make_rsrc(mid_4 + plane_off, (u32)n_blocks * (D * CB / 2));
-    const __amdgpu_buffer_rsrc_t rL = make_rsrc(last_4 + plane_off, (u32)n_blocks * (D * CB / 2));
-    unsigned short *s_row = s + (int64_t)bh * ((int64_t)(n_blocks + 1) * CB);
-
-    for (int blk = first_blk; blk < end_blk; ++blk) {
-        float acc[16];
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-#pragma unroll
-        for (int g0 = 0; g0 < NG; g0 += GC) {
-            u32x4 hv[GC];
-            u32x2 mv[GC], lv[GC];
-#pragma unroll
-            for (int g = 0; g < GC; ++g) {
-                const int gg = g0 + g;
-                hv[g] = __builtin_amdgcn_raw_buffer_load_b128(rH, blk * (D * CB) + gg * 1024 + lane * 16, 0, 0);
-                int mo = ((need_mid >> gg) & 1u) ? blk * (D * CB / 2) + gg * 512 + lane * 8 : kSkip;
-                int lo = ((need_last >> gg) & 1u) ? blk * (D * CB / 2) + gg * 512 + lane * 8 : kSkip;
-                mv[g] = __builtin_amdgcn_raw_buffer_load_b64(rM, mo, 0, 0);
-                lv[g] = __builtin_amdgcn_raw_buffer_load_b64(rL, lo, 0, 0);
-            }
-#pragma unroll
-            for (int g = 0; g < GC; ++g) {
-                const int gg = g0 + g;
-                const u32 cm = ((need_mid >> gg) & 1u) ? 0u : 0x88888888u;                            // level 2
-                const u32 cl = (((need_mid >> gg) & 1u) && !((need_last >> gg) & 1u)) ? 0x88888888u : 0u;  // level 1
-                fma8(acc, hv[g].x, hv[g].y, mv[g].x | cm, lv[g].x | cl, qf[gg]);
-                fma8(acc + 8, hv[g].z, hv[g].w, mv[g].y | cm, lv[g].y | cl, qf[gg]);
-            }
-        }
-        // acc[i] is the partial score of slot (lane&3)*16 + i over this lane's channels
-        reduce_scatter_step<16>(acc, 32);
-        reduce_scatter_step<8>(acc, 16);
-        reduce_scatter_step<4>(acc, 8);
-        reduce_scatter_step<2>(acc, 4);
-        const int slot = (lane & 3) * 16 + ((lane & 32) ? 8 : 0) + ((lane & 16) ? 4 : 0) + ((lane & 8) ? 2 : 0) +
-                         ((lane & 4) ? 1 : 0);
-        s_row[blk * CB + slot] = float_to_half_bits(acc[0] * scale);
-    }
+    k_score_blocks<D>(first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
+                      need_mid, need_last, s + (int64_t)bh * ((int64_t)(n_blocks + 1) * CB), scale);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -235,9 +184,7 @@ template <int D, bool REF>
 static void launch_k_cb64(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *sum_u8,
                           const uint8_t *max_u8, const uint8_t *q, uint8_t *s, uint8_t *levels, int B, int H,
                           int n_blocks, int n_max_blocks, float scale, hipStream_t st) {
-    // enough waves to fill 256 CUs several times over, a few blocks per wave to amortise set-up
-    int bpw = 1;
-    while (bpw < 4 && (int64_t)B * H * ((n_blocks + bpw * 2 - 1) / (bpw * 2)) >= 8192) bpw *= 2;
+    const int bpw = k_blocks_per_wave(B, H, n_blocks);
     dim3 grid((n_blocks + 4 * bpw - 1) / (4 * bpw), H, B);
     hipLaunchKernelGGL((k_compute_cb64_kernel<D, REF>), grid, dim3(256), 0, st, f8, m4, l4, sum_u8, max_u8,
                        reinterpret_cast<const unsigned short *>(q), reinterpret_cast<unsigned short *>(s), levels,
@@ -248,9 +195,10 @@ static void launch_k_cb64(const uint8_t *f8, const uint8_t *m4, const uint8_t *l
 
 using namespace akv;
 
-extern "C" int akv_k_cache_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *k_new, int bsz,
-                                int n_kv_heads, int n_blocks, int n_max_blocks, int d_head, int d_block,
-                                int start_pos, int seqlen, akv_stream_t stream) {
+namespace akv {
+int launch_k_save_blocks(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *k_new, int bsz, int n_kv_heads,
+                         int n_blocks, int n_max_blocks, int d_head, int d_block, int start_pos, int seqlen,
+                         hipStream_t st) {
     AKV_REQUIRE(first_8 && mid_4 && last_4 && k_new, "k_cache_save: null pointer");
     AKV_REQUIRE(bsz > 0 && n_kv_heads > 0 && d_head > 0 && d_block > 0 && n_max_blocks > 0,
                 "k_cache_save: non-positive dimension (bsz=%d heads=%d d_head=%d d_block=%d n_max_blocks=%d)", bsz,
@@ -259,7 +207,6 @@ extern "C" int akv_k_cache_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_
                 d_block, d_head);
     AKV_REQUIRE(start_pos >= 0 && seqlen >= 0 && n_blocks >= 0, "k_cache_save: negative start_pos/seqlen/n_blocks");
     AKV_REQUIRE(bsz <= 65535 && n_kv_heads <= 65535, "k_cache_save: bsz/heads exceed the grid limit 65535");
-    hipStream_t st = static_cast<hipStream_t>(stream);
     if (start_pos == 0 || seqlen % d_block == 0) {
         if (n_blocks == 0) return AKV_OK;
         const int start_block = start_pos / d_block;
@@ -286,6 +233,14 @@ extern "C" int akv_k_cache_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_
     }
     // the reference launches nothing for this combination (extension/csrc/K_cache.cu:120,142)
     return AKV_OK;
+}
+}  // namespace akv
+
+extern "C" int akv_k_cache_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *k_new, int bsz,
+                                int n_kv_heads, int n_blocks, int n_max_blocks, int d_head, int d_block,
+                                int start_pos, int seqlen, akv_stream_t stream) {
+    return launch_k_save_blocks(first_8, mid_4, last_4, k_new, bsz, n_kv_heads, n_blocks, n_max_blocks, d_head, d_block,
+                                start_pos, seqlen, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int akv_k_cache_compute(const uint8_t *first_8, const uint8_t *mid_4, const uint8_t *last_4,

@@ -12,7 +12,7 @@
 // the substitution byte.  Each lane keeps 16 fp32 accumulators (its channels); a reduce-scatter
 // over the lanes that share channels, LDS across the 4 waves, then fp32 partial sums per chunk
 // that a second small kernel adds up in a fixed order (deterministic output bits).
-#include "akv_common.h"
+#include "akv_cores.h"
 
 namespace akv {
 
@@ -102,41 +102,6 @@ __global__ void v_test_kernel(const uint8_t *__restrict__ first_8, const unsigne
 // ------------------------------------------------------------------------------------------------
 // v_cache_compute
 // ------------------------------------------------------------------------------------------------
-struct VPlan {
-    bool tuned;
-    int tokens_per_wave;   // tuned kernel
-    int chunk_tokens;      // tokens per workgroup
-    int n_chunks;
-};
-
-static VPlan v_plan(int B, int H, int D, int n_tokens) {
-    VPlan p;
-    p.tuned = (D == 64 || D == 128 || D == 256);
-    if (p.tuned) {
-        const int iter_tokens = D == 256 ? 32 : 64;
-        int k = 1;
-        while (k < 8 && (int64_t)B * H * ((n_tokens + 4 * iter_tokens * k * 2 - 1) / (4 * iter_tokens * k * 2)) >= 2048) k *= 2;
-        p.tokens_per_wave = iter_tokens * k;
-        p.chunk_tokens = 4 * p.tokens_per_wave;
-    } else {
-        p.tokens_per_wave = 0;
-        p.chunk_tokens = 256;
-    }
-    p.n_chunks = n_tokens > 0 ? (n_tokens + p.chunk_tokens - 1) / p.chunk_tokens : 0;
-    return p;
-}
-
-template <int N>
-__device__ __forceinline__ void v_reduce_scatter_step(float *a, int lane_mask) {
-    const bool up = (threadIdx.x & lane_mask) != 0;
-#pragma unroll
-    for (int i = 0; i < N / 2; ++i) {
-        float send = up ? a[i] : a[i + N / 2];
-        float keep = up ? a[i + N / 2] : a[i];
-        a[i] = keep + __shfl_xor(send, lane_mask, 64);
-    }
-}
-
 // grid (n_chunks, H, B), 256 threads.  partial: fp32 [B*H, n_chunks, D].
 template <int D, bool REF>
 __global__ __launch_bounds__(256) void v_compute_tuned_kernel(
@@ -144,76 +109,21 @@ __global__ __launch_bounds__(256) void v_compute_tuned_kernel(
     const unsigned short *__restrict__ s, const uint8_t *__restrict__ amin_u8, float *__restrict__ partial,
     uint8_t *__restrict__ levels_out, int H, int max_seq_len, int s_last_dim, int n_tokens, int tokens_per_wave,
     int n_chunks) {
-    constexpr int LPR = D / 16;            // lanes per token row
-    constexpr int TPL = 64 / LPR;          // token rows per wave-wide load
-    constexpr int U = LPR < 8 ? LPR : 8;   // loads in flight per iteration
     __shared__ float wave_part[4][D];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wave = threadIdx.x >> 6;
     const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int bh = b * H + h;
-    const int tl = lane / LPR, cl = lane % LPR;
     const int t_begin = (chunk * 4 + wave) * tokens_per_wave;
     const int t_end = min(t_begin + tokens_per_wave, n_tokens);
     const unsigned char amin = REF ? 0 : amin_u8[bh];
-
     const int64_t row0 = (int64_t)bh * max_seq_len;
-    const __amdgpu_buffer_rsrc_t rH = make_rsrc(first_8 + row0 * D, (u32)n_tokens * D);
-    const __amdgpu_buffer_rsrc_t rM = make_rsrc(mid_4 + row0 * (D / 2), (u32)n_tokens * (D / 2));
-    const __amdgpu_buffer_rsrc_t rL = make_rsrc(last_4 + row0 * (D / 2), (u32)n_tokens * (D / 2));
-    const unsigned short *s_row = s + (int64_t)bh * s_last_dim;
-
     float acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-
-    for (int base = t_begin; base < t_end; base += U * TPL) {
-        u32x4 hv[U];
-        u32x2 mv[U], lv[U];
-        float sf[U];
-        u32 cm[U], cl_[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int t = base + u * TPL + tl;
-            const bool valid = t < t_end;
-            const u32 sbits = valid ? (u32)s_row[t] : 0u;
-            const int level = REF ? 0 : v_level(amin, (unsigned short)sbits);
-            sf[u] = half_bits_to_float(sbits);
-            hv[u] = __builtin_amdgcn_raw_buffer_load_b128(rH, valid ? t * D + cl * 16 : kSkip, 0, 0);
-            mv[u] = __builtin_amdgcn_raw_buffer_load_b64(rM, (valid && level < 2) ? t * (D / 2) + cl * 8 : kSkip, 0, 0);
-            lv[u] = __builtin_amdgcn_raw_buffer_load_b64(rL, (valid && level == 0) ? t * (D / 2) + cl * 8 : kSkip, 0, 0);
-            cm[u] = level == 2 ? 0x88888888u : 0u;
-            cl_[u] = level == 1 ? 0x88888888u : 0u;
-            if (levels_out != nullptr && valid && cl == 0) levels_out[(int64_t)bh * n_tokens + t] = (uint8_t)level;
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            fma8(acc, hv[u].x, hv[u].y, mv[u].x | cm[u], lv[u].x | cl_[u], sf[u]);
-            fma8(acc + 8, hv[u].z, hv[u].w, mv[u].y | cm[u], lv[u].y | cl_[u], sf[u]);
-        }
-    }
-
-    // acc[i]: channel cl*16 + i summed over this lane's tokens; fold the token lanes together
-    int ch = cl * 16;
-    constexpr int NV = LPR == 16 ? 4 : (LPR == 8 ? 2 : 1);   // sums left per lane
-    v_reduce_scatter_step<16>(acc, 32);
-    ch += (lane & 32) ? 8 : 0;
-    v_reduce_scatter_step<8>(acc, 16);
-    ch += (lane & 16) ? 4 : 0;
-    if constexpr (LPR <= 8) {
-        v_reduce_scatter_step<4>(acc, 8);
-        ch += (lane & 8) ? 2 : 0;
-    }
-    if constexpr (LPR <= 4) {
-        v_reduce_scatter_step<2>(acc, 4);
-        ch += (lane & 4) ? 1 : 0;
-    }
-#pragma unroll
-    for (int i = 0; i < NV; ++i) wave_part[wave][ch + i] = acc[i];
-    __syncthreads();
-    for (int d = threadIdx.x; d < D; d += 256) {
-        float v = (wave_part[0][d] + wave_part[1][d]) + (wave_part[2][d] + wave_part[3][d]);
-        partial[((int64_t)bh * n_chunks + chunk) * D + d] = v;
-    }
+    v_accumulate<D, REF>(first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
+                         s + (int64_t)bh * s_last_dim, amin, t_begin, t_end, acc,
+                         levels_out != nullptr ? levels_out + (int64_t)bh * n_tokens : nullptr);
+    v_fold_workgroup<D>(acc, wave_part, partial + ((int64_t)bh * n_chunks + chunk) * D);
 }
 
 // any even head_dim: grid (n_chunks, H, B), one thread per channel pair, serial over the chunk's tokens.
@@ -275,9 +185,9 @@ static void launch_v_tuned(bool ref, const uint8_t *f8, const uint8_t *m4, const
 
 using namespace akv;
 
-extern "C" int akv_v_cache_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *v_new, int bsz,
-                                int n_local_kv_heads, int max_seq_len, int head_dim, int start_pos, int seq_len,
-                                int v_new_seq, akv_stream_t stream) {
+namespace akv {
+int launch_v_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *v_new, int bsz, int n_local_kv_heads,
+                  int max_seq_len, int head_dim, int start_pos, int seq_len, int v_new_seq, hipStream_t st) {
     if (seq_len == 0) return AKV_OK;   // reference: extension/csrc/V_cache.cu:54-55
     AKV_REQUIRE(first_8 && mid_4 && last_4 && v_new, "v_cache_save: null pointer");
     AKV_REQUIRE(bsz > 0 && n_local_kv_heads > 0 && max_seq_len > 0 && head_dim > 0 && head_dim % 2 == 0,
@@ -286,7 +196,6 @@ extern "C" int akv_v_cache_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_
     AKV_REQUIRE(seq_len > 0 && start_pos >= 0 && start_pos + seq_len <= max_seq_len,
                 "v_cache_save: rows %d..%d outside the plane of %d rows", start_pos, start_pos + seq_len, max_seq_len);
     AKV_REQUIRE(v_new_seq >= seq_len, "v_cache_save: v_new holds %d tokens, %d requested", v_new_seq, seq_len);
-    hipStream_t st = static_cast<hipStream_t>(stream);
     const unsigned short *src = reinterpret_cast<const unsigned short *>(v_new);
     if (head_dim % 8 == 0) {
         int64_t total = (int64_t)bsz * seq_len * n_local_kv_heads * (head_dim / 8);
@@ -298,6 +207,14 @@ extern "C" int akv_v_cache_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_
                            last_4, src, n_local_kv_heads, head_dim, max_seq_len, start_pos, seq_len, v_new_seq, total);
     }
     return check_launch("v_cache_save");
+}
+}  // namespace akv
+
+extern "C" int akv_v_cache_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *v_new, int bsz,
+                                int n_local_kv_heads, int max_seq_len, int head_dim, int start_pos, int seq_len,
+                                int v_new_seq, akv_stream_t stream) {
+    return launch_v_save(first_8, mid_4, last_4, v_new, bsz, n_local_kv_heads, max_seq_len, head_dim, start_pos, seq_len,
+                         v_new_seq, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int akv_v_cache_test_compute(const uint8_t *first_8, const uint8_t *mid_4, const uint8_t *last_4,

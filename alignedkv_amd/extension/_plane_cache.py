@@ -87,6 +87,14 @@ class PlaneCacheBase(torch.nn.Module):
     def _store_planes(self, tokens: torch.Tensor, start_pos: int, n_tokens: int):
         raise NotImplementedError
 
+    def _advance_after_fused_step(self):
+        """Host counters after the fused step appended one token (and flushed a full rest buffer)."""
+        self.current_cache_len += 1
+        self._restlen += 1
+        if self._restlen == column_block:
+            self._restlen = 0
+            self.reststartpos += column_block
+
     def _zero_state(self):
         # the reference leaves the rest buffer untouched here (extension/k_cache_file.py:62-67); a prefill
         # always follows a reset and re-creates it, clearing it as well is harmless

@@ -63,6 +63,13 @@ class QuantizedCache_AlignedKV(_HFCache):
                                                   self.head_dim, idx, device, register, 32, literal_colmax,
                                                   literal_broadcast))
         self.reference = False   # True: every plane is read (dense-in-planes baseline), model/KVCache_AlignedKV.py:46
+        # True: a decode step is one call of the fused HIP step (4 launches); False: the reference's sequence
+        # of ops and framework kernels (K op -> mask -> softmax -> probe op -> V op), kept for A/B checks.
+        self.fused = self.head_dim in (64, 128, 256)
+        self.literal_broadcast = literal_broadcast
+        self._device = device
+        self._scores = None
+        self._probs = None
 
     def update(self, key_states, value_states, layer_idx, cache_kwargs=None):
         raise Exception("This function is not used in AlignedKV")
@@ -103,7 +110,55 @@ class QuantizedCache_AlignedKV(_HFCache):
         self.value_cache[layer_id].save(v, start_pos, seqlen)
         return self.value_cache[layer_id].decoding_compute(scores, start_pos, seqlen, self.reference)
 
+    def _fused_mask(self, mask, width: int):
+        """[B|1, 1, 1, width] additive mask -> 2-d uint8 view, or False if the fused step cannot take it."""
+        if mask is None:
+            return None
+        if mask.dim() != 4 or mask.shape[1] != 1 or mask.shape[2] != 1 or mask.shape[-1] < width:
+            return False
+        if mask.dtype != torch.half or mask.shape[0] not in (1, self.max_batch_size):
+            return False
+        return mask.reshape(mask.shape[0], mask.shape[-1]).contiguous().view(torch.uint8)
+
+    def decoding_fused(self, q, k, v, start_pos: int, mask2d, layer_id: int):
+        """One decode step through akv_decode_step; same state transitions as decoding_k + decoding_v."""
+        from ..extension.KV_cache_cpp_extention import cuda_module
+        from ..extension._plane_cache import column_block
+        kc, vc = self.key_cache[layer_id], self.value_cache[layer_id]
+        kc._check_save(k, start_pos, 1, "new_k")
+        vc._check_save(v, start_pos, 1, "new_v")
+        assert tuple(q.shape) == tuple(k.shape), f"q.shape: {tuple(q.shape)} != {tuple(k.shape)}"
+        B, H, D = self.max_batch_size, self.num_key_value_heads, self.head_dim
+        if self._scores is None:
+            width = (kc.n_max_blocks + 1) * column_block
+            self._scores = torch.empty((B, H, width), dtype=torch.half, device=q.device)
+            self._probs = torch.empty((B, H, width), dtype=torch.half, device=q.device)
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        out = torch.empty_like(q)
+        flushed = kc.reststartpos + (column_block if kc._restlen + 1 == column_block else 0)
+        klv = vlv = amin = None
+        if kc.record_levels or vc.record_levels:
+            klv = torch.empty((B, H, D), dtype=torch.uint8, device=q.device)
+            vlv = torch.empty((B, H, flushed), dtype=torch.uint8, device=q.device) if flushed else None
+            amin = torch.empty((B, H), dtype=torch.uint8, device=q.device)
+        cuda_module.decode_step(
+            (kc.k_cache_first_8, kc.k_cache_mid_4, kc.k_cache_last_4),
+            (vc.v_cache_first_8, vc.v_cache_mid_4, vc.v_cache_last_4),
+            kc._colmax, vc._colmax, kc._rest.view(torch.uint8), vc._rest.view(torch.uint8),
+            q.view(torch.uint8), k.view(torch.uint8), v.view(torch.uint8), mask2d, out.view(torch.uint8),
+            self._scores.view(torch.uint8), self._probs.view(torch.uint8), B, H, kc.n_max_blocks, self.max_cache_len,
+            D, column_block, vc.top_max_k, start_pos, kc.reststartpos, kc._restlen, self.reference,
+            self.literal_broadcast, klv, vlv, amin)
+        kc._advance_after_fused_step()
+        vc._advance_after_fused_step()
+        kc.last_levels, vc.last_levels, vc.last_alignment_min = klv, vlv, amin
+        return out
+
     def decoding(self, q, k, v, start_pos: int, seqlen: int, mask, layer_id: int):
+        if self.fused and seqlen == 1:
+            mask2d = self._fused_mask(mask, start_pos + seqlen)
+            if mask2d is not False:
+                return self.decoding_fused(q, k, v, start_pos, mask2d, layer_id)
         scores = self.decoding_k(q, k, start_pos, seqlen, layer_id)
         if mask is not None:
             scores[:, :, :, :start_pos + seqlen] += mask

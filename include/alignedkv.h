@@ -117,6 +117,42 @@ AKV_API int akv_v_cache_compute(const uint8_t *first_8, const uint8_t *mid_4, co
                         int bsz, int n_local_kv_heads, int max_seq_len, int head_dim, int s_last_dim,
                         int start_pos_add_seqlen, int reference, akv_stream_t stream);
 
+/*
+ * Fused decode step for one layer: appends one token per sequence and attends over the whole cache.
+ * Replaces, in one call, what the reference does in Python around its three compute ops:
+ * QuantizedCache_AlignedKV.decoding (model/KVCache_AlignedKV.py:116-124), K_Cache_Class.save /
+ * decoding_compute (extension/k_cache_file.py:97-118,132-159) and V_Cache_Class.save / test_compute /
+ * decoding_compute (extension/v_cache_file.py:97-116,119-190), with the same arithmetic and order:
+ * column-max update, rest-buffer append (flush of a full 64-token buffer into the planes first), plane
+ * scores with per-channel fetch levels, fp16 tail scores, optional additive fp16 mask, fp32 softmax to
+ * fp16 probabilities, 32-bucket arg-max probe, alignment threshold, plane output with per-token fetch
+ * levels, fp16 tail output.
+ *
+ * State, updated in place: K/V planes; k_/v_exp_column_max uint8 [bsz,1,heads,head_dim]; restk/restv fp16
+ * [bsz, d_block, heads, head_dim].  The caller keeps the three counters and advances them after the call:
+ * cur_len += 1; rest_len += 1; if rest_len == d_block: rest_start += d_block, rest_len = 0.
+ * q, k_new, v_new, out: fp16 [bsz,1,heads,head_dim].  mask: optional fp16 [bsz, >= cur_len+1] with row
+ * stride mask_stride (halves; 0 = one row shared by all sequences), added to the scores of every head.
+ * scores / probs: fp16 [bsz, heads, row_stride] scratch that also serves as debug output (scores of the
+ * flushed blocks and the tail before the mask; probabilities of tokens < cur_len+1); row_stride % 8 == 0,
+ * row_stride >= flushed tokens + d_block.
+ * k_levels_out uint8 [bsz,heads,head_dim], v_levels_out uint8 [bsz,heads,flushed tokens], amin_out uint8
+ * [bsz,heads]: optional (NULL) records of the fetch decisions.
+ * literal_broadcast != 0 reproduces the reference's threshold indexing as written
+ * (extension/v_cache_file.py:157-160 broadcasts [B,H,1,D] against [B,1,H,D]).
+ * Supported: head_dim 64/128/256, d_block 64, top_max_k 32; other shapes go through the five ops.
+ */
+AKV_API size_t akv_decode_step_workspace_bytes(int bsz, int n_kv_heads, int head_dim, int max_seq_len);
+AKV_API int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,
+                            uint8_t *v_mid_4, uint8_t *v_last_4, uint8_t *k_exp_column_max,
+                            uint8_t *v_exp_column_max, uint8_t *restk, uint8_t *restv, const uint8_t *q,
+                            const uint8_t *k_new, const uint8_t *v_new, const uint8_t *mask, int mask_stride,
+                            uint8_t *out, uint8_t *scores, uint8_t *probs, int row_stride, void *workspace,
+                            size_t workspace_bytes, uint8_t *k_levels_out, uint8_t *v_levels_out, uint8_t *amin_out,
+                            int bsz, int n_kv_heads, int n_max_blocks, int max_seq_len, int head_dim, int d_block,
+                            int top_max_k, int cur_len, int rest_start, int rest_len, int reference,
+                            int literal_broadcast, akv_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -32,15 +32,17 @@ def planes_equal(cache, oc, layer=0):
     return True
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("prefill,steps,literal_broadcast", [(200, 70, False), (64, 3, False), (1, 66, False),
                                                              (130, 5, True)])
-def test_cache_matches_oracle_step_by_step(prefill, steps, literal_broadcast):
+def test_cache_matches_oracle_step_by_step(prefill, steps, literal_broadcast, fused):
     from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
     B, H, D = 2, 4, 128
     Lmax = prefill + steps + 10
     q_all, k, v = make_qkv(B, prefill + steps, H, D, seed=prefill)
     rng = np.random.default_rng(prefill)
     cache = QuantizedCache_AlignedKV(cfg(H, D), B, Lmax, "cuda", torch.half, literal_broadcast=literal_broadcast)
+    cache.fused = fused
     oc = O.OracleCache(B, Lmax, H, D, literal_broadcast=literal_broadcast)
     kc, vc = cache.key_cache[0], cache.value_cache[0]
     kc.record_levels = vc.record_levels = True
@@ -67,6 +69,19 @@ def test_cache_matches_oracle_step_by_step(prefill, steps, literal_broadcast):
             got_lv = vc.last_levels.cpu().numpy()
             flips += int((got_lv != oc.last["v_levels"]).sum())
             total += got_lv.size
+            if fused:
+                # bit exact for the probabilities and the threshold the kernels themselves produced
+                R = oc.rest_start
+                pk = cache._probs[:, :, :R].cpu().numpy()
+                amin = vc.last_alignment_min.cpu().numpy()
+                assert np.array_equal(got_lv, O.v_levels(amin, O.as_bits(pk)))
+                tv, ti = O.bucket_max(cache._probs[:, :, None, :R].cpu().numpy(), t + 1)
+                to = O.v_cache_test_compute(oc.v_planes[0], O.as_bits(tv), ti)
+                want_amin = O.alignment_min(O.test_o_exponent(to), oc.v_colmax, literal_broadcast)
+                assert np.array_equal(amin, want_amin), f"threshold differs at token {t}"
+                pd = np.abs(cache._probs[:, :, :t + 1].cpu().numpy().astype(np.float32)
+                            - oc.last["probs"][:, :, 0, :t + 1].astype(np.float32)).max()
+                assert pd <= 2e-3
         err = np.max(np.abs(out.cpu().numpy().astype(np.float32) - want.astype(np.float32)))
         # end to end a score may round to the neighbouring fp16 value (different summation order), which
         # moves a sharp softmax by ~0.4 %: 2e-3 here; with identical op inputs the ops hold 1e-3 (test_gpu_ops.py)
@@ -141,3 +156,45 @@ def test_save_assertions_mirror_the_reference():
     kc.save(x, 0, 8)
     with pytest.raises(AssertionError, match="seqlen"):
         kc.save(x[:, :2], 8, 2)
+
+
+def test_fused_step_with_mask_and_reference_flag():
+    """The fused step with an additive fp16 mask ([B,1,1,L], -inf on a few positions of one sequence)
+    equals the unfused op sequence on the same cache contents, in aligned and in reference mode."""
+    from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
+    B, H, D, prefill = 2, 4, 128, 150
+    q, k, v = make_qkv(B, prefill + 4, H, D, seed=31)
+    rng = np.random.default_rng(3)
+    for reference in (False, True):
+        caches = []
+        for fused in (True, False):
+            c = QuantizedCache_AlignedKV(cfg(H, D), B, 256, "cuda", torch.half)
+            c.fused, c.reference = fused, reference
+            c.auto_compute(dev(q[:, :1].repeat(prefill, axis=1)), dev(k[:, :prefill]), dev(v[:, :prefill]), 0, None)
+            caches.append(c)
+        for t in range(prefill, prefill + 4):
+            qt = dev(rng.standard_normal((B, 1, H, D)).astype(np.float16))
+            mask = torch.zeros((B, 1, 1, t + 1), dtype=torch.half, device="cuda")
+            mask[1, 0, 0, 3:40] = float("-inf")
+            outs = [c.auto_compute(qt, dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, mask) for c in caches]
+            assert torch.isfinite(outs[0]).all()
+            assert (outs[0].float() - outs[1].float()).abs().max().item() <= 2e-3
+            assert caches[0]._probs[1, :, 3:40].abs().max().item() == 0.0
+
+
+def test_fused_step_rejects_bad_state():
+    from alignedkv_amd.extension.KV_cache_cpp_extention import cuda_module as m
+    B, H, D, cb, Lmax = 1, 2, 128, 64, 128
+    z = lambda *shape: torch.zeros(shape, dtype=torch.uint8, device="cuda")
+    kp = (z(B, H, 2, D, cb), z(B, H, 2, D, cb // 2), z(B, H, 2, D, cb // 2))
+    vp = (z(B, H, Lmax, D), z(B, H, Lmax, D // 2), z(B, H, Lmax, D // 2))
+    tok = lambda: z(B, 1, H, D * 2)
+    rest = lambda: z(B, cb, H, D * 2)
+    sc = lambda: z(B, H, (Lmax + cb) * 2)
+    args = lambda cur, rs, rl: (kp, vp, z(B, 1, H, D), z(B, 1, H, D), rest(), rest(), tok(), tok(), tok(), None, tok(),
+                                sc(), sc(), B, H, 2, Lmax, D, cb, 32, cur, rs, rl, False, False)
+    with pytest.raises(RuntimeError, match="inconsistent state"):
+        m.decode_step(*args(10, 64, 3))
+    with pytest.raises(RuntimeError, match="cache full"):
+        m.decode_step(*args(128, 128, 0))
+    m.decode_step(*args(5, 0, 5))
