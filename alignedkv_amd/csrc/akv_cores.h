@@ -80,7 +80,7 @@ __device__ __forceinline__ void k_score_blocks(const uint8_t *f8, const uint8_t 
 //   Lane layout: lane -> token (lane / (D/16)) of each wave-wide load, channels (lane % (D/16))*16..+16.
 //   s_row: fp16 probabilities of this (batch, head).  levels_row (may be null): level per token.
 // ------------------------------------------------------------------------------------------------
-template <int D, bool REF>
+template <int D, bool REF, int NIT>
 __device__ __forceinline__ void v_accumulate(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_tokens,
                                              const unsigned short *s_row, unsigned char amin, int t_begin, int t_end,
                                              float *acc, uint8_t *levels_row) {
@@ -92,19 +92,35 @@ __device__ __forceinline__ void v_accumulate(const uint8_t *f8, const uint8_t *m
     const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
     const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_tokens * (D / 2));
     const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_tokens * (D / 2));
-    for (int base = t_begin; base < t_end; base += U * TPL) {
+    const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)n_tokens * 2);
+    // The probabilities of all the wave's tokens first: the fetch level of a token depends on its
+    // probability, and a load per iteration would put a memory round trip in front of every batch.
+    u32 sb[NIT][U];
+#pragma unroll
+    for (int it = 0; it < NIT; ++it)
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int t = t_begin + (it * U + u) * TPL + tl;
+            sb[it][u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < t_end ? t * 2 : kSkip, 0, 0);
+        }
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+        const int base = t_begin + it * U * TPL;
+        if (base >= t_end) break;
         u32x4 hv[U];
         u32x2 mv[U], lv[U];
-        float sf[U];
+        // the high-byte rows do not depend on the level: issue them before the probabilities are looked at
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int t = base + u * TPL + tl;
+            hv[u] = __builtin_amdgcn_raw_buffer_load_b128(rH, t < t_end ? t * D + cl * 16 : kSkip, 0, 0);
+        }
         u32 cm[U], cl_[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int t = base + u * TPL + tl;
             const bool valid = t < t_end;
-            const u32 sbits = valid ? (u32)s_row[t] : 0u;
-            const int level = REF ? 0 : v_level(amin, (unsigned short)sbits);
-            sf[u] = half_bits_to_float(sbits);
-            hv[u] = __builtin_amdgcn_raw_buffer_load_b128(rH, valid ? t * D + cl * 16 : kSkip, 0, 0);
+            const int level = REF ? 0 : v_level(amin, (unsigned short)sb[it][u]);
             mv[u] = __builtin_amdgcn_raw_buffer_load_b64(rM, (valid && level < 2) ? t * (D / 2) + cl * 8 : kSkip, 0, 0);
             lv[u] = __builtin_amdgcn_raw_buffer_load_b64(rL, (valid && level == 0) ? t * (D / 2) + cl * 8 : kSkip, 0, 0);
             cm[u] = level == 2 ? 0x88888888u : 0u;
@@ -113,8 +129,9 @@ __device__ __forceinline__ void v_accumulate(const uint8_t *f8, const uint8_t *m
         }
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            fma8(acc, hv[u].x, hv[u].y, mv[u].x | cm[u], lv[u].x | cl_[u], sf[u]);
-            fma8(acc + 8, hv[u].z, hv[u].w, mv[u].y | cm[u], lv[u].y | cl_[u], sf[u]);
+            const float sf = half_bits_to_float(sb[it][u]);
+            fma8(acc, hv[u].x, hv[u].y, mv[u].x | cm[u], lv[u].x | cl_[u], sf);
+            fma8(acc + 8, hv[u].z, hv[u].w, mv[u].y | cm[u], lv[u].y | cl_[u], sf);
         }
     }
 }
@@ -149,7 +166,8 @@ __device__ __forceinline__ void v_fold_workgroup(float *acc, float (*wave_part)[
 // Split of the sequence over workgroups for the V pass (shared by the op and the fused step).
 struct VPlan {
     bool tuned;
-    int tokens_per_wave;   // tuned kernel
+    int iters_per_wave;    // tuned kernel: 1, 2 or 4 batches of 64 (32 for head_dim 256) tokens per wave
+    int tokens_per_wave;
     int chunk_tokens;      // tokens per workgroup
     int n_chunks;
 };
@@ -159,11 +177,13 @@ inline VPlan v_plan(int B, int H, int D, int n_tokens) {
     p.tuned = (D == 64 || D == 128 || D == 256);
     if (p.tuned) {
         const int iter_tokens = D == 256 ? 32 : 64;
-        int k = 1;
-        while (k < 8 && (int64_t)B * H * ((n_tokens + 4 * iter_tokens * k * 2 - 1) / (4 * iter_tokens * k * 2)) >= 2048) k *= 2;
+        int k = 1;   // iterations per wave: 1, 2 or 4
+        while (k < 4 && (int64_t)B * H * ((n_tokens + 4 * iter_tokens * k * 2 - 1) / (4 * iter_tokens * k * 2)) >= 2048) k *= 2;
+        p.iters_per_wave = k;
         p.tokens_per_wave = iter_tokens * k;
         p.chunk_tokens = 4 * p.tokens_per_wave;
     } else {
+        p.iters_per_wave = 0;
         p.tokens_per_wave = 0;
         p.chunk_tokens = 256;
     }

@@ -27,6 +27,15 @@ int launch_v_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8
 
 __device__ __forceinline__ u32 exp_field(u32 half_bits) { return (half_bits >> 10) & 0x1fu; }
 
+// Optional per-phase timing of the fused step (benchmark aid): when enabled, events are recorded on the
+// step's stream around the K pass, the middle kernel, the V pass and the combine kernel.
+static bool g_profile = false;
+static hipEvent_t g_ev[5];
+static bool g_ev_ready = false;
+static inline void mark(int i, hipStream_t st) {
+    if (g_profile) (void)hipEventRecord(g_ev[i], st);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
@@ -260,11 +269,14 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
         }
         __syncthreads();
         for (int d = tid; d < D; d += 256) {
+            // the 32 gathered bytes first, then the sum: 32 independent loads in flight instead of a chain
+            u32 hi[32];
+#pragma unroll
+            for (int i = 0; i < 32; ++i) hi[i] = a.v_first_8[((int64_t)bh * a.max_seq_len + probe_t[i]) * D + d];
             float acc = 0.f;
-            for (int i = 0; i < top_k; ++i) {
-                const u32 hi = a.v_first_8[((int64_t)bh * a.max_seq_len + probe_t[i]) * D + d];
-                acc = fmaf(half_bits_to_float(((hi << 8) | 0x80u) & 0x7fffu), probe_p[i], acc);
-            }
+#pragma unroll
+            for (int i = 0; i < 32; ++i)
+                acc = fmaf(half_bits_to_float(((hi[i] << 8) | 0x80u) & 0x7fffu), probe_p[i], acc);
             // exponent with the lowest bit cleared (`& 0x1F - 1`, extension/v_cache_file.py:142)
             a.toe[(int64_t)bh * D + d] = (uint8_t)(exp_field(float_to_half_bits(acc)) & 0x1eu);
         }
@@ -283,7 +295,7 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
 // ------------------------------------------------------------------------------------------------
 // V pass.  grid (n_chunks, H, B), 256 threads.
 // ------------------------------------------------------------------------------------------------
-template <int D, bool REF>
+template <int D, bool REF, int NIT>
 __global__ __launch_bounds__(256) void fused_v_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const unsigned short *__restrict__ probs, const uint8_t *__restrict__ toe, const uint8_t *__restrict__ vcm,
@@ -314,7 +326,7 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
     float acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    v_accumulate<D, REF>(first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
+    v_accumulate<D, REF, NIT>(first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
                          probs + (int64_t)bh * row_stride, amin, t_begin, t_end, acc,
                          levels_out != nullptr ? levels_out + (int64_t)bh * n_tokens : nullptr);
     v_fold_workgroup<D>(acc, wave_part, partial + ((int64_t)bh * n_chunks + chunk) * D);
@@ -383,6 +395,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         persist = 0;
     }
     const int n_blocks = R / cb;
+    mark(0, st);
     // the kernel multiplies by the fp16-rounded scale (extension/csrc/K_cache.cu:306)
     const float scale = __half2float(__float2half_rn(1.0f / sqrtf((float)D)));
     if (n_blocks > 0) {
@@ -397,6 +410,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         int rc = check_launch("decode_step(k_pass)");
         if (rc != AKV_OK) return rc;
     }
+    mark(1, st);
     MiddleArgs ma;
     ma.q = q16; ma.k_new = k16; ma.v_new = v16;
     ma.mask = reinterpret_cast<const unsigned short *>(mask);
@@ -409,22 +423,32 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     hipLaunchKernelGGL((fused_middle_kernel<D>), dim3(B * H), dim3(256), 0, st, ma);
     int rc = check_launch("decode_step(middle)");
     if (rc != AKV_OK) return rc;
+    mark(2, st);
     const VPlan p = v_plan(B, H, D, R);
     if (p.n_chunks > 0) {
         dim3 grid(p.n_chunks, H, B);
-        if (ref)
-            hipLaunchKernelGGL((fused_v_pass_kernel<D, true>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, toe, vcm,
-                               partial, v_levels_out, amin_out, H, max_seq_len, row_stride, R, p.tokens_per_wave,
-                               p.n_chunks, literal_broadcast);
-        else
-            hipLaunchKernelGGL((fused_v_pass_kernel<D, false>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, toe, vcm,
-                               partial, v_levels_out, amin_out, H, max_seq_len, row_stride, R, p.tokens_per_wave,
-                               p.n_chunks, literal_broadcast);
+#define AKV_VP(R, N)                                                                                                  \
+    hipLaunchKernelGGL((fused_v_pass_kernel<D, R, N>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, toe, vcm, partial, \
+                       v_levels_out, amin_out, H, max_seq_len, row_stride, R_tokens, p.tokens_per_wave, p.n_chunks,   \
+                       literal_broadcast)
+        const int R_tokens = R;
+        if (ref) {
+            if (p.iters_per_wave == 1) AKV_VP(true, 1);
+            else if (p.iters_per_wave == 2) AKV_VP(true, 2);
+            else AKV_VP(true, 4);
+        } else {
+            if (p.iters_per_wave == 1) AKV_VP(false, 1);
+            else if (p.iters_per_wave == 2) AKV_VP(false, 2);
+            else AKV_VP(false, 4);
+        }
+#undef AKV_VP
         rc = check_launch("decode_step(v_pass)");
         if (rc != AKV_OK) return rc;
     }
+    mark(3, st);
     hipLaunchKernelGGL(fused_combine_kernel, dim3(B * H), dim3(D < 256 ? D : 256), 0, st, partial, otail,
                        reinterpret_cast<unsigned short *>(out), D, p.n_chunks);
+    mark(4, st);
     (void)cur_len;
     return check_launch("decode_step(combine)");
 }
@@ -432,6 +456,35 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
 }  // namespace akv
 
 using namespace akv;
+
+extern "C" int akv_profile_enable(int enable) {
+    if (enable && !g_ev_ready) {
+        for (int i = 0; i < 5; ++i) {
+            if (hipEventCreate(&g_ev[i]) != hipSuccess) {
+                set_error("profile_enable: hipEventCreate failed");
+                return AKV_ERR_LAUNCH;
+            }
+        }
+        g_ev_ready = true;
+    }
+    g_profile = enable != 0;
+    return AKV_OK;
+}
+
+extern "C" int akv_profile_read(float *phase_ms) {
+    AKV_REQUIRE(phase_ms != nullptr && g_ev_ready, "profile_read: profiling was never enabled");
+    if (hipEventSynchronize(g_ev[4]) != hipSuccess) {
+        set_error("profile_read: no completed step to read");
+        return AKV_ERR_LAUNCH;
+    }
+    for (int i = 0; i < 4; ++i) {
+        if (hipEventElapsedTime(&phase_ms[i], g_ev[i], g_ev[i + 1]) != hipSuccess) {
+            set_error("profile_read: hipEventElapsedTime failed");
+            return AKV_ERR_LAUNCH;
+        }
+    }
+    return AKV_OK;
+}
 
 extern "C" size_t akv_decode_step_workspace_bytes(int bsz, int n_kv_heads, int head_dim, int max_seq_len) {
     if (bsz <= 0 || n_kv_heads <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;

@@ -25,6 +25,21 @@ int check_launch(const char *what) {
 
 }  // namespace akv
 
+// Plain streaming copy, 16 bytes per thread and iteration: the known-size kernel that hardware byte
+// counters of the other kernels are scaled against.
+__global__ __launch_bounds__(256) void copy_probe_kernel(u32x4 *__restrict__ dst, const u32x4 *__restrict__ src, size_t n16) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+
+extern "C" int akv_copy_probe(void *dst, const void *src, size_t bytes, akv_stream_t stream) {
+    AKV_REQUIRE(dst && src && bytes % 16 == 0 && (((uintptr_t)dst | (uintptr_t)src) & 15) == 0,
+                "copy_probe: needs 16-byte aligned pointers and size");
+    hipLaunchKernelGGL(copy_probe_kernel, dim3(256 * 16), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<u32x4 *>(dst), static_cast<const u32x4 *>(src), bytes / 16);
+    return akv::check_launch("copy_probe");
+}
+
 extern "C" int akv_version(void) { return 100; }
 
 extern "C" const char *akv_last_error(void) { return akv::g_error; }

@@ -103,7 +103,7 @@ __global__ void v_test_kernel(const uint8_t *__restrict__ first_8, const unsigne
 // v_cache_compute
 // ------------------------------------------------------------------------------------------------
 // grid (n_chunks, H, B), 256 threads.  partial: fp32 [B*H, n_chunks, D].
-template <int D, bool REF>
+template <int D, bool REF, int NIT>
 __global__ __launch_bounds__(256) void v_compute_tuned_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const unsigned short *__restrict__ s, const uint8_t *__restrict__ amin_u8, float *__restrict__ partial,
@@ -120,7 +120,7 @@ __global__ __launch_bounds__(256) void v_compute_tuned_kernel(
     float acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    v_accumulate<D, REF>(first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
+    v_accumulate<D, REF, NIT>(first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
                          s + (int64_t)bh * s_last_dim, amin, t_begin, t_end, acc,
                          levels_out != nullptr ? levels_out + (int64_t)bh * n_tokens : nullptr);
     v_fold_workgroup<D>(acc, wave_part, partial + ((int64_t)bh * n_chunks + chunk) * D);
@@ -166,19 +166,31 @@ __global__ void v_combine_kernel(const float *__restrict__ partial, unsigned sho
     }
 }
 
+template <int D, bool REF, int NIT>
+static void launch_v_tuned_nit(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *s,
+                               const uint8_t *amin, float *partial, uint8_t *levels, int B, int H, int max_seq_len,
+                               int s_last_dim, int n_tokens, const VPlan &p, hipStream_t st) {
+    hipLaunchKernelGGL((v_compute_tuned_kernel<D, REF, NIT>), dim3(p.n_chunks, H, B), dim3(256), 0, st, f8, m4, l4,
+                       reinterpret_cast<const unsigned short *>(s), amin, partial, levels, H, max_seq_len, s_last_dim,
+                       n_tokens, p.tokens_per_wave, p.n_chunks);
+}
+
 template <int D>
 static void launch_v_tuned(bool ref, const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *s,
                            const uint8_t *amin, float *partial, uint8_t *levels, int B, int H, int max_seq_len,
                            int s_last_dim, int n_tokens, const VPlan &p, hipStream_t st) {
-    dim3 grid(p.n_chunks, H, B);
-    if (ref)
-        hipLaunchKernelGGL((v_compute_tuned_kernel<D, true>), grid, dim3(256), 0, st, f8, m4, l4,
-                           reinterpret_cast<const unsigned short *>(s), amin, partial, levels, H, max_seq_len,
-                           s_last_dim, n_tokens, p.tokens_per_wave, p.n_chunks);
-    else
-        hipLaunchKernelGGL((v_compute_tuned_kernel<D, false>), grid, dim3(256), 0, st, f8, m4, l4,
-                           reinterpret_cast<const unsigned short *>(s), amin, partial, levels, H, max_seq_len,
-                           s_last_dim, n_tokens, p.tokens_per_wave, p.n_chunks);
+#define AKV_V_CASE(R, N)                                                                                       \
+    launch_v_tuned_nit<D, R, N>(f8, m4, l4, s, amin, partial, levels, B, H, max_seq_len, s_last_dim, n_tokens, p, st)
+    if (ref) {
+        if (p.iters_per_wave == 1) AKV_V_CASE(true, 1);
+        else if (p.iters_per_wave == 2) AKV_V_CASE(true, 2);
+        else AKV_V_CASE(true, 4);
+    } else {
+        if (p.iters_per_wave == 1) AKV_V_CASE(false, 1);
+        else if (p.iters_per_wave == 2) AKV_V_CASE(false, 2);
+        else AKV_V_CASE(false, 4);
+    }
+#undef AKV_V_CASE
 }
 
 }  // namespace akv

@@ -1,0 +1,290 @@
+#!/usr/bin/env python3
+"""Benchmark of the AlignedKV decode-attention hot path on one MI355X.
+
+One "step" = one decode step of one layer at the headline configuration: batch 8, 32 heads x 128,
+4096 cached tokens in the split-precision planes, append one K/V token per sequence and attend over
+the 4097 tokens (K pass, softmax + probe, V pass, combine: one akv_decode_step call).  Inputs are
+synthetic and resident in HBM before the timed region: q ~ N(0,1), K ~ N(0,1) with 4 fixed outlier
+channels per head scaled x10, V ~ N(0,0.5), fp16 storage, fp32 accumulation.  Steps rotate over
+several layers' caches so that no step finds its planes in the 256 MiB last-level cache.
+
+Prints ONE JSON line (see the README of the harness contract): metric value = microseconds per step,
+plus `roofline` for the dominant kernel (the K pass), `cpu_baseline` (the C restatement of the
+algorithm on the host cores) and a few extra fields (effective bandwidth, bytes versus dense fp16,
+the dense baselines).
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--heads", type=int, default=32)
+    ap.add_argument("--head-dim", type=int, default=128)
+    ap.add_argument("--cache-len", type=int, default=4096)
+    ap.add_argument("--layers", type=int, default=4, help="caches the steps rotate over")
+    ap.add_argument("--k-kind", default="outlier", choices=["outlier", "lognormal"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-steps", type=int, default=3)
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a plain 256 MiB copy kernel (known size, for scaling hardware byte counters)")
+    return ap.parse_args()
+
+
+def make_layer_inputs(torch, B, L, H, D, seed, k_kind):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    k = torch.randn((B, L, H, D), device="cuda", generator=g)
+    if k_kind == "outlier":
+        for h in range(H):
+            ch = torch.randperm(D, generator=torch.Generator().manual_seed(1000 + h))[:4].cuda()
+            k[:, :, h, ch] *= 10.0
+    else:
+        k *= torch.exp(torch.randn((B, L, 1, 1), device="cuda", generator=g))
+    v = 0.5 * torch.randn((B, L, H, D), device="cuda", generator=g)
+    return k.half(), v.half()
+
+
+class StepRunner:
+    """Pre-marshalled akv_decode_step call for one layer at a fixed state (cur_len = cache_len)."""
+
+    def __init__(self, torch, lib, cache, layer, q, k_new, v_new, out, reference, record):
+        from alignedkv_amd.extension._plane_cache import column_block
+        self.lib = lib
+        kc, vc = cache.key_cache[layer], cache.value_cache[layer]
+        B, H, D = cache.max_batch_size, cache.num_key_value_heads, cache.head_dim
+        width = (kc.n_max_blocks + 1) * column_block
+        self.scores = torch.empty((B, H, width), dtype=torch.half, device="cuda")
+        self.probs = torch.empty((B, H, width), dtype=torch.half, device="cuda")
+        need = lib.akv_decode_step_workspace_bytes(B, H, D, cache.max_cache_len)
+        self.ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        R = kc.reststartpos
+        self.k_levels = torch.empty((B, H, D), dtype=torch.uint8, device="cuda") if record else None
+        self.v_levels = torch.empty((B, H, R), dtype=torch.uint8, device="cuda") if record else None
+        self.amin = torch.empty((B, H), dtype=torch.uint8, device="cuda") if record else None
+        p = lambda t: None if t is None else t.data_ptr()
+        self.keep = (q, k_new, v_new, out, kc, vc)
+        self.args = [p(kc.k_cache_first_8), p(kc.k_cache_mid_4), p(kc.k_cache_last_4), p(vc.v_cache_first_8),
+                     p(vc.v_cache_mid_4), p(vc.v_cache_last_4), p(kc._colmax), p(vc._colmax), p(kc._rest), p(vc._rest),
+                     p(q), p(k_new), p(v_new), None, 0, p(out), p(self.scores), p(self.probs), width, p(self.ws),
+                     self.ws.numel(), p(self.k_levels), p(self.v_levels), p(self.amin), B, H, kc.n_max_blocks,
+                     cache.max_cache_len, D, column_block, vc.top_max_k, kc.current_cache_len, kc.reststartpos,
+                     kc._restlen, int(reference), 0, torch.cuda.current_stream().cuda_stream]
+
+    def __call__(self):
+        rc = self.lib.akv_decode_step(*self.args)
+        if rc != 0:
+            raise RuntimeError(self.lib.akv_last_error().decode())
+
+
+def time_steps(torch, runners, steps, warmup):
+    n = len(runners)
+    for i in range(warmup):
+        runners[i % n]()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        runners[i % n]()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def phase_times(torch, lib, runners, steps):
+    """Average duration (us) of the four kernels of the step, HIP events on the step's stream."""
+    import ctypes
+    lib.akv_profile_enable(1)
+    buf = (ctypes.c_float * 4)()
+    acc = [0.0] * 4
+    n = len(runners)
+    for i in range(8):
+        runners[i % n]()
+    torch.cuda.synchronize()
+    for i in range(steps):
+        runners[i % n]()
+        if lib.akv_profile_read(buf) != 0:
+            raise RuntimeError(lib.akv_last_error().decode())
+        for j in range(4):
+            acc[j] += buf[j] * 1e3
+    lib.akv_profile_enable(0)
+    return [a / steps for a in acc]
+
+
+def algorithmic_bytes(k_levels, v_levels, B, H, D, R, L, top_k=32):
+    """Bytes one decode step has to move given the fetch levels (0: all planes, 1: no last_4, 2: high byte
+    only): per plane element 1 + 1/2 [level < 2] + 1/2 [level == 0] bytes, plus the fp16 tail, q, the
+    score/probability rows and the probe rows.  Dense fp16 reads 2 bytes per K and per V element."""
+    tail = L - R
+    k_plane = float(R) * (k_levels.size + 0.5 * (k_levels < 2).sum() + 0.5 * (k_levels == 0).sum())
+    v_plane = float(D) * (v_levels.size + 0.5 * (v_levels < 2).sum() + 0.5 * (v_levels == 0).sum())
+    k_other = B * H * tail * D * 2 + B * H * D * 3 + B * H + B * H * L * 2
+    v_other = B * H * top_k * D + B * H * L * 2 + B * H * tail * D * 2 + B * H * D * 2
+    return dict(k_plane=k_plane, v_plane=v_plane, total=k_plane + v_plane + k_other + v_other,
+                dense=float(2 * B * H * L * D * 2),
+                f_mid_k=float((k_levels < 2).mean()), f_last_k=float((k_levels == 0).mean()),
+                f_mid_v=float((v_levels < 2).mean()), f_last_v=float((v_levels == 0).mean()))
+
+
+def cpu_baseline(torch, cache, q, k_new, v_new, n_steps):
+    """The C restatement of the algorithm (oracle/akv_oracle.c, OpenMP) on the host cores, same inputs:
+    one full-size decode step (planes already flushed, one tail token), timed n_steps times."""
+    import numpy as np
+    from oracle import akv_oracle as O
+    from oracle import akv_oracle_c as OC
+    kc, vc = cache.key_cache[0], cache.value_cache[0]
+    B, H, D = cache.max_batch_size, cache.num_key_value_heads, cache.head_dim
+    R, cb = kc.reststartpos, 64
+    nb = R // cb
+    kp = [t.cpu().numpy() for t in (kc.k_cache_first_8, kc.k_cache_mid_4, kc.k_cache_last_4)]
+    vp = [t.cpu().numpy() for t in (vc.v_cache_first_8, vc.v_cache_mid_4, vc.v_cache_last_4)]
+    kcm, vcm = kc._colmax.cpu().numpy(), vc._colmax.cpu().numpy()
+    qn, kn, vn = (t.cpu().numpy() for t in (q, k_new, v_new))
+    OC.lib()
+    times = []
+    out = None
+    for _ in range(n_steps):
+        t0 = time.perf_counter()
+        kcm2 = O.colmax_update(kcm, kn)
+        vcm2 = O.colmax_update(vcm, vn)
+        ksum, kmax = O.k_sum_and_max(qn, kcm2)
+        s, klv = OC.k_cache_compute(*kp, ksum, kmax, O.as_bits(qn), nb, cb, 1.0 / math.sqrt(D), False)
+        s = s.copy()
+        restk = np.zeros((B, cb, H, D), np.float16)
+        restv = np.zeros((B, cb, H, D), np.float16)
+        restk[:, :1], restv[:, :1] = kn, vn
+        s[:, :, :, R:R + 1] = O.rest_scores(qn, restk, 1, D)
+        s[:, :, :, R + 1:] = -np.inf
+        p = O.softmax_fp32_to_half(s)
+        tv, ti = O.bucket_max(p[..., :R], R + 1)
+        to = OC.v_cache_test_compute(vp[0], O.as_bits(tv), ti, 32)
+        amin = O.alignment_min(O.test_o_exponent(to), vcm2)
+        o, vlv = OC.v_cache_compute(*vp, O.as_bits(np.ascontiguousarray(p)), amin, R, False)
+        o = (o + O.rest_output(p[..., R:R + 1], restv, 1)).astype(np.float16)
+        times.append(time.perf_counter() - t0)
+        out = o
+    return min(times), out.reshape(B, 1, H, D), klv, vlv, OC.num_threads()
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+    import alignedkv_amd
+    from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
+    from types import SimpleNamespace
+
+    lib = alignedkv_amd.load_library()
+    B, H, D, L = a.batch, a.heads, a.head_dim, a.cache_len
+    assert L % 64 == 0, "the cache length of the benchmark must be a multiple of the 64-token flush block"
+    cfg = SimpleNamespace(num_hidden_layers=a.layers, num_attention_heads=H, num_key_value_heads=H, hidden_size=H * D,
+                          max_position_embeddings=L + 64)
+    cache = QuantizedCache_AlignedKV(cfg, B, L + 64, "cuda", torch.half)
+    for layer in range(a.layers):
+        k, v = make_layer_inputs(torch, B, L, H, D, a.seed + layer, a.k_kind)
+        cache.key_cache[layer].save(k, 0, L)
+        cache.value_cache[layer].save(v, 0, L)
+        del k, v
+    g = torch.Generator(device="cuda").manual_seed(a.seed + 999)
+    q = torch.randn((B, 1, H, D), device="cuda", generator=g).half()
+    k_new = torch.randn((B, 1, H, D), device="cuda", generator=g).half()
+    v_new = (0.5 * torch.randn((B, 1, H, D), device="cuda", generator=g)).half()
+    out = torch.empty_like(q)
+    torch.cuda.synchronize()
+
+    copy_gbps = None
+    if a.copy_probe:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        st = torch.cuda.current_stream().cuda_stream
+        for _ in range(3):
+            lib.akv_copy_probe(dst.data_ptr(), src.data_ptr(), src.numel(), st)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(20):
+            lib.akv_copy_probe(dst.data_ptr(), src.data_ptr(), src.numel(), st)
+        torch.cuda.synchronize()
+        copy_gbps = 2 * src.numel() * 20 / (time.perf_counter() - t0) / 1e9
+        del src, dst
+
+    runners = [StepRunner(torch, lib, cache, i, q, k_new, v_new, out, False, i == 0) for i in range(a.layers)]
+    sec = time_steps(torch, runners, a.steps, a.warmup)
+    us = sec * 1e6
+    out_aligned = out.clone()
+    k_levels = runners[0].k_levels.cpu().numpy()
+    v_levels = runners[0].v_levels.cpu().numpy()
+
+    # bytes the algorithm has to move for this input (from the fetch decisions the kernels took)
+    R = L
+    by = algorithmic_bytes(k_levels, v_levels, B, H, D, R, L + 1)
+    eff_gbps = by["total"] / sec / 1e9
+
+    # per-kernel durations (HIP events on the stream) -> roofline of the dominant kernel, the K pass
+    ph = phase_times(torch, lib, runners, min(a.steps, 200))
+    k_pass_bytes = by["k_plane"] + B * H * D * (2 + 1 + 2) + B * H * R * 2     # planes + q, column max, new key + scores
+    v_pass_bytes = by["v_plane"] + B * H * R * 2 + B * H * D * 2 + B * H * (R // 256) * D * 4
+    achieved = k_pass_bytes / (ph[0] * 1e-6) / 1e9
+
+    # dense-in-planes baseline: same kernels, every plane read (the reference's `reference=True` mode)
+    ref_runners = [StepRunner(torch, lib, cache, i, q, k_new, v_new, out, True, False) for i in range(a.layers)]
+    sec_ref = time_steps(torch, ref_runners, max(a.steps // 2, 20), 10)
+
+    res = {
+        "metric": "decode-attn us/step (+ effective HBM GB/s, %% of peak), B=%d L=%d %dx%d" % (B, L, H, D),
+        "value": round(us, 2), "unit": "us/step", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(us / 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp16 storage, f32 accumulate", "data": "synthetic",
+        "config": {"workload": "C2: batch %d, %d heads x %d, cache %d + 1 appended token, K %s, %d layers rotated"
+                               % (B, H, D, L, a.k_kind, a.layers)},
+        "effective_hbm_gbps": round(eff_gbps, 1), "pct_hbm_peak": round(100 * eff_gbps / HBM_PEAK_GBPS, 1),
+        "algorithmic_bytes": int(by["total"]), "dense_fp16_bytes": int(by["dense"]),
+        "bytes_vs_dense": round(by["total"] / by["dense"], 4),
+        "level_fractions": {"k_mid": round(by["f_mid_k"], 4), "k_last": round(by["f_last_k"], 4),
+                            "v_mid": round(by["f_mid_v"], 4), "v_last": round(by["f_last_v"], 4)},
+        "kernel_us": {"k_pass": round(ph[0], 2), "middle": round(ph[1], 2), "v_pass": round(ph[2], 2),
+                      "combine": round(ph[3], 2)},
+        "v_pass_gbps": round(v_pass_bytes / (ph[2] * 1e-6) / 1e9, 1),
+        "dense_in_planes_us": round(sec_ref * 1e6, 2),
+        "speedup_vs_dense_in_planes": round(sec_ref / sec, 3),
+        "roofline": {"kernel": "fused_k_pass_kernel<128,false>", "bound": "hbm", "achieved": round(achieved, 1),
+                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": None, "algorithmic_bytes_per_launch": int(k_pass_bytes),
+                     "avg_launch_us": round(ph[0], 2)},
+    }
+    if copy_gbps is not None:
+        res["copy_probe_gbps_read_plus_write"] = round(copy_gbps, 1)
+    try:
+        from alignedkv_amd import dense_baseline
+        res.update(dense_baseline.bench(torch, lib, B, H, D, L + 1, a.layers, max(a.steps // 2, 20), sec))
+    except ImportError:
+        pass
+    if not a.no_cpu:
+        cpu_sec, cpu_out, cklv, cvlv, threads = cpu_baseline(torch, cache, q, k_new, v_new, a.cpu_steps)
+        runners[0]()
+        torch.cuda.synchronize()
+        err = float(np.max(np.abs(out.cpu().numpy().astype(np.float32) - cpu_out.astype(np.float32))))
+        res["cpu_baseline"] = {"value": round(cpu_sec * 1e6, 1), "unit": "us/step", "cores": threads, "kind": "port",
+                               "sample": "%d full-size steps of layer 0 (min), C restatement with OpenMP + NumPy host logic"
+                                         % a.cpu_steps}
+        res["parity"] = {"max_abs_err_vs_oracle": err, "k_levels_equal": bool(np.array_equal(cklv, k_levels)),
+                         "v_level_mismatches": int((cvlv != v_levels).sum()), "v_levels_total": int(v_levels.size)}
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -153,6 +153,16 @@ AKV_API int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_las
                             int top_max_k, int cur_len, int rest_start, int rest_len, int reference,
                             int literal_broadcast, akv_stream_t stream);
 
+/*
+ * Benchmark aid, no counterpart in the reference: with profiling enabled, akv_decode_step records HIP
+ * events on its stream around its four phases; akv_profile_read waits for the last recorded step and
+ * returns the elapsed milliseconds of {K pass, middle, V pass, combine}.  Process-wide, not thread safe.
+ */
+AKV_API int akv_profile_enable(int enable);
+/* Plain device copy of `bytes` bytes (multiple of 16): the known-size kernel hardware byte counters are scaled against. */
+AKV_API int akv_copy_probe(void *dst, const void *src, size_t bytes, akv_stream_t stream);
+AKV_API int akv_profile_read(float *phase_ms /* [4] */);
+
 #ifdef __cplusplus
 }
 #endif
