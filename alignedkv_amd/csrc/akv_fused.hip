@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
 struct MiddleArgs {
     const unsigned short *q, *k_new, *v_new, *mask;
     unsigned short *restk, *restv, *scores, *probs, *otail;
-    uint8_t *kcm, *vcm, *toe;
+    uint8_t *kcm, *vcm, *toe, *amin;
     const uint8_t *v_first_8;
     int H, cb, max_seq_len, row_stride, mask_stride;
     int R;        // flushed tokens (multiple of cb)
@@ -134,15 +134,33 @@ __device__ __forceinline__ float block_reduce(float v, bool is_max, float *red) 
     return is_max ? fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])) : ((red[0] + red[1]) + (red[2] + red[3]));
 }
 
+// Decodes 8 fp16 scores (one 16-byte vector) into floats, adding the fp16 mask in fp16 if there is one.
+__device__ __forceinline__ void decode_scores8(const u32x4 w, const unsigned short *mrow, int t0, float *x) {
+    const u32 ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const u32 lo = ww[j] & 0xffffu, hi = ww[j] >> 16;
+        if (mrow == nullptr) {
+            x[2 * j] = half_bits_to_float(lo);
+            x[2 * j + 1] = half_bits_to_float(hi);
+        } else {
+            x[2 * j] = half_bits_to_float(float_to_half_bits(half_bits_to_float(lo) + half_bits_to_float(mrow[t0 + 2 * j])));
+            x[2 * j + 1] = half_bits_to_float(float_to_half_bits(half_bits_to_float(hi) + half_bits_to_float(mrow[t0 + 2 * j + 1])));
+        }
+    }
+}
+
 template <int D>
 __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
+    constexpr int VPT = 4;                    // 16-byte score vectors a thread keeps in registers
     __shared__ float red[4];
     __shared__ unsigned short tail_s[64];     // fp16 scores of the tail (mask not yet added)
     __shared__ float tail_p[64];              // probabilities of the tail
     __shared__ float cand_v[64][33];
     __shared__ int cand_t[64][33];
-    __shared__ float probe_p[64];
-    __shared__ int probe_t[64];
+    __shared__ float probe_p[32];
+    __shared__ int probe_t[32];
+    __shared__ u32 red_min[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.x, b = bh / a.H, h = bh - b * a.H;
     const int R = a.R, nrest = a.nrest, newest = nrest - 1;
@@ -152,17 +170,35 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
     unsigned short *srow = a.scores + (int64_t)bh * a.row_stride;
     unsigned short *prow = a.probs + (int64_t)bh * a.row_stride;
     const unsigned short *mrow = a.mask ? a.mask + (int64_t)b * a.mask_stride : nullptr;
+    const int nvec = R >> 3;
+    const bool in_regs = nvec <= 256 * VPT;
 
-    // (a) append the token: rest buffers and column maxima (extension/k_cache_file.py:98-101)
-    if (a.persist) {
-        for (int d = tid; d < D; d += 256) {
+    // Everything that does not depend on anything else is requested first: the score vectors of the
+    // flushed part, the new token and the column maxima.
+    u32x4 sv[VPT];
+    if (in_regs) {
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int i = tid + 256 * v;
+            sv[v] = i < nvec ? *reinterpret_cast<const u32x4 *>(srow + i * 8) : (u32x4){0u, 0u, 0u, 0u};
+        }
+    }
+    // (a) append the token: rest buffers and column maxima (extension/k_cache_file.py:98-101).
+    //     vcm_mine: this thread's channel of the V column maxima after the update (threads < D).
+    u32 vcm_mine = 0;
+    for (int d = tid; d < D; d += 256) {
+        u32 kc = a.kcm[(int64_t)bh * D + d], vc = a.vcm[(int64_t)bh * D + d];
+        if (a.persist) {
             const u32 kb = knew[d], vb = vnew[d];
             const int64_t at = (((int64_t)b * a.cb + newest) * a.H + h) * D + d;
             a.restk[at] = (unsigned short)kb;
             a.restv[at] = (unsigned short)vb;
-            a.kcm[(int64_t)bh * D + d] = (uint8_t)max((u32)a.kcm[(int64_t)bh * D + d], exp_field(kb));
-            a.vcm[(int64_t)bh * D + d] = (uint8_t)max((u32)a.vcm[(int64_t)bh * D + d], exp_field(vb));
+            kc = max(kc, exp_field(kb));
+            vc = max(vc, exp_field(vb));
+            a.kcm[(int64_t)bh * D + d] = (uint8_t)kc;
+            a.vcm[(int64_t)bh * D + d] = (uint8_t)vc;
         }
+        vcm_mine = vc;
     }
     // (b) scores of the tail: fp16(fp16(q.k) / sqrt(D)), the two roundings of an fp16 matmul followed by
     //     an fp16 division (extension/k_cache_file.py:156)
@@ -181,41 +217,14 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
     }
     __syncthreads();
 
-    // (c) softmax over [0, L): scores + mask in fp16, softmax in fp32, probabilities in fp16
-    //     (model/KVCache_AlignedKV.py:119-121).  Flushed part 8 tokens per thread and iteration.
-    auto masked = [&](u32 sbits, int t) -> float {
+    // (c) softmax over [0, R + nrest): scores + mask in fp16, softmax in fp32, probabilities in fp16
+    //     (model/KVCache_AlignedKV.py:119-121), and the running arg-max of the residue classes mod 32:
+    //     vector i holds tokens 8i..8i+7, a thread's vectors are 256 apart, so its j-th token always has
+    //     residue (8*(tid&3) + j) mod 32.
+    auto masked1 = [&](u32 sbits, int t) -> float {
         if (mrow == nullptr) return half_bits_to_float(sbits);
         return half_bits_to_float(float_to_half_bits(half_bits_to_float(sbits) + half_bits_to_float(mrow[t])));
     };
-    const int nvec = R >> 3;
-    float m = -INFINITY;
-    for (int i = tid; i < nvec; i += 256) {
-        const u32x4 w = *reinterpret_cast<const u32x4 *>(srow + i * 8);
-        const u32 ww[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            m = fmaxf(m, masked(ww[j] & 0xffffu, i * 8 + 2 * j));
-            m = fmaxf(m, masked(ww[j] >> 16, i * 8 + 2 * j + 1));
-        }
-    }
-    if (tid < nrest) m = fmaxf(m, masked(tail_s[tid], R + tid));
-    m = block_reduce(m, true, red);
-    float sum = 0.f;
-    for (int i = tid; i < nvec; i += 256) {
-        const u32x4 w = *reinterpret_cast<const u32x4 *>(srow + i * 8);
-        const u32 ww[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            sum += expf(masked(ww[j] & 0xffffu, i * 8 + 2 * j) - m);
-            sum += expf(masked(ww[j] >> 16, i * 8 + 2 * j + 1) - m);
-        }
-    }
-    if (tid < nrest) sum += expf(masked(tail_s[tid], R + tid) - m);
-    sum = block_reduce(sum, false, red);
-
-    // probabilities + running arg-max of the 8 residue classes this thread sees: token i*8+j has residue
-    // (8*(tid&3) + j) mod 32 when 32 | top_k ... the general residue is (i*8+j) % top_k, tracked per j
-    const int top_k = a.top_k;
     float best_v[8];
     int best_t[8];
 #pragma unroll
@@ -223,43 +232,121 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
         best_v[j] = -1.f;
         best_t[j] = 0x7fffffff;
     }
-    for (int i = tid; i < nvec; i += 256) {
-        const u32x4 w = *reinterpret_cast<const u32x4 *>(srow + i * 8);
-        const u32 ww[4] = {w.x, w.y, w.z, w.w};
-        u32 out[4];
+    const float xt = tid < nrest ? masked1(tail_s[tid], R + tid) : -INFINITY;
+    float m = xt, sum = 0.f;
+    if (in_regs) {
+        float x[VPT][8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const u32 p0 = float_to_half_bits(expf(masked(ww[j] & 0xffffu, i * 8 + 2 * j) - m) / sum);
-            const u32 p1 = float_to_half_bits(expf(masked(ww[j] >> 16, i * 8 + 2 * j + 1) - m) / sum);
-            out[j] = p0 | (p1 << 16);
-            const float f0 = half_bits_to_float(p0), f1 = half_bits_to_float(p1);
-            if (f0 > best_v[2 * j]) { best_v[2 * j] = f0; best_t[2 * j] = i * 8 + 2 * j; }
-            if (f1 > best_v[2 * j + 1]) { best_v[2 * j + 1] = f1; best_t[2 * j + 1] = i * 8 + 2 * j + 1; }
+        for (int v = 0; v < VPT; ++v) {
+            const int i = tid + 256 * v;
+            if (i < nvec) {
+                decode_scores8(sv[v], mrow, i * 8, x[v]);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) m = fmaxf(m, x[v][j]);
+            }
         }
-        u32x4 o = {out[0], out[1], out[2], out[3]};
-        *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
+        m = block_reduce(m, true, red);
+#pragma unroll
+        for (int v = 0; v < VPT; ++v)
+            if (tid + 256 * v < nvec) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    x[v][j] = expf(x[v][j] - m);
+                    sum += x[v][j];
+                }
+            }
+        const float et = tid < nrest ? expf(xt - m) : 0.f;
+        sum = block_reduce(sum + et, false, red);
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int i = tid + 256 * v;
+            if (i < nvec) {
+                u32 out[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const u32 p0 = float_to_half_bits(x[v][2 * j] / sum), p1 = float_to_half_bits(x[v][2 * j + 1] / sum);
+                    out[j] = p0 | (p1 << 16);
+                    const float f0 = half_bits_to_float(p0), f1 = half_bits_to_float(p1);
+                    if (f0 > best_v[2 * j]) { best_v[2 * j] = f0; best_t[2 * j] = i * 8 + 2 * j; }
+                    if (f1 > best_v[2 * j + 1]) { best_v[2 * j + 1] = f1; best_t[2 * j + 1] = i * 8 + 2 * j + 1; }
+                }
+                const u32x4 o = {out[0], out[1], out[2], out[3]};
+                *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
+            }
+        }
+        if (tid < nrest) {
+            const unsigned short p = float_to_half_bits(et / sum);
+            prow[R + tid] = p;
+            tail_p[tid] = half_bits_to_float(p);
+        }
+    } else {
+        // long rows: three passes over the scores (they stay in the L2 of this workgroup's XCD)
+        float x[8];
+        for (int i = tid; i < nvec; i += 256) {
+            decode_scores8(*reinterpret_cast<const u32x4 *>(srow + i * 8), mrow, i * 8, x);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) m = fmaxf(m, x[j]);
+        }
+        m = block_reduce(m, true, red);
+        for (int i = tid; i < nvec; i += 256) {
+            decode_scores8(*reinterpret_cast<const u32x4 *>(srow + i * 8), mrow, i * 8, x);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) sum += expf(x[j] - m);
+        }
+        const float et = tid < nrest ? expf(xt - m) : 0.f;
+        sum = block_reduce(sum + et, false, red);
+        for (int i = tid; i < nvec; i += 256) {
+            decode_scores8(*reinterpret_cast<const u32x4 *>(srow + i * 8), mrow, i * 8, x);
+            u32 out[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const u32 p0 = float_to_half_bits(expf(x[2 * j] - m) / sum), p1 = float_to_half_bits(expf(x[2 * j + 1] - m) / sum);
+                out[j] = p0 | (p1 << 16);
+                const float f0 = half_bits_to_float(p0), f1 = half_bits_to_float(p1);
+                if (f0 > best_v[2 * j]) { best_v[2 * j] = f0; best_t[2 * j] = i * 8 + 2 * j; }
+                if (f1 > best_v[2 * j + 1]) { best_v[2 * j + 1] = f1; best_t[2 * j + 1] = i * 8 + 2 * j + 1; }
+            }
+            const u32x4 o = {out[0], out[1], out[2], out[3]};
+            *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
+        }
+        if (tid < nrest) {
+            const unsigned short p = float_to_half_bits(et / sum);
+            prow[R + tid] = p;
+            tail_p[tid] = half_bits_to_float(p);
+        }
     }
-    if (tid < nrest) {
-        const unsigned short p = float_to_half_bits(expf(masked(tail_s[tid], R + tid) - m) / sum);
-        prow[R + tid] = p;
-        tail_p[tid] = half_bits_to_float(p);
-    }
-    __syncthreads();
 
-    // (d)+(e) probe over the flushed part (extension/v_cache_file.py:119-143): needs top_k == 32 and
-    //     256 % top_k == 0 so that a thread's 8 tokens keep their residues from iteration to iteration
+    // (d)+(e) probe over the flushed part (extension/v_cache_file.py:119-143) and the alignment threshold
+    //     of this (batch, head) (extension/v_cache_file.py:156-160)
     if (R > 0) {
-        // thread tid covers residues 8*(tid&3)+j; 64 threads share each residue
+        // thread tid saw residues 8*(tid&3)+j; 64 threads share each residue
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             cand_v[tid >> 2][8 * (tid & 3) + j] = best_v[j];
             cand_t[tid >> 2][8 * (tid & 3) + j] = best_t[j];
         }
         __syncthreads();
-        if (tid < top_k) {
+        {
+            // 8 threads per residue scan 8 candidates each, then fold; ties go to the smallest token
+            const int res = tid & 31, part = tid >> 5;
             float bv = -1.f;
             int bt = 0x7fffffff;
-            for (int k = 0; k < 64; ++k) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const float v = cand_v[part * 8 + k][res];
+                const int t = cand_t[part * 8 + k][res];
+                if (v > bv || (v == bv && t < bt)) { bv = v; bt = t; }
+            }
+            __syncthreads();
+            cand_v[part][res] = bv;
+            cand_t[part][res] = bt;
+        }
+        __syncthreads();
+        if (tid < 32) {
+            float bv = -1.f;
+            int bt = 0x7fffffff;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
                 const float v = cand_v[k][tid];
                 const int t = cand_t[k][tid];
                 if (v > bv || (v == bv && t < bt)) { bv = v; bt = t; }
@@ -268,6 +355,7 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
             probe_t[tid] = bt;
         }
         __syncthreads();
+        u32 align = 0xffu;
         for (int d = tid; d < D; d += 256) {
             // the 32 gathered bytes first, then the sum: 32 independent loads in flight instead of a chain
             u32 hi[32];
@@ -278,8 +366,17 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
             for (int i = 0; i < 32; ++i)
                 acc = fmaf(half_bits_to_float(((hi[i] << 8) | 0x80u) & 0x7fffu), probe_p[i], acc);
             // exponent with the lowest bit cleared (`& 0x1F - 1`, extension/v_cache_file.py:142)
-            a.toe[(int64_t)bh * D + d] = (uint8_t)(exp_field(float_to_half_bits(acc)) & 0x1eu);
+            const u32 e = exp_field(float_to_half_bits(acc)) & 0x1eu;
+            a.toe[(int64_t)bh * D + d] = (uint8_t)e;
+            align = min(align, (e + 15u - vcm_mine) & 0xffu);     // uint8 wrap, as the reference's tensor arithmetic
         }
+#pragma unroll
+        for (int mk = 32; mk >= 1; mk >>= 1) align = min(align, (u32)__shfl_xor((int)align, mk, 64));
+        if (lane == 0) red_min[wave] = align;
+        __syncthreads();
+        if (tid == 0) a.amin[bh] = (uint8_t)min(min(red_min[0], red_min[1]), min(red_min[2], red_min[3]));
+    } else {
+        __syncthreads();
     }
     // (f) the tail's share of the output, an fp16 matmul result (extension/v_cache_file.py:189)
     for (int d = tid; d < D; d += 256) {
@@ -292,34 +389,35 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
     }
 }
 
+// Threshold indexing of the reference expression as written (extension/v_cache_file.py:157-160): entry b*H+h
+// pairs the probe of (b / H, b % H) with the column maxima of (b / H, h).  grid (B*H), 64 threads.
+__global__ void fused_amin_literal_kernel(const uint8_t *__restrict__ toe, const uint8_t *__restrict__ vcm,
+                                          uint8_t *__restrict__ amin, int H, int D) {
+    const int bh = blockIdx.x, b = bh / H, h = bh - b * H;
+    const int probe_bh = (b / H) * H + (b % H), cm_bh = (b / H) * H + h;
+    u32 mn = 0xffu;
+    for (int c = threadIdx.x; c < D; c += 64)
+        mn = min(mn, ((u32)toe[(int64_t)probe_bh * D + c] + 15u - (u32)vcm[(int64_t)cm_bh * D + c]) & 0xffu);
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) mn = min(mn, (u32)__shfl_xor((int)mn, m, 64));
+    if (threadIdx.x == 0) amin[bh] = (uint8_t)mn;
+}
+
 // ------------------------------------------------------------------------------------------------
 // V pass.  grid (n_chunks, H, B), 256 threads.
 // ------------------------------------------------------------------------------------------------
 template <int D, bool REF, int NIT>
 __global__ __launch_bounds__(256) void fused_v_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
-    const unsigned short *__restrict__ probs, const uint8_t *__restrict__ toe, const uint8_t *__restrict__ vcm,
-    float *__restrict__ partial, uint8_t *__restrict__ levels_out, uint8_t *__restrict__ amin_out, int H,
-    int max_seq_len, int row_stride, int n_tokens, int tokens_per_wave, int n_chunks, int literal_broadcast) {
+    const unsigned short *__restrict__ probs, const uint8_t *__restrict__ amin_u8, float *__restrict__ partial,
+    uint8_t *__restrict__ levels_out, uint8_t *__restrict__ amin_out, int H, int max_seq_len, int row_stride,
+    int n_tokens, int tokens_per_wave, int n_chunks) {
     __shared__ float wave_part[4][D];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wave = threadIdx.x >> 6;
     const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int bh = b * H + h;
-    // alignment threshold: min over channels of probe exponent + 15 - column max, wrapping uint8
-    // (extension/v_cache_file.py:156-160).  literal_broadcast pairs entry b*H+h with the probe of
-    // (b / H, b % H) and the column maxima of (b / H, h), which is what the reference expression reads.
-    unsigned char amin = 0;
-    if (!REF) {
-        const int probe_bh = literal_broadcast ? (b / H) * H + (b % H) : bh;
-        const int cm_bh = literal_broadcast ? (b / H) * H + h : bh;
-        u32 mn = 0xffu;
-        for (int c = lane; c < D; c += 64)
-            mn = min(mn, ((u32)toe[(int64_t)probe_bh * D + c] + 15u - (u32)vcm[(int64_t)cm_bh * D + c]) & 0xffu);
-#pragma unroll
-        for (int m = 32; m >= 1; m >>= 1) mn = min(mn, (u32)__shfl_xor((int)mn, m, 64));
-        amin = (unsigned char)mn;
-        if (amin_out != nullptr && chunk == 0 && threadIdx.x == 0) amin_out[bh] = amin;
-    }
+    const unsigned char amin = REF ? 0 : amin_u8[bh];
+    if (!REF && amin_out != nullptr && chunk == 0 && threadIdx.x == 0) amin_out[bh] = amin;
     const int t_begin = (chunk * 4 + wave) * tokens_per_wave;
     const int t_end = min(t_begin + tokens_per_wave, n_tokens);
     const int64_t row0 = (int64_t)bh * max_seq_len;
@@ -327,8 +425,8 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
     v_accumulate<D, REF, NIT>(first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
-                         probs + (int64_t)bh * row_stride, amin, t_begin, t_end, acc,
-                         levels_out != nullptr ? levels_out + (int64_t)bh * n_tokens : nullptr);
+                              probs + (int64_t)bh * row_stride, amin, t_begin, t_end, acc,
+                              levels_out != nullptr ? levels_out + (int64_t)bh * n_tokens : nullptr);
     v_fold_workgroup<D>(acc, wave_part, partial + ((int64_t)bh * n_chunks + chunk) * D);
 }
 
@@ -345,7 +443,7 @@ __global__ void fused_combine_kernel(const float *__restrict__ partial, const un
 }
 
 struct StepLayout {
-    size_t toe, otail, partial, total;
+    size_t toe, amin, otail, partial, total;
 };
 
 static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
@@ -356,7 +454,8 @@ static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
     size_t max_chunks = (size_t)(max_seq_len + 4 * (D == 256 ? 32 : 64) - 1) / (4 * (D == 256 ? 32 : 64));
     (void)p;
     l.toe = 0;
-    l.otail = up((size_t)B * H * D);
+    l.amin = up((size_t)B * H * D);
+    l.otail = l.amin + up((size_t)B * H);
     l.partial = l.otail + up((size_t)B * H * D * 2);
     l.total = l.partial + up((size_t)B * H * max_chunks * D * sizeof(float));
     return l;
@@ -371,6 +470,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
                     int rest_start, int rest_len, bool ref, int literal_broadcast, hipStream_t st) {
     const StepLayout lay = step_layout(B, H, D, max_seq_len);
     uint8_t *toe = ws + lay.toe;
+    uint8_t *amin = ws + lay.amin;
     unsigned short *otail = reinterpret_cast<unsigned short *>(ws + lay.otail);
     float *partial = reinterpret_cast<float *>(ws + lay.partial);
     const unsigned short *q16 = reinterpret_cast<const unsigned short *>(q);
@@ -417,20 +517,24 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     ma.restk = reinterpret_cast<unsigned short *>(restk);
     ma.restv = reinterpret_cast<unsigned short *>(restv);
     ma.scores = s16; ma.probs = p16; ma.otail = otail;
-    ma.kcm = kcm; ma.vcm = vcm; ma.toe = toe; ma.v_first_8 = vf8;
+    ma.kcm = kcm; ma.vcm = vcm; ma.toe = toe; ma.amin = amin; ma.v_first_8 = vf8;
     ma.H = H; ma.cb = cb; ma.max_seq_len = max_seq_len; ma.row_stride = row_stride; ma.mask_stride = mask_stride;
     ma.R = R; ma.nrest = nrest; ma.top_k = top_k; ma.persist = persist;
     hipLaunchKernelGGL((fused_middle_kernel<D>), dim3(B * H), dim3(256), 0, st, ma);
     int rc = check_launch("decode_step(middle)");
     if (rc != AKV_OK) return rc;
+    if (literal_broadcast && !ref && R > 0) {
+        hipLaunchKernelGGL(fused_amin_literal_kernel, dim3(B * H), dim3(64), 0, st, toe, vcm, amin, H, D);
+        rc = check_launch("decode_step(amin)");
+        if (rc != AKV_OK) return rc;
+    }
     mark(2, st);
     const VPlan p = v_plan(B, H, D, R);
     if (p.n_chunks > 0) {
         dim3 grid(p.n_chunks, H, B);
 #define AKV_VP(R, N)                                                                                                  \
-    hipLaunchKernelGGL((fused_v_pass_kernel<D, R, N>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, toe, vcm, partial, \
-                       v_levels_out, amin_out, H, max_seq_len, row_stride, R_tokens, p.tokens_per_wave, p.n_chunks,   \
-                       literal_broadcast)
+    hipLaunchKernelGGL((fused_v_pass_kernel<D, R, N>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, amin, partial, \
+                       v_levels_out, amin_out, H, max_seq_len, row_stride, R_tokens, p.tokens_per_wave, p.n_chunks)
         const int R_tokens = R;
         if (ref) {
             if (p.iters_per_wave == 1) AKV_VP(true, 1);
