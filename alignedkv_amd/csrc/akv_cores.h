@@ -4,6 +4,8 @@
 
 #include "akv_common.h"
 
+#include <stdlib.h>
+
 namespace akv {
 
 template <int N>
@@ -179,6 +181,7 @@ inline VPlan v_plan(int B, int H, int D, int n_tokens) {
         const int iter_tokens = D == 256 ? 32 : 64;
         int k = 1;   // iterations per wave: 1, 2 or 4
         while (k < 4 && (int64_t)B * H * ((n_tokens + 4 * iter_tokens * k * 2 - 1) / (4 * iter_tokens * k * 2)) >= 2048) k *= 2;
+        if (const char *e = getenv("AKV_TUNE_V_ITERS")) k = atoi(e) == 4 ? 4 : (atoi(e) == 2 ? 2 : 1);
         p.iters_per_wave = k;
         p.tokens_per_wave = iter_tokens * k;
         p.chunk_tokens = 4 * p.tokens_per_wave;
@@ -195,6 +198,7 @@ inline int k_blocks_per_wave(int B, int H, int n_blocks) {
     // enough waves to fill 256 CUs several times over, a few blocks per wave to amortise set-up
     int bpw = 1;
     while (bpw < 4 && (int64_t)B * H * ((n_blocks + bpw * 2 - 1) / (bpw * 2)) >= 8192) bpw *= 2;
+    if (const char *e = getenv("AKV_TUNE_K_BPW")) bpw = atoi(e) > 0 ? atoi(e) : bpw;
     return bpw;
 }
 

@@ -154,6 +154,18 @@ AKV_API int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_las
                             int literal_broadcast, akv_stream_t stream);
 
 /*
+ * Dense fp16 decode attention, the baseline of the benchmark (semantics of the reference's dense branch,
+ * model/Llama_AlignedKV.py:130-139): appends k_new / v_new at row cur_len of the head-major fp16 caches
+ * [bsz, heads, max_seq_len, head_dim] and attends over cur_len + 1 tokens.  q, k_new, v_new, out: fp16
+ * [bsz,1,heads,head_dim]; scores / probs: fp16 [bsz, heads, row_stride] scratch.  head_dim 128 only.
+ */
+AKV_API size_t akv_dense_decode_step_workspace_bytes(int bsz, int n_heads, int head_dim, int max_seq_len);
+AKV_API int akv_dense_decode_step(uint8_t *k_cache, uint8_t *v_cache, const uint8_t *q, const uint8_t *k_new,
+                                  const uint8_t *v_new, uint8_t *out, uint8_t *scores, uint8_t *probs, int row_stride,
+                                  void *workspace, size_t workspace_bytes, int bsz, int n_heads, int max_seq_len,
+                                  int head_dim, int cur_len, akv_stream_t stream);
+
+/*
  * Benchmark aid, no counterpart in the reference: with profiling enabled, akv_decode_step records HIP
  * events on its stream around its four phases; akv_profile_read waits for the last recorded step and
  * returns the elapsed milliseconds of {K pass, middle, V pass, combine}.  Process-wide, not thread safe.
