@@ -26,6 +26,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
 
+# HBM bytes per launch of the K pass at the default workload, from the rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs summarised in profiles/decode_step_c2_hbm_traffic.txt (FETCH_SIZE scaled x2.0 by the
+# known-size copy kernel, WRITE_SIZE x1.0): 222.4 MiB read + 2.0 MiB written.
+MEASURED_K_PASS_TRAFFIC = {(8, 32, 128, 4096, "outlier"): int((222.4 + 2.0) * (1 << 20))}
+
 
 def parse():
     ap = argparse.ArgumentParser()
@@ -248,7 +253,7 @@ def main():
         "metric": "decode-attn us/step (+ effective HBM GB/s, %% of peak), B=%d L=%d %dx%d" % (B, L, H, D),
         "value": round(us, 2), "unit": "us/step", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(us / 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp16 storage, f32 accumulate", "data": "synthetic",
+        "dtype": "f32", "data": "synthetic",
         "config": {"workload": "C2: batch %d, %d heads x %d, cache %d + 1 appended token, K %s, %d layers rotated"
                                % (B, H, D, L, a.k_kind, a.layers)},
         "effective_hbm_gbps": round(eff_gbps, 1), "pct_hbm_peak": round(100 * eff_gbps / HBM_PEAK_GBPS, 1),
@@ -263,7 +268,7 @@ def main():
         "speedup_vs_dense_in_planes": round(sec_ref / sec, 3),
         "roofline": {"kernel": "fused_k_pass_kernel<128,false>", "bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": None, "algorithmic_bytes_per_launch": int(k_pass_bytes),
+                     "traffic": MEASURED_K_PASS_TRAFFIC.get((B, H, D, L, a.k_kind)), "algorithmic_bytes_per_launch": int(k_pass_bytes),
                      "avg_launch_us": round(ph[0], 2)},
     }
     if copy_gbps is not None:
