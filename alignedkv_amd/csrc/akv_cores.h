@@ -28,50 +28,104 @@ __device__ __forceinline__ void reduce_scatter_step(float *a, int lane_mask) {
 //   qf[g]: q of the lane's channel in group g; bit g of need_mid / need_last: fetch that plane.
 //   s_row: fp16 scores of this (batch, head); s_row[blk*64 + slot] = fp16(dot * scale).
 // ------------------------------------------------------------------------------------------------
+template <int HG>
+struct KHalfTile {   // HG load groups of one block: 16 channels x 64 slots each
+    u32x4 h[HG];
+    u32x2 m[HG], l[HG];
+};
+
+template <int D, int HG>
+__device__ __forceinline__ void k_issue_half_h(KHalfTile<HG> &t, const __amdgpu_buffer_rsrc_t rH, int blk, int g0) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int g = 0; g < HG; ++g)
+        t.h[g] = __builtin_amdgcn_raw_buffer_load_b128(rH, blk * (D * 64) + (g0 + g) * 1024 + lane * 16, 0, 0);
+}
+
+template <int D, int HG>
+__device__ __forceinline__ void k_issue_half_ml(KHalfTile<HG> &t, const __amdgpu_buffer_rsrc_t rM,
+                                                const __amdgpu_buffer_rsrc_t rL, int blk, int g0, u32 need_mid,
+                                                u32 need_last) {
+    const int lane = threadIdx.x & 63;
+#pragma unroll
+    for (int g = 0; g < HG; ++g) {
+        const int gg = g0 + g;
+        const int mo = ((need_mid >> gg) & 1u) ? blk * (D * 32) + gg * 512 + lane * 8 : kSkip;
+        const int lo = ((need_last >> gg) & 1u) ? blk * (D * 32) + gg * 512 + lane * 8 : kSkip;
+        t.m[g] = __builtin_amdgcn_raw_buffer_load_b64(rM, mo, 0, 0);
+        t.l[g] = __builtin_amdgcn_raw_buffer_load_b64(rL, lo, 0, 0);
+    }
+}
+
+template <int D, int HG>
+__device__ __forceinline__ void k_issue_half(KHalfTile<HG> &t, const __amdgpu_buffer_rsrc_t rH,
+                                             const __amdgpu_buffer_rsrc_t rM, const __amdgpu_buffer_rsrc_t rL, int blk,
+                                             int g0, u32 need_mid, u32 need_last) {
+    k_issue_half_h<D, HG>(t, rH, blk, g0);
+    k_issue_half_ml<D, HG>(t, rM, rL, blk, g0, need_mid, need_last);
+}
+
+// The high-byte rows of the wave's first half tile do not depend on the fetch levels: a kernel calls this
+// first, works out q and the levels while the loads are in flight, then calls k_score_blocks.
 template <int D>
-__device__ __forceinline__ void k_score_blocks(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_blocks,
-                                               int first_blk, int end_blk, const float *qf, u32 need_mid,
-                                               u32 need_last, unsigned short *s_row, float scale) {
+__device__ __forceinline__ void k_prefetch_first(KHalfTile<D / 32> &ta, const uint8_t *f8, int n_blocks, int first_blk) {
+    k_issue_half_h<D, D / 32>(ta, make_rsrc(f8, (u32)n_blocks * (D * 64)), first_blk, 0);
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <int HG>
+__device__ __forceinline__ void k_compute_half(float *acc, const KHalfTile<HG> &t, int g0, const float *qf,
+                                               u32 need_mid, u32 need_last) {
+#pragma unroll
+    for (int g = 0; g < HG; ++g) {
+        const int gg = g0 + g;
+        const u32 cm = ((need_mid >> gg) & 1u) ? 0u : 0x88888888u;                                 // level 2
+        const u32 cl = (((need_mid >> gg) & 1u) && !((need_last >> gg) & 1u)) ? 0x88888888u : 0u;  // level 1
+        fma8(acc, t.h[g].x, t.h[g].y, t.m[g].x | cm, t.l[g].x | cl, qf[gg]);
+        fma8(acc + 8, t.h[g].z, t.h[g].w, t.m[g].y | cm, t.l[g].y | cl, qf[gg]);
+    }
+}
+
+// Software pipeline over half blocks: while one half tile is being multiplied, the loads of the next
+// half tile (same block or the wave's next block) are in flight.
+template <int D>
+__device__ __forceinline__ void k_score_blocks(KHalfTile<D / 32> &ta, const uint8_t *f8, const uint8_t *m4,
+                                               const uint8_t *l4, int n_blocks, int first_blk, int end_blk,
+                                               const float *qf, u32 need_mid, u32 need_last, unsigned short *s_row,
+                                               float scale) {
     constexpr int CB = 64;
     constexpr int NG = D / 16;
-    constexpr int GC = NG < 8 ? NG : 8;   // load groups in flight at a time
+    constexpr int HG = NG / 2;
     const int lane = threadIdx.x & 63;
     const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_blocks * (D * CB));
     const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_blocks * (D * CB / 2));
     const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_blocks * (D * CB / 2));
+    const int slot = (lane & 3) * 16 + ((lane & 32) ? 8 : 0) + ((lane & 16) ? 4 : 0) + ((lane & 8) ? 2 : 0) +
+                     ((lane & 4) ? 1 : 0);
+    // sched_barrier(0): the instruction scheduler must not move loads or arithmetic across the phase
+    // boundaries, otherwise it merges the two half tiles into one wait-for-everything block.  Every wait
+    // in the loop sees exactly one younger half tile in flight, from the prologue and from the back edge.
+    KHalfTile<HG> tb;
+    k_issue_half_ml<D, HG>(ta, rM, rL, first_blk, 0, need_mid, need_last);   // its high bytes: k_prefetch_first
+    __builtin_amdgcn_sched_barrier(0);
     for (int blk = first_blk; blk < end_blk; ++blk) {
         float acc[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-#pragma unroll
-        for (int g0 = 0; g0 < NG; g0 += GC) {
-            u32x4 hv[GC];
-            u32x2 mv[GC], lv[GC];
-#pragma unroll
-            for (int g = 0; g < GC; ++g) {
-                const int gg = g0 + g;
-                hv[g] = __builtin_amdgcn_raw_buffer_load_b128(rH, blk * (D * CB) + gg * 1024 + lane * 16, 0, 0);
-                int mo = ((need_mid >> gg) & 1u) ? blk * (D * CB / 2) + gg * 512 + lane * 8 : kSkip;
-                int lo = ((need_last >> gg) & 1u) ? blk * (D * CB / 2) + gg * 512 + lane * 8 : kSkip;
-                mv[g] = __builtin_amdgcn_raw_buffer_load_b64(rM, mo, 0, 0);
-                lv[g] = __builtin_amdgcn_raw_buffer_load_b64(rL, lo, 0, 0);
-            }
-#pragma unroll
-            for (int g = 0; g < GC; ++g) {
-                const int gg = g0 + g;
-                const u32 cm = ((need_mid >> gg) & 1u) ? 0u : 0x88888888u;                                 // level 2
-                const u32 cl = (((need_mid >> gg) & 1u) && !((need_last >> gg) & 1u)) ? 0x88888888u : 0u;  // level 1
-                fma8(acc, hv[g].x, hv[g].y, mv[g].x | cm, lv[g].x | cl, qf[gg]);
-                fma8(acc + 8, hv[g].z, hv[g].w, mv[g].y | cm, lv[g].y | cl, qf[gg]);
-            }
-        }
+        k_issue_half<D, HG>(tb, rH, rM, rL, blk, HG, need_mid, need_last);
+        __builtin_amdgcn_sched_barrier(0);
+        k_compute_half<HG>(acc, ta, 0, qf, need_mid, need_last);
+        __builtin_amdgcn_sched_barrier(0);
+        // past the last block the offsets fall outside the buffer resources: the loads return 0 and fetch nothing
+        k_issue_half<D, HG>(ta, rH, rM, rL, blk + 1 < end_blk ? blk + 1 : n_blocks, 0, need_mid, need_last);
+        __builtin_amdgcn_sched_barrier(0);
+        k_compute_half<HG>(acc, tb, HG, qf, need_mid, need_last);
+        __builtin_amdgcn_sched_barrier(0);
         // acc[i]: partial score of slot (lane&3)*16 + i over this lane's channels
         reduce_scatter_step<16>(acc, 32);
         reduce_scatter_step<8>(acc, 16);
         reduce_scatter_step<4>(acc, 8);
         reduce_scatter_step<2>(acc, 4);
-        const int slot = (lane & 3) * 16 + ((lane & 32) ? 8 : 0) + ((lane & 16) ? 4 : 0) + ((lane & 8) ? 2 : 0) +
-                         ((lane & 4) ? 1 : 0);
         s_row[blk * CB + slot] = float_to_half_bits(acc[0] * scale);
     }
 }
@@ -82,59 +136,142 @@ __device__ __forceinline__ void k_score_blocks(const uint8_t *f8, const uint8_t 
 //   Lane layout: lane -> token (lane / (D/16)) of each wave-wide load, channels (lane % (D/16))*16..+16.
 //   s_row: fp16 probabilities of this (batch, head).  levels_row (may be null): level per token.
 // ------------------------------------------------------------------------------------------------
-template <int D, bool REF, int NIT>
-__device__ __forceinline__ void v_accumulate(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_tokens,
-                                             const unsigned short *s_row, unsigned char amin, int t_begin, int t_end,
-                                             float *acc, uint8_t *levels_row) {
-    constexpr int LPR = D / 16;            // lanes per token row
-    constexpr int TPL = 64 / LPR;          // token rows per wave-wide load
-    constexpr int U = LPR < 8 ? LPR : 8;   // loads in flight per iteration
+// Empty volatile asm that reads and writes the 16 accumulators: pins the arithmetic that produced them
+// before this point and everything after it behind (the compiler otherwise sinks side-effect-free
+// multiply-adds past later loads and branches, which undoes the software pipeline).
+__device__ __forceinline__ void pin_accumulators(float *a) {
+    asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]),
+                      "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15]));
+}
+
+template <int HV>
+struct VHalfTile {   // HV wave-wide loads: 64/(D/16) token rows each
+    u32x4 h[HV];
+    u32x2 m[HV], l[HV];
+    u32 cm[HV], cl[HV];   // substitution bytes of skipped planes
+};
+
+// Requests the rows of the tokens base + u*TPL + tl (u < HV).  The high-byte rows do not depend on the
+// fetch level and are requested before the probabilities (sb) are looked at.
+template <int D, int HV>
+__device__ __forceinline__ void v_issue_half_h(VHalfTile<HV> &t, const __amdgpu_buffer_rsrc_t rH, int base, int t_end) {
+    constexpr int LPR = D / 16, TPL = 64 / LPR;
     const int lane = threadIdx.x & 63;
     const int tl = lane / LPR, cl = lane % LPR;
+#pragma unroll
+    for (int u = 0; u < HV; ++u) {
+        const int tok = base + u * TPL + tl;
+        t.h[u] = __builtin_amdgcn_raw_buffer_load_b128(rH, tok < t_end ? tok * D + cl * 16 : kSkip, 0, 0);
+    }
+}
+
+template <int D, bool REF, int HV>
+__device__ __forceinline__ void v_issue_half_ml(VHalfTile<HV> &t, const __amdgpu_buffer_rsrc_t rM,
+                                                const __amdgpu_buffer_rsrc_t rL, int base, int t_end, const u32 *sb,
+                                                unsigned char amin) {
+    constexpr int LPR = D / 16, TPL = 64 / LPR;
+    const int lane = threadIdx.x & 63;
+    const int tl = lane / LPR, cl = lane % LPR;
+#pragma unroll
+    for (int u = 0; u < HV; ++u) {
+        const int tok = base + u * TPL + tl;
+        const bool valid = tok < t_end;
+        const int level = REF ? 0 : v_level(amin, (unsigned short)sb[u]);
+        t.m[u] = __builtin_amdgcn_raw_buffer_load_b64(rM, (valid && level < 2) ? tok * (D / 2) + cl * 8 : kSkip, 0, 0);
+        t.l[u] = __builtin_amdgcn_raw_buffer_load_b64(rL, (valid && level == 0) ? tok * (D / 2) + cl * 8 : kSkip, 0, 0);
+        t.cm[u] = level == 2 ? 0x88888888u : 0u;
+        t.cl[u] = level == 1 ? 0x88888888u : 0u;
+    }
+}
+
+template <int D, bool REF, int HV>
+__device__ __forceinline__ void v_issue_half(VHalfTile<HV> &t, const __amdgpu_buffer_rsrc_t rH,
+                                             const __amdgpu_buffer_rsrc_t rM, const __amdgpu_buffer_rsrc_t rL, int base,
+                                             int t_end, const u32 *sb, unsigned char amin) {
+    v_issue_half_h<D, HV>(t, rH, base, t_end);
+    v_issue_half_ml<D, REF, HV>(t, rM, rL, base, t_end, sb, amin);
+}
+
+template <int D>
+struct VFirstTile {
+    VHalfTile<(D / 16 < 8 ? D / 16 : 8) / 2> t;
+};
+
+// The high-byte rows of the wave's first half tile depend on nothing: a kernel calls this first, then loads
+// the threshold, then calls v_accumulate.
+template <int D>
+__device__ __forceinline__ void v_prefetch_first(VFirstTile<D> &ft, const uint8_t *f8, int n_tokens, int t_begin, int t_end) {
+    v_issue_half_h<D, (D / 16 < 8 ? D / 16 : 8) / 2>(ft.t, make_rsrc(f8, (u32)n_tokens * D), t_begin, t_end);
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <int HV>
+__device__ __forceinline__ void v_compute_half(float *acc, const VHalfTile<HV> &t, const u32 *sb) {
+#pragma unroll
+    for (int u = 0; u < HV; ++u) {
+        const float sf = half_bits_to_float(sb[u]);
+        fma8(acc, t.h[u].x, t.h[u].y, t.m[u].x | t.cm[u], t.l[u].x | t.cl[u], sf);
+        fma8(acc + 8, t.h[u].z, t.h[u].w, t.m[u].y | t.cm[u], t.l[u].y | t.cl[u], sf);
+    }
+}
+
+template <int D, bool REF, int NIT>
+__device__ __forceinline__ void v_accumulate(VFirstTile<D> &ft, const uint8_t *f8, const uint8_t *m4, const uint8_t *l4,
+                                             int n_tokens, const unsigned short *s_row, unsigned char amin, int t_begin,
+                                             int t_end, float *acc, uint8_t *levels_row) {
+    constexpr int LPR = D / 16;            // lanes per token row
+    constexpr int TPL = 64 / LPR;          // token rows per wave-wide load
+    constexpr int U = LPR < 8 ? LPR : 8;   // wave-wide loads per batch of 64 (32 for head_dim 256) tokens
+    constexpr int HV = U / 2;              // loads per half tile
+    constexpr int NH = 2 * NIT;            // half tiles per wave
+    const int lane = threadIdx.x & 63;
+    const int tl = lane / LPR;
     const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
     const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_tokens * (D / 2));
     const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_tokens * (D / 2));
     const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)n_tokens * 2);
     // The probabilities of all the wave's tokens first: the fetch level of a token depends on its
-    // probability, and a load per iteration would put a memory round trip in front of every batch.
-    u32 sb[NIT][U];
+    // probability, and a load per batch would put a memory round trip in front of every batch.
+    u32 sb[NH][HV];
 #pragma unroll
-    for (int it = 0; it < NIT; ++it)
+    for (int hf = 0; hf < NH; ++hf)
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int t = t_begin + (it * U + u) * TPL + tl;
-            sb[it][u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < t_end ? t * 2 : kSkip, 0, 0);
+        for (int u = 0; u < HV; ++u) {
+            const int t = t_begin + (hf * HV + u) * TPL + tl;
+            sb[hf][u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < t_end ? t * 2 : kSkip, 0, 0);
         }
+    __builtin_amdgcn_sched_barrier(0);
+    // Software pipeline over half tiles (see k_score_blocks): one half tile is in flight while the other is
+    // multiplied; sched_barrier(0) keeps the instruction scheduler from merging the phases.
+    VHalfTile<HV> &ta = ft.t;
+    VHalfTile<HV> tb;
+    v_issue_half_ml<D, REF, HV>(ta, rM, rL, t_begin, t_end, sb[0], amin);   // its high bytes: v_prefetch_first
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int it = 0; it < NIT; ++it) {
-        const int base = t_begin + it * U * TPL;
-        if (base >= t_end) break;
-        u32x4 hv[U];
-        u32x2 mv[U], lv[U];
-        // the high-byte rows do not depend on the level: issue them before the probabilities are looked at
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int t = base + u * TPL + tl;
-            hv[u] = __builtin_amdgcn_raw_buffer_load_b128(rH, t < t_end ? t * D + cl * 16 : kSkip, 0, 0);
+    for (int hf = 0; hf < NH; hf += 2) {
+        v_issue_half<D, REF, HV>(tb, rH, rM, rL, t_begin + (hf + 1) * HV * TPL, t_end, sb[hf + 1], amin);
+        __builtin_amdgcn_sched_barrier(0);
+        v_compute_half<HV>(acc, ta, sb[hf]);
+        pin_accumulators(acc);
+        __builtin_amdgcn_sched_barrier(0);
+        if (hf + 2 < NH) {
+            v_issue_half<D, REF, HV>(ta, rH, rM, rL, t_begin + (hf + 2) * HV * TPL, t_end, sb[hf + 2], amin);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        u32 cm[U], cl_[U];
+        v_compute_half<HV>(acc, tb, sb[hf + 1]);
+        pin_accumulators(acc);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // optional record of the levels, outside the pipeline (a store under a branch inside it would split
+    // the loop body into blocks and let the compiler sink the arithmetic past the loads)
+    if (levels_row != nullptr && (lane % LPR) == 0) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int t = base + u * TPL + tl;
-            const bool valid = t < t_end;
-            const int level = REF ? 0 : v_level(amin, (unsigned short)sb[it][u]);
-            mv[u] = __builtin_amdgcn_raw_buffer_load_b64(rM, (valid && level < 2) ? t * (D / 2) + cl * 8 : kSkip, 0, 0);
-            lv[u] = __builtin_amdgcn_raw_buffer_load_b64(rL, (valid && level == 0) ? t * (D / 2) + cl * 8 : kSkip, 0, 0);
-            cm[u] = level == 2 ? 0x88888888u : 0u;
-            cl_[u] = level == 1 ? 0x88888888u : 0u;
-            if (levels_row != nullptr && valid && cl == 0) levels_row[t] = (uint8_t)level;
-        }
+        for (int hf = 0; hf < NH; ++hf)
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const float sf = half_bits_to_float(sb[it][u]);
-            fma8(acc, hv[u].x, hv[u].y, mv[u].x | cm[u], lv[u].x | cl_[u], sf);
-            fma8(acc + 8, hv[u].z, hv[u].w, mv[u].y | cm[u], lv[u].y | cl_[u], sf);
-        }
+            for (int u = 0; u < HV; ++u) {
+                const int t = t_begin + (hf * HV + u) * TPL + tl;
+                if (t < t_end) levels_row[t] = (uint8_t)(REF ? 0 : v_level(amin, (unsigned short)sb[hf][u]));
+            }
     }
 }
 

@@ -82,6 +82,9 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     if (first_blk >= n_blocks) return;
     const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
 
+    const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
+    KHalfTile<D / 32> ta;
+    k_prefetch_first<D>(ta, first_8 + plane_off * 2, n_blocks, first_blk);
     float qf[NG];
     u32 esum[NG];
     u32 mx = 0;
@@ -106,8 +109,7 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
         if (levels_out != nullptr && blockIdx.x == 0 && wave == 0 && (lane & 3) == 0)
             levels_out[(int64_t)bh * D + g * 16 + (lane >> 2)] = (uint8_t)lv;
     }
-    const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
-    k_score_blocks<D>(first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
+    k_score_blocks<D>(ta, first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
                       need_mid, need_last, scores + (int64_t)bh * row_stride, scale);
 }
 
@@ -416,15 +418,17 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
     const int wave = threadIdx.x >> 6;
     const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int bh = b * H + h;
-    const unsigned char amin = REF ? 0 : amin_u8[bh];
-    if (!REF && amin_out != nullptr && chunk == 0 && threadIdx.x == 0) amin_out[bh] = amin;
     const int t_begin = (chunk * 4 + wave) * tokens_per_wave;
     const int t_end = min(t_begin + tokens_per_wave, n_tokens);
     const int64_t row0 = (int64_t)bh * max_seq_len;
+    VFirstTile<D> ft;
+    v_prefetch_first<D>(ft, first_8 + row0 * D, n_tokens, t_begin, t_end);
+    const unsigned char amin = REF ? 0 : amin_u8[bh];
+    if (!REF && amin_out != nullptr && chunk == 0 && threadIdx.x == 0) amin_out[bh] = amin;
     float acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    v_accumulate<D, REF, NIT>(first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
+    v_accumulate<D, REF, NIT>(ft, first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
                               probs + (int64_t)bh * row_stride, amin, t_begin, t_end, acc,
                               levels_out != nullptr ? levels_out + (int64_t)bh * n_tokens : nullptr);
     v_fold_workgroup<D>(acc, wave_part, partial + ((int64_t)bh * n_chunks + chunk) * D);

@@ -129,6 +129,9 @@ __global__ __launch_bounds__(256) void k_compute_cb64_kernel(
     if (first_blk >= n_blocks) return;
     const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
 
+    const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
+    KHalfTile<D / 32> ta;
+    k_prefetch_first<D>(ta, first_8 + plane_off * 2, n_blocks, first_blk);
     // per-lane channel data: channel of group g is g*16 + lane/4
     float qf[NG];
     u32 need_mid = 0, need_last = 0;
@@ -143,8 +146,7 @@ __global__ __launch_bounds__(256) void k_compute_cb64_kernel(
         if (levels_out != nullptr && blockIdx.x == 0 && wave == 0 && (lane & 3) == 0)
             levels_out[(int64_t)bh * D + c] = (uint8_t)lv;
     }
-    const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
-    k_score_blocks<D>(first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
+    k_score_blocks<D>(ta, first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
                       need_mid, need_last, s + (int64_t)bh * ((int64_t)(n_blocks + 1) * CB), scale);
 }
 

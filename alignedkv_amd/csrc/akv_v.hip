@@ -115,12 +115,14 @@ __global__ __launch_bounds__(256) void v_compute_tuned_kernel(
     const int bh = b * H + h;
     const int t_begin = (chunk * 4 + wave) * tokens_per_wave;
     const int t_end = min(t_begin + tokens_per_wave, n_tokens);
-    const unsigned char amin = REF ? 0 : amin_u8[bh];
     const int64_t row0 = (int64_t)bh * max_seq_len;
+    VFirstTile<D> ft;
+    v_prefetch_first<D>(ft, first_8 + row0 * D, n_tokens, t_begin, t_end);
+    const unsigned char amin = REF ? 0 : amin_u8[bh];
     float acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    v_accumulate<D, REF, NIT>(first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
+    v_accumulate<D, REF, NIT>(ft, first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
                          s + (int64_t)bh * s_last_dim, amin, t_begin, t_end, acc,
                          levels_out != nullptr ? levels_out + (int64_t)bh * n_tokens : nullptr);
     v_fold_workgroup<D>(acc, wave_part, partial + ((int64_t)bh * n_chunks + chunk) * D);
