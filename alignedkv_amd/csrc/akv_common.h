@@ -89,6 +89,24 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, u3
 }
 constexpr int kSkip = 0x7fffffff;   // an offset no plane slice reaches
 
+// Cache-policy bits of buffer loads/stores on gfx950: sc1 = device (agent) scope.  Data that one
+// workgroup writes and another workgroup of the SAME launch reads (scores, partial sums) goes through
+// these: the eight XCDs have separate L2 caches that are only reconciled at kernel boundaries, and a
+// device-wide fence (write back + invalidate of a whole L2) costs far more than the few bytes exchanged.
+constexpr int kDeviceScope = 1 << 4;
+__device__ __forceinline__ void store_u16_device(const __amdgpu_buffer_rsrc_t r, int byte_off, unsigned short v) {
+    __builtin_amdgcn_raw_buffer_store_b16((short)v, r, byte_off, 0, kDeviceScope);
+}
+__device__ __forceinline__ void store_f32_device(const __amdgpu_buffer_rsrc_t r, int byte_off, float v) {
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, byte_off, 0, kDeviceScope);
+}
+__device__ __forceinline__ float load_f32_device(const __amdgpu_buffer_rsrc_t r, int byte_off) {
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, kDeviceScope));
+}
+__device__ __forceinline__ u32x4 load_b128_device(const __amdgpu_buffer_rsrc_t r, int byte_off) {
+    return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, kDeviceScope);
+}
+
 __device__ __forceinline__ float wave_xor_add(float v, int mask) { return v + __shfl_xor(v, mask, 64); }
 
 }  // namespace akv

@@ -100,6 +100,7 @@ __device__ __forceinline__ void k_score_blocks(KHalfTile<D / 32> &ta, const uint
     const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_blocks * (D * CB));
     const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_blocks * (D * CB / 2));
     const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_blocks * (D * CB / 2));
+    const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)n_blocks * CB * 2);
     const int slot = (lane & 3) * 16 + ((lane & 32) ? 8 : 0) + ((lane & 16) ? 4 : 0) + ((lane & 8) ? 2 : 0) +
                      ((lane & 4) ? 1 : 0);
     // sched_barrier(0): the instruction scheduler must not move loads or arithmetic across the phase
@@ -126,7 +127,8 @@ __device__ __forceinline__ void k_score_blocks(KHalfTile<D / 32> &ta, const uint
         reduce_scatter_step<8>(acc, 16);
         reduce_scatter_step<4>(acc, 8);
         reduce_scatter_step<2>(acc, 4);
-        s_row[blk * CB + slot] = float_to_half_bits(acc[0] * scale);
+        // device scope: the workgroup that runs the softmax for this (batch, head) may sit on another XCD
+        store_u16_device(rS, (blk * CB + slot) * 2, float_to_half_bits(acc[0] * scale));
     }
 }
 
@@ -298,8 +300,9 @@ __device__ __forceinline__ void v_fold_workgroup(float *acc, float (*wave_part)[
 #pragma unroll
     for (int i = 0; i < NV; ++i) wave_part[wave][ch + i] = acc[i];
     __syncthreads();
+    const __amdgpu_buffer_rsrc_t rO = make_rsrc(out, (u32)D * 4);
     for (int d = threadIdx.x; d < D; d += 256)
-        out[d] = (wave_part[0][d] + wave_part[1][d]) + (wave_part[2][d] + wave_part[3][d]);
+        store_f32_device(rO, d * 4, (wave_part[0][d] + wave_part[1][d]) + (wave_part[2][d] + wave_part[3][d]));
 }
 
 // Split of the sequence over workgroups for the V pass (shared by the op and the fused step).

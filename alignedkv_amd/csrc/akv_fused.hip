@@ -16,6 +16,8 @@
 // run first, exactly as the reference flushes before it computes.
 #include "akv_cores.h"
 
+#include <atomic>
+
 namespace akv {
 
 // defined in akv_k.hip / akv_v.hip
@@ -32,8 +34,33 @@ __device__ __forceinline__ u32 exp_field(u32 half_bits) { return (half_bits >> 1
 static bool g_profile = false;
 static hipEvent_t g_ev[5];
 static bool g_ev_ready = false;
+// epochs of the arrival counters: process-wide, never 0
+static std::atomic<unsigned long long> g_epoch_source{1};
+static inline unsigned long long next_epoch() {
+    unsigned long long e = g_epoch_source.fetch_add(1) & 0xffffffffffffull;
+    return e ? e : (g_epoch_source.fetch_add(1) & 0xffffffffffffull);
+}
 static inline void mark(int i, hipStream_t st) {
     if (g_profile) (void)hipEventRecord(g_ev[i], st);
+}
+
+// Arrival counter that needs no initialisation: a 64-bit word holds (epoch << 16 | arrivals).  Every call of
+// the step uses a fresh epoch (process-wide counter on the host), so whatever an earlier call or an
+// uninitialised workspace left in the word reads as "no arrival yet".  Returns true for the last of
+// `expected` arrivals.  Call with one thread per workgroup, after a __threadfence() + __syncthreads().
+__device__ __forceinline__ bool arrive_and_test_last(unsigned long long *word, unsigned long long epoch, u32 expected) {
+    unsigned long long seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    while (true) {
+        const unsigned long long count = (seen >> 16) == epoch ? (seen & 0xffffull) : 0ull;
+        const unsigned long long want = (epoch << 16) | (count + 1);
+        if (__hip_atomic_compare_exchange_strong(word, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT)) {
+            if (count + 1 != expected) return false;
+            // leave the word empty: a captured graph replays the step with the epoch it was recorded with
+            __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return true;
+        }
+    }
 }
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -64,6 +91,21 @@ __global__ void fused_persist_kernel(const unsigned short *__restrict__ k_new, c
     }
 }
 
+struct MiddleArgs {
+    const unsigned short *q, *k_new, *v_new, *mask;
+    unsigned short *restk, *restv, *scores, *probs, *otail;
+    uint8_t *kcm, *vcm, *toe, *amin;
+    const uint8_t *v_first_8;
+    int H, cb, max_seq_len, row_stride, mask_stride;
+    int R;        // flushed tokens (multiple of cb)
+    int nrest;    // tokens in the rest buffer including the one of this step (0 on a flush step)
+    int top_k;
+    int persist;  // this kernel appends the token (no flush happened in this step)
+};
+
+template <int D>
+__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh);
+
 // ------------------------------------------------------------------------------------------------
 // K pass.  grid (ceil(n_blocks / (4*blocks_per_wave)), H, B), 256 threads.
 // ------------------------------------------------------------------------------------------------
@@ -72,14 +114,14 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
     unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, int n_blocks, int n_max_blocks, int H,
-    int row_stride, int blocks_per_wave, float scale) {
+    int row_stride, int blocks_per_wave, float scale, MiddleArgs ma, unsigned long long *done_k,
+    unsigned long long epoch) {
     constexpr int CB = 64;
     constexpr int NG = D / 16;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int h = blockIdx.y, b = blockIdx.z;
     const int bh = b * H + h;
-    const int first_blk = (blockIdx.x * 4 + wave) * blocks_per_wave;
-    if (first_blk >= n_blocks) return;
+    const int first_blk = (blockIdx.x * 4 + wave) * blocks_per_wave;   // may lie past the end: the wave then idles
     const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
 
     const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
@@ -111,23 +153,23 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     }
     k_score_blocks<D>(ta, first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
                       need_mid, need_last, scores + (int64_t)bh * row_stride, scale);
+    if (done_k == nullptr) return;
+    // The workgroup that finishes the last chunk of this (batch, head) runs the middle stage for it, while
+    // other workgroups are still streaming their blocks: no separate launch, no idle machine in between.
+    // The scores were stored at device scope; the workgroup-scope fence + barrier below waits until every
+    // wave's stores have completed before one thread reports the arrival, and the middle stage reads the
+    // scores at device scope: no device-wide fence (a whole-L2 write back and invalidate) is needed.
+    __shared__ int is_last;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    if (threadIdx.x == 0) is_last = arrive_and_test_last(done_k + bh, epoch, gridDim.x) ? 1 : 0;
+    __syncthreads();
+    if (is_last) middle_body<D>(ma, bh);
 }
 
 // ------------------------------------------------------------------------------------------------
 // middle.  grid (B*H), 256 threads.
 // ------------------------------------------------------------------------------------------------
-struct MiddleArgs {
-    const unsigned short *q, *k_new, *v_new, *mask;
-    unsigned short *restk, *restv, *scores, *probs, *otail;
-    uint8_t *kcm, *vcm, *toe, *amin;
-    const uint8_t *v_first_8;
-    int H, cb, max_seq_len, row_stride, mask_stride;
-    int R;        // flushed tokens (multiple of cb)
-    int nrest;    // tokens in the rest buffer including the one of this step (0 on a flush step)
-    int top_k;
-    int persist;  // this kernel appends the token (no flush happened in this step)
-};
-
 __device__ __forceinline__ float block_reduce(float v, bool is_max, float *red) {
     v = is_max ? wave_max(v) : wave_sum(v);
     __syncthreads();
@@ -153,7 +195,7 @@ __device__ __forceinline__ void decode_scores8(const u32x4 w, const unsigned sho
 }
 
 template <int D>
-__global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
+__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     constexpr int VPT = 4;                    // 16-byte score vectors a thread keeps in registers
     __shared__ float red[4];
     __shared__ unsigned short tail_s[64];     // fp16 scores of the tail (mask not yet added)
@@ -164,7 +206,7 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
     __shared__ int probe_t[32];
     __shared__ u32 red_min[4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int bh = blockIdx.x, b = bh / a.H, h = bh - b * a.H;
+    const int b = bh / a.H, h = bh - b * a.H;
     const int R = a.R, nrest = a.nrest, newest = nrest - 1;
     const unsigned short *qrow = a.q + (int64_t)bh * D;
     const unsigned short *knew = a.k_new + (int64_t)bh * D;
@@ -174,6 +216,8 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
     const unsigned short *mrow = a.mask ? a.mask + (int64_t)b * a.mask_stride : nullptr;
     const int nvec = R >> 3;
     const bool in_regs = nvec <= 256 * VPT;
+    // scores of the flushed part are read at device scope: other workgroups of the same launch wrote them
+    const __amdgpu_buffer_rsrc_t rScores = make_rsrc(srow, (u32)R * 2);
 
     // Everything that does not depend on anything else is requested first: the score vectors of the
     // flushed part, the new token and the column maxima.
@@ -182,7 +226,7 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
             const int i = tid + 256 * v;
-            sv[v] = i < nvec ? *reinterpret_cast<const u32x4 *>(srow + i * 8) : (u32x4){0u, 0u, 0u, 0u};
+            sv[v] = load_b128_device(rScores, i < nvec ? i * 16 : kSkip);
         }
     }
     // (a) append the token: rest buffers and column maxima (extension/k_cache_file.py:98-101).
@@ -285,20 +329,20 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
         // long rows: three passes over the scores (they stay in the L2 of this workgroup's XCD)
         float x[8];
         for (int i = tid; i < nvec; i += 256) {
-            decode_scores8(*reinterpret_cast<const u32x4 *>(srow + i * 8), mrow, i * 8, x);
+            decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
 #pragma unroll
             for (int j = 0; j < 8; ++j) m = fmaxf(m, x[j]);
         }
         m = block_reduce(m, true, red);
         for (int i = tid; i < nvec; i += 256) {
-            decode_scores8(*reinterpret_cast<const u32x4 *>(srow + i * 8), mrow, i * 8, x);
+            decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
 #pragma unroll
             for (int j = 0; j < 8; ++j) sum += expf(x[j] - m);
         }
         const float et = tid < nrest ? expf(xt - m) : 0.f;
         sum = block_reduce(sum + et, false, red);
         for (int i = tid; i < nvec; i += 256) {
-            decode_scores8(*reinterpret_cast<const u32x4 *>(srow + i * 8), mrow, i * 8, x);
+            decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
             u32 out[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -391,6 +435,12 @@ __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
     }
 }
 
+// grid (B*H), 256 threads: the middle stage on its own (no flushed block yet, or fusion switched off).
+template <int D>
+__global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
+    middle_body<D>(a, blockIdx.x);
+}
+
 // Threshold indexing of the reference expression as written (extension/v_cache_file.py:157-160): entry b*H+h
 // pairs the probe of (b / H, b % H) with the column maxima of (b / H, h).  grid (B*H), 64 threads.
 __global__ void fused_amin_literal_kernel(const uint8_t *__restrict__ toe, const uint8_t *__restrict__ vcm,
@@ -413,7 +463,8 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const unsigned short *__restrict__ probs, const uint8_t *__restrict__ amin_u8, float *__restrict__ partial,
     uint8_t *__restrict__ levels_out, uint8_t *__restrict__ amin_out, int H, int max_seq_len, int row_stride,
-    int n_tokens, int tokens_per_wave, int n_chunks) {
+    int n_tokens, int tokens_per_wave, int n_chunks, const unsigned short *__restrict__ otail,
+    unsigned short *__restrict__ out, unsigned long long *done_v, unsigned long long epoch) {
     __shared__ float wave_part[4][D];
     const int wave = threadIdx.x >> 6;
     const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -432,6 +483,23 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
                               probs + (int64_t)bh * row_stride, amin, t_begin, t_end, acc,
                               levels_out != nullptr ? levels_out + (int64_t)bh * n_tokens : nullptr);
     v_fold_workgroup<D>(acc, wave_part, partial + ((int64_t)bh * n_chunks + chunk) * D);
+    if (done_v == nullptr) return;
+    // The workgroup that delivers the last chunk of this (batch, head) adds the partials up (in chunk order:
+    // the output bits do not depend on which workgroup comes last) and writes the output.
+    __shared__ int is_last;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // partial sums were stored at device scope
+    __syncthreads();
+    if (threadIdx.x == 0) is_last = arrive_and_test_last(done_v + bh, epoch, (u32)n_chunks) ? 1 : 0;
+    __syncthreads();
+    if (is_last) {
+        const __amdgpu_buffer_rsrc_t rP = make_rsrc(partial + (int64_t)bh * n_chunks * D, (u32)n_chunks * D * 4);
+        for (int d = threadIdx.x; d < D; d += 256) {
+            float sum = 0.f;
+            for (int c = 0; c < n_chunks; ++c) sum += load_f32_device(rP, (c * D + d) * 4);
+            const float o16 = half_bits_to_float(float_to_half_bits(sum));
+            out[(int64_t)bh * D + d] = float_to_half_bits(o16 + half_bits_to_float(otail[(int64_t)bh * D + d]));
+        }
+    }
 }
 
 // grid (B*H), D threads: out = fp16(fp16(sum of partials) + tail), the fp16 `o += tail` of the reference.
@@ -447,7 +515,7 @@ __global__ void fused_combine_kernel(const float *__restrict__ partial, const un
 }
 
 struct StepLayout {
-    size_t toe, amin, otail, partial, total;
+    size_t done_k, done_v, toe, amin, otail, partial, total;
 };
 
 static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
@@ -457,8 +525,10 @@ static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
     // the plan for fewer tokens never has more chunks than the plan for max_seq_len has at its finest split
     size_t max_chunks = (size_t)(max_seq_len + 4 * (D == 256 ? 32 : 64) - 1) / (4 * (D == 256 ? 32 : 64));
     (void)p;
-    l.toe = 0;
-    l.amin = up((size_t)B * H * D);
+    l.done_k = 0;
+    l.done_v = up((size_t)B * H * 8);
+    l.toe = l.done_v + up((size_t)B * H * 8);
+    l.amin = l.toe + up((size_t)B * H * D);
     l.otail = l.amin + up((size_t)B * H);
     l.partial = l.otail + up((size_t)B * H * D * 2);
     l.total = l.partial + up((size_t)B * H * max_chunks * D * sizeof(float));
@@ -475,6 +545,15 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     const StepLayout lay = step_layout(B, H, D, max_seq_len);
     uint8_t *toe = ws + lay.toe;
     uint8_t *amin = ws + lay.amin;
+    // Optional fusion of the middle stage into the K pass and of the combine stage into the V pass ("last
+    // workgroup of a (batch, head) does the next stage").  Measured slower than separate launches on MI355X
+    // (every workgroup has to wait for its device-scope stores and the arrival atomic before it can retire),
+    // so it is off unless AKV_TUNE_TAIL_FUSION=1.
+    static const bool no_fusion = getenv("AKV_TUNE_TAIL_FUSION") == nullptr;
+    const unsigned long long epoch = next_epoch();
+    const bool fuse_middle = !no_fusion && !(literal_broadcast && !ref);   // the literal threshold needs every probe first
+    unsigned long long *done_k = fuse_middle ? reinterpret_cast<unsigned long long *>(ws + lay.done_k) : nullptr;
+    unsigned long long *done_v = !no_fusion ? reinterpret_cast<unsigned long long *>(ws + lay.done_v) : nullptr;
     unsigned short *otail = reinterpret_cast<unsigned short *>(ws + lay.otail);
     float *partial = reinterpret_cast<float *>(ws + lay.partial);
     const unsigned short *q16 = reinterpret_cast<const unsigned short *>(q);
@@ -499,22 +578,6 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         persist = 0;
     }
     const int n_blocks = R / cb;
-    mark(0, st);
-    // the kernel multiplies by the fp16-rounded scale (extension/csrc/K_cache.cu:306)
-    const float scale = __half2float(__float2half_rn(1.0f / sqrtf((float)D)));
-    if (n_blocks > 0) {
-        const int bpw = k_blocks_per_wave(B, H, n_blocks);
-        dim3 grid((n_blocks + 4 * bpw - 1) / (4 * bpw), H, B);
-        if (ref)
-            hipLaunchKernelGGL((fused_k_pass_kernel<D, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                               k_levels_out, n_blocks, n_max_blocks, H, row_stride, bpw, scale);
-        else
-            hipLaunchKernelGGL((fused_k_pass_kernel<D, false>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                               k_levels_out, n_blocks, n_max_blocks, H, row_stride, bpw, scale);
-        int rc = check_launch("decode_step(k_pass)");
-        if (rc != AKV_OK) return rc;
-    }
-    mark(1, st);
     MiddleArgs ma;
     ma.q = q16; ma.k_new = k16; ma.v_new = v16;
     ma.mask = reinterpret_cast<const unsigned short *>(mask);
@@ -524,9 +587,30 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     ma.kcm = kcm; ma.vcm = vcm; ma.toe = toe; ma.amin = amin; ma.v_first_8 = vf8;
     ma.H = H; ma.cb = cb; ma.max_seq_len = max_seq_len; ma.row_stride = row_stride; ma.mask_stride = mask_stride;
     ma.R = R; ma.nrest = nrest; ma.top_k = top_k; ma.persist = persist;
-    hipLaunchKernelGGL((fused_middle_kernel<D>), dim3(B * H), dim3(256), 0, st, ma);
-    int rc = check_launch("decode_step(middle)");
-    if (rc != AKV_OK) return rc;
+    mark(0, st);
+    // the kernel multiplies by the fp16-rounded scale (extension/csrc/K_cache.cu:306)
+    const float scale = __half2float(__float2half_rn(1.0f / sqrtf((float)D)));
+    bool middle_done = false;
+    if (n_blocks > 0) {
+        const int bpw = k_blocks_per_wave(B, H, n_blocks);
+        dim3 grid((n_blocks + 4 * bpw - 1) / (4 * bpw), H, B);
+        if (ref)
+            hipLaunchKernelGGL((fused_k_pass_kernel<D, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
+                               k_levels_out, n_blocks, n_max_blocks, H, row_stride, bpw, scale, ma, done_k, epoch);
+        else
+            hipLaunchKernelGGL((fused_k_pass_kernel<D, false>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
+                               k_levels_out, n_blocks, n_max_blocks, H, row_stride, bpw, scale, ma, done_k, epoch);
+        int rc = check_launch("decode_step(k_pass)");
+        if (rc != AKV_OK) return rc;
+        middle_done = done_k != nullptr;
+    }
+    mark(1, st);
+    int rc = AKV_OK;
+    if (!middle_done) {
+        hipLaunchKernelGGL((fused_middle_kernel<D>), dim3(B * H), dim3(256), 0, st, ma);
+        rc = check_launch("decode_step(middle)");
+        if (rc != AKV_OK) return rc;
+    }
     if (literal_broadcast && !ref && R > 0) {
         hipLaunchKernelGGL(fused_amin_literal_kernel, dim3(B * H), dim3(64), 0, st, toe, vcm, amin, H, D);
         rc = check_launch("decode_step(amin)");
@@ -538,7 +622,8 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         dim3 grid(p.n_chunks, H, B);
 #define AKV_VP(R, N)                                                                                                  \
     hipLaunchKernelGGL((fused_v_pass_kernel<D, R, N>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, amin, partial, \
-                       v_levels_out, amin_out, H, max_seq_len, row_stride, R_tokens, p.tokens_per_wave, p.n_chunks)
+                       v_levels_out, amin_out, H, max_seq_len, row_stride, R_tokens, p.tokens_per_wave, p.n_chunks,   \
+                       otail, reinterpret_cast<unsigned short *>(out), done_v, epoch)
         const int R_tokens = R;
         if (ref) {
             if (p.iters_per_wave == 1) AKV_VP(true, 1);
@@ -554,11 +639,14 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
     }
     mark(3, st);
-    hipLaunchKernelGGL(fused_combine_kernel, dim3(B * H), dim3(D < 256 ? D : 256), 0, st, partial, otail,
-                       reinterpret_cast<unsigned short *>(out), D, p.n_chunks);
+    if (p.n_chunks == 0 || done_v == nullptr) {
+        hipLaunchKernelGGL(fused_combine_kernel, dim3(B * H), dim3(D < 256 ? D : 256), 0, st, partial, otail,
+                           reinterpret_cast<unsigned short *>(out), D, p.n_chunks);
+        rc = check_launch("decode_step(combine)");
+    }
     mark(4, st);
     (void)cur_len;
-    return check_launch("decode_step(combine)");
+    return rc;
 }
 
 }  // namespace akv
