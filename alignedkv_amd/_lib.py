@@ -8,7 +8,7 @@ from ctypes import c_float, c_int, c_size_t, c_void_p
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_PKG, "csrc")
-LIB_PATH = os.path.join(_PKG, "libalignedkv_hip.so")
+LIB_PATH = os.environ.get("ALIGNEDKV_LIB", os.path.join(_PKG, "libalignedkv_hip.so"))
 HEADER = os.path.join(os.path.dirname(_PKG), "include", "alignedkv.h")
 
 _lib = None

@@ -178,9 +178,19 @@ __device__ __forceinline__ void v_issue_half_ml(VHalfTile<HV> &t, const __amdgpu
     for (int u = 0; u < HV; ++u) {
         const int tok = base + u * TPL + tl;
         const bool valid = tok < t_end;
+#if defined(AKV_V_VARIANT) && AKV_V_VARIANT >= 1
+        const int level = 2;
+        (void)valid;
+#else
         const int level = REF ? 0 : v_level(amin, (unsigned short)sb[u]);
+#endif
+#if defined(AKV_V_VARIANT) && AKV_V_VARIANT >= 2
+        t.m[u] = (u32x2){0u, 0u};
+        t.l[u] = (u32x2){0u, 0u};
+#else
         t.m[u] = __builtin_amdgcn_raw_buffer_load_b64(rM, (valid && level < 2) ? tok * (D / 2) + cl * 8 : kSkip, 0, 0);
         t.l[u] = __builtin_amdgcn_raw_buffer_load_b64(rL, (valid && level == 0) ? tok * (D / 2) + cl * 8 : kSkip, 0, 0);
+#endif
         t.cm[u] = level == 2 ? 0x88888888u : 0u;
         t.cl[u] = level == 1 ? 0x88888888u : 0u;
     }
@@ -212,8 +222,12 @@ __device__ __forceinline__ void v_compute_half(float *acc, const VHalfTile<HV> &
 #pragma unroll
     for (int u = 0; u < HV; ++u) {
         const float sf = half_bits_to_float(sb[u]);
+#if defined(AKV_V_VARIANT) && AKV_V_VARIANT >= 3
+        acc[0] += __uint_as_float((t.h[u].x ^ t.h[u].y ^ t.h[u].z ^ t.h[u].w) & 0x3fffffffu) * sf;
+#else
         fma8(acc, t.h[u].x, t.h[u].y, t.m[u].x | t.cm[u], t.l[u].x | t.cl[u], sf);
         fma8(acc + 8, t.h[u].z, t.h[u].w, t.m[u].y | t.cm[u], t.l[u].y | t.cl[u], sf);
+#endif
     }
 }
 
@@ -277,8 +291,44 @@ __device__ __forceinline__ void v_accumulate(VFirstTile<D> &ft, const uint8_t *f
     }
 }
 
+// Tokens [t_begin, t_end) in groups of two batches (128 tokens, 64 for head_dim 256): any range length.
+template <int D, bool REF>
+__device__ __forceinline__ void v_accumulate_range(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_tokens,
+                                                   const unsigned short *s_row, unsigned char amin, int t_begin,
+                                                   int t_end, float *acc, uint8_t *levels_row) {
+    constexpr int GT = 2 * (D == 256 ? 32 : 64);
+    for (int g = t_begin; g < t_end; g += GT) {
+        VFirstTile<D> ft;
+        v_prefetch_first<D>(ft, f8, n_tokens, g, t_end);
+        v_accumulate<D, REF, 2>(ft, f8, m4, l4, n_tokens, s_row, amin, g, min(g + GT, t_end), acc, levels_row);
+    }
+}
+
 // Folds the token lanes of a wave together and adds the 4 waves of the workgroup:
 // out[d] (d < D) = sum over all 256 lanes of their acc for channel d.  wave_part: LDS [4][D].
+template <int D, int NW = 4>
+__device__ __forceinline__ void v_fold_lanes(float *acc, float (*wave_part)[D]) {
+    // leaves wave_part[wave][d] = this wave's sum for channel d (caller synchronises)
+    constexpr int LPR = D / 16;
+    constexpr int NV = LPR == 16 ? 4 : (LPR == 8 ? 2 : 1);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int ch = (lane % LPR) * 16;
+    reduce_scatter_step<16>(acc, 32);
+    ch += (lane & 32) ? 8 : 0;
+    reduce_scatter_step<8>(acc, 16);
+    ch += (lane & 16) ? 4 : 0;
+    if constexpr (LPR <= 8) {
+        reduce_scatter_step<4>(acc, 8);
+        ch += (lane & 8) ? 2 : 0;
+    }
+    if constexpr (LPR <= 4) {
+        reduce_scatter_step<2>(acc, 4);
+        ch += (lane & 4) ? 1 : 0;
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) wave_part[wave][ch + i] = acc[i];
+}
+
 template <int D>
 __device__ __forceinline__ void v_fold_workgroup(float *acc, float (*wave_part)[D], float *out) {
     constexpr int LPR = D / 16;

@@ -103,7 +103,7 @@ struct MiddleArgs {
     int persist;  // this kernel appends the token (no flush happened in this step)
 };
 
-template <int D>
+template <int D, int NT>
 __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh);
 
 // ------------------------------------------------------------------------------------------------
@@ -164,18 +164,29 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     __syncthreads();
     if (threadIdx.x == 0) is_last = arrive_and_test_last(done_k + bh, epoch, gridDim.x) ? 1 : 0;
     __syncthreads();
-    if (is_last) middle_body<D>(ma, bh);
+    if (is_last) middle_body<D, 256>(ma, bh);
 }
 
 // ------------------------------------------------------------------------------------------------
 // middle.  grid (B*H), 256 threads.
 // ------------------------------------------------------------------------------------------------
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
+// global store of the wave (here: 8 KiB of probabilities on their way to memory), which nobody inside the
+// middle stage reads back; the stage ends with a full barrier.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <int NW>
 __device__ __forceinline__ float block_reduce(float v, bool is_max, float *red) {
     v = is_max ? wave_max(v) : wave_sum(v);
-    __syncthreads();
+    lds_barrier();
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    return is_max ? fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])) : ((red[0] + red[1]) + (red[2] + red[3]));
+    lds_barrier();
+    float r = red[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) r = is_max ? fmaxf(r, red[w]) : r + red[w];
+    return r;
 }
 
 // Decodes 8 fp16 scores (one 16-byte vector) into floats, adding the fp16 mask in fp16 if there is one.
@@ -194,17 +205,18 @@ __device__ __forceinline__ void decode_scores8(const u32x4 w, const unsigned sho
     }
 }
 
-template <int D>
+// NT threads (a multiple of 256) of one workgroup run the stage for one (batch, head).
+template <int D, int NT>
 __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     constexpr int VPT = 4;                    // 16-byte score vectors a thread keeps in registers
-    __shared__ float red[4];
+    constexpr int NW = NT / 64;               // waves
+    __shared__ float red[NW];
     __shared__ unsigned short tail_s[64];     // fp16 scores of the tail (mask not yet added)
     __shared__ float tail_p[64];              // probabilities of the tail
-    __shared__ float cand_v[64][33];
-    __shared__ int cand_t[64][33];
+    __shared__ u32 cand_key[NW][32];
     __shared__ float probe_p[32];
     __shared__ int probe_t[32];
-    __shared__ u32 red_min[4];
+    __shared__ u32 red_min[NW];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int b = bh / a.H, h = bh - b * a.H;
     const int R = a.R, nrest = a.nrest, newest = nrest - 1;
@@ -215,7 +227,14 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     unsigned short *prow = a.probs + (int64_t)bh * a.row_stride;
     const unsigned short *mrow = a.mask ? a.mask + (int64_t)b * a.mask_stride : nullptr;
     const int nvec = R >> 3;
-    const bool in_regs = nvec <= 256 * VPT;
+    const bool in_regs = nvec <= NT * VPT;
+#ifdef AKV_DEBUG_TS
+    unsigned long long *mts = reinterpret_cast<unsigned long long *>(a.toe) + 2 * 1024 * 1024 / 8 + (int64_t)bh * 16;
+#define AKV_MTS(i) if (threadIdx.x == 0) mts[i] = wall_clock64();
+#else
+#define AKV_MTS(i)
+#endif
+    AKV_MTS(0)
     // scores of the flushed part are read at device scope: other workgroups of the same launch wrote them
     const __amdgpu_buffer_rsrc_t rScores = make_rsrc(srow, (u32)R * 2);
 
@@ -225,14 +244,14 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     if (in_regs) {
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
-            const int i = tid + 256 * v;
+            const int i = tid + NT * v;
             sv[v] = load_b128_device(rScores, i < nvec ? i * 16 : kSkip);
         }
     }
     // (a) append the token: rest buffers and column maxima (extension/k_cache_file.py:98-101).
     //     vcm_mine: this thread's channel of the V column maxima after the update (threads < D).
     u32 vcm_mine = 0;
-    for (int d = tid; d < D; d += 256) {
+    for (int d = tid; d < D; d += NT) {
         u32 kc = a.kcm[(int64_t)bh * D + d], vc = a.vcm[(int64_t)bh * D + d];
         if (a.persist) {
             const u32 kb = knew[d], vb = vnew[d];
@@ -249,7 +268,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     // (b) scores of the tail: fp16(fp16(q.k) / sqrt(D)), the two roundings of an fp16 matmul followed by
     //     an fp16 division (extension/k_cache_file.py:156)
     const float sqrt_d = sqrtf((float)D);
-    for (int r = wave; r < nrest; r += 4) {
+    for (int r = wave; r < nrest; r += NW) {
         const unsigned short *krow = (r == newest && a.persist) ? knew : a.restk + (((int64_t)b * a.cb + r) * a.H + h) * D;
         float part = 0.f;
         for (int c = lane; c < D; c += 64) part = fmaf(half_bits_to_float(krow[c]), half_bits_to_float(qrow[c]), part);
@@ -261,7 +280,8 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
             srow[R + r] = sc;
         }
     }
-    __syncthreads();
+    lds_barrier();
+    AKV_MTS(1)
 
     // (c) softmax over [0, R + nrest): scores + mask in fp16, softmax in fp32, probabilities in fp16
     //     (model/KVCache_AlignedKV.py:119-121), and the running arg-max of the residue classes mod 32:
@@ -271,30 +291,31 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
         if (mrow == nullptr) return half_bits_to_float(sbits);
         return half_bits_to_float(float_to_half_bits(half_bits_to_float(sbits) + half_bits_to_float(mrow[t])));
     };
-    float best_v[8];
-    int best_t[8];
+    // arg-max key of a token: probability bits (fp16 of a non-negative number: ordered like an integer)
+    // in the high half, 0xFFFF - (token / 32) in the low half: the largest key is the largest probability
+    // and, among equals, the smallest token (first maximal index, as torch.max returns it)
+    u32 best[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        best_v[j] = -1.f;
-        best_t[j] = 0x7fffffff;
-    }
+    for (int j = 0; j < 8; ++j) best[j] = 0u;
     const float xt = tid < nrest ? masked1(tail_s[tid], R + tid) : -INFINITY;
     float m = xt, sum = 0.f;
     if (in_regs) {
         float x[VPT][8];
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
-            const int i = tid + 256 * v;
+            const int i = tid + NT * v;
             if (i < nvec) {
                 decode_scores8(sv[v], mrow, i * 8, x[v]);
 #pragma unroll
                 for (int j = 0; j < 8; ++j) m = fmaxf(m, x[v][j]);
             }
         }
-        m = block_reduce(m, true, red);
+        AKV_MTS(2)
+        m = block_reduce<NW>(m, true, red);
+        AKV_MTS(3)
 #pragma unroll
         for (int v = 0; v < VPT; ++v)
-            if (tid + 256 * v < nvec) {
+            if (tid + NT * v < nvec) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     x[v][j] = expf(x[v][j] - m);
@@ -302,19 +323,20 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
                 }
             }
         const float et = tid < nrest ? expf(xt - m) : 0.f;
-        sum = block_reduce(sum + et, false, red);
+        sum = block_reduce<NW>(sum + et, false, red);
+        AKV_MTS(4)
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
-            const int i = tid + 256 * v;
+            const int i = tid + NT * v;
             if (i < nvec) {
                 u32 out[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const u32 p0 = float_to_half_bits(x[v][2 * j] / sum), p1 = float_to_half_bits(x[v][2 * j + 1] / sum);
                     out[j] = p0 | (p1 << 16);
-                    const float f0 = half_bits_to_float(p0), f1 = half_bits_to_float(p1);
-                    if (f0 > best_v[2 * j]) { best_v[2 * j] = f0; best_t[2 * j] = i * 8 + 2 * j; }
-                    if (f1 > best_v[2 * j + 1]) { best_v[2 * j + 1] = f1; best_t[2 * j + 1] = i * 8 + 2 * j + 1; }
+                    const u32 grp = 0xffffu - (u32)(i >> 2);     // token / 32 = vector index / 4
+                    best[2 * j] = max(best[2 * j], (p0 << 16) | grp);
+                    best[2 * j + 1] = max(best[2 * j + 1], (p1 << 16) | grp);
                 }
                 const u32x4 o = {out[0], out[1], out[2], out[3]};
                 *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
@@ -328,29 +350,29 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     } else {
         // long rows: three passes over the scores (they stay in the L2 of this workgroup's XCD)
         float x[8];
-        for (int i = tid; i < nvec; i += 256) {
+        for (int i = tid; i < nvec; i += NT) {
             decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
 #pragma unroll
             for (int j = 0; j < 8; ++j) m = fmaxf(m, x[j]);
         }
-        m = block_reduce(m, true, red);
-        for (int i = tid; i < nvec; i += 256) {
+        m = block_reduce<NW>(m, true, red);
+        for (int i = tid; i < nvec; i += NT) {
             decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
 #pragma unroll
             for (int j = 0; j < 8; ++j) sum += expf(x[j] - m);
         }
         const float et = tid < nrest ? expf(xt - m) : 0.f;
-        sum = block_reduce(sum + et, false, red);
-        for (int i = tid; i < nvec; i += 256) {
+        sum = block_reduce<NW>(sum + et, false, red);
+        for (int i = tid; i < nvec; i += NT) {
             decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
             u32 out[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const u32 p0 = float_to_half_bits(expf(x[2 * j] - m) / sum), p1 = float_to_half_bits(expf(x[2 * j + 1] - m) / sum);
                 out[j] = p0 | (p1 << 16);
-                const float f0 = half_bits_to_float(p0), f1 = half_bits_to_float(p1);
-                if (f0 > best_v[2 * j]) { best_v[2 * j] = f0; best_t[2 * j] = i * 8 + 2 * j; }
-                if (f1 > best_v[2 * j + 1]) { best_v[2 * j + 1] = f1; best_t[2 * j + 1] = i * 8 + 2 * j + 1; }
+                const u32 grp = 0xffffu - (u32)(i >> 2);
+                best[2 * j] = max(best[2 * j], (p0 << 16) | grp);
+                best[2 * j + 1] = max(best[2 * j + 1], (p1 << 16) | grp);
             }
             const u32x4 o = {out[0], out[1], out[2], out[3]};
             *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
@@ -362,47 +384,37 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
         }
     }
 
+    AKV_MTS(5)
     // (d)+(e) probe over the flushed part (extension/v_cache_file.py:119-143) and the alignment threshold
     //     of this (batch, head) (extension/v_cache_file.py:156-160)
     if (R > 0) {
-        // thread tid saw residues 8*(tid&3)+j; 64 threads share each residue
+        // thread tid saw residues 8*(tid&3)+j.  Lanes of a wave that share (tid&3): two row rotations (DPP)
+        // inside a 16-lane row, two shuffles across rows; then one LDS row per wave and a last scan.
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            cand_v[tid >> 2][8 * (tid & 3) + j] = best_v[j];
-            cand_t[tid >> 2][8 * (tid & 3) + j] = best_t[j];
+            best[j] = max(best[j], (u32)__builtin_amdgcn_update_dpp(0, (int)best[j], 0x124, 0xf, 0xf, false));   // row_ror:4
+            best[j] = max(best[j], (u32)__builtin_amdgcn_update_dpp(0, (int)best[j], 0x128, 0xf, 0xf, false));   // row_ror:8
+            best[j] = max(best[j], (u32)__shfl_xor((int)best[j], 16, 64));
+            best[j] = max(best[j], (u32)__shfl_xor((int)best[j], 32, 64));
         }
-        __syncthreads();
-        {
-            // 8 threads per residue scan 8 candidates each, then fold; ties go to the smallest token
-            const int res = tid & 31, part = tid >> 5;
-            float bv = -1.f;
-            int bt = 0x7fffffff;
+        AKV_MTS(8)
+        if (lane < 4) {
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const float v = cand_v[part * 8 + k][res];
-                const int t = cand_t[part * 8 + k][res];
-                if (v > bv || (v == bv && t < bt)) { bv = v; bt = t; }
-            }
-            __syncthreads();
-            cand_v[part][res] = bv;
-            cand_t[part][res] = bt;
+            for (int j = 0; j < 8; ++j) cand_key[wave][8 * lane + j] = best[j];
         }
-        __syncthreads();
+        lds_barrier();
+        AKV_MTS(9)
         if (tid < 32) {
-            float bv = -1.f;
-            int bt = 0x7fffffff;
+            u32 key = 0u;
 #pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const float v = cand_v[k][tid];
-                const int t = cand_t[k][tid];
-                if (v > bv || (v == bv && t < bt)) { bv = v; bt = t; }
-            }
-            probe_p[tid] = bv;
-            probe_t[tid] = bt;
+            for (int k = 0; k < NW; ++k) key = max(key, cand_key[k][tid]);
+            probe_p[tid] = half_bits_to_float(key >> 16);
+            probe_t[tid] = (int)(0xffffu - (key & 0xffffu)) * 32 + tid;
         }
-        __syncthreads();
+        lds_barrier();
+        AKV_MTS(6)
         u32 align = 0xffu;
-        for (int d = tid; d < D; d += 256) {
+        for (int d = tid; d < D; d += NT) {
             // the 32 gathered bytes first, then the sum: 32 independent loads in flight instead of a chain
             u32 hi[32];
 #pragma unroll
@@ -419,13 +431,19 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
 #pragma unroll
         for (int mk = 32; mk >= 1; mk >>= 1) align = min(align, (u32)__shfl_xor((int)align, mk, 64));
         if (lane == 0) red_min[wave] = align;
-        __syncthreads();
-        if (tid == 0) a.amin[bh] = (uint8_t)min(min(red_min[0], red_min[1]), min(red_min[2], red_min[3]));
+        lds_barrier();
+        if (tid == 0) {
+            u32 mn = red_min[0];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) mn = min(mn, red_min[w]);
+            a.amin[bh] = (uint8_t)mn;
+        }
     } else {
-        __syncthreads();
+        lds_barrier();
     }
+    AKV_MTS(7)
     // (f) the tail's share of the output, an fp16 matmul result (extension/v_cache_file.py:189)
-    for (int d = tid; d < D; d += 256) {
+    for (int d = tid; d < D; d += NT) {
         float acc = 0.f;
         for (int r = 0; r < nrest; ++r) {
             const unsigned short *vrow = (r == newest && a.persist) ? vnew : a.restv + (((int64_t)b * a.cb + r) * a.H + h) * D;
@@ -438,7 +456,109 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
 // grid (B*H), 256 threads: the middle stage on its own (no flushed block yet, or fusion switched off).
 template <int D>
 __global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
-    middle_body<D>(a, blockIdx.x);
+    middle_body<D, 256>(a, blockIdx.x);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Whole step in one launch: one workgroup of 16 waves per (batch, head) runs the K pass, the middle
+// stage and the V pass back to back.  Used when there are about as many (batch, head) pairs as compute
+// units: nothing is exchanged between workgroups (no partial sums, no second and third launch with
+// their ramp-up and drain), scores and probabilities never leave the compute unit's caches.
+// grid (B*H), 1024 threads.
+// ------------------------------------------------------------------------------------------------
+template <int D, bool REF>
+__global__ __launch_bounds__(1024) void mono_step_kernel(
+    const uint8_t *__restrict__ k_first_8, const uint8_t *__restrict__ k_mid_4, const uint8_t *__restrict__ k_last_4,
+    const uint8_t *__restrict__ v_first_8, const uint8_t *__restrict__ v_mid_4, const uint8_t *__restrict__ v_last_4,
+    MiddleArgs ma, unsigned short *__restrict__ out, uint8_t *__restrict__ k_levels_out,
+    uint8_t *__restrict__ v_levels_out, uint8_t *__restrict__ amin_out, int n_blocks, int n_max_blocks, float scale) {
+    constexpr int CB = 64;
+    constexpr int NG = D / 16;
+    constexpr int NT = 1024, NW = NT / 64;
+    __shared__ float wave_part[NW][D];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int bh = blockIdx.x;
+    const int H = ma.H;
+#ifdef AKV_DEBUG_TS
+    unsigned long long *ts = reinterpret_cast<unsigned long long *>(ma.toe) + 1024 * 1024 / 8 + (int64_t)bh * 8;
+    if (threadIdx.x == 0) ts[0] = wall_clock64();
+#endif
+    // ---- K pass: wave w scores blocks [w*bpw, (w+1)*bpw)
+    {
+        const int bpw = (n_blocks + NW - 1) / NW;
+        const int first_blk = wave * bpw;
+        const int end_blk = min(first_blk + bpw, n_blocks);
+        const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
+        KHalfTile<D / 32> ta;
+        k_prefetch_first<D>(ta, k_first_8 + plane_off * 2, n_blocks, first_blk);
+        float qf[NG];
+        u32 esum[NG];
+        u32 mx = 0;
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            const int c = g * 16 + (lane >> 2);
+            const u32 qb = ma.q[(int64_t)bh * D + c];
+            qf[g] = half_bits_to_float(qb);
+            const u32 cm = max((u32)ma.kcm[(int64_t)bh * D + c], exp_field(ma.k_new[(int64_t)bh * D + c]));
+            esum[g] = (exp_field(qb) + cm) & 0xffu;
+            mx = max(mx, esum[g]);
+        }
+#pragma unroll
+        for (int m = 4; m <= 32; m <<= 1) mx = max(mx, (u32)__shfl_xor((int)mx, m, 64));
+        u32 need_mid = 0, need_last = 0;
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)esum[g]);
+            need_mid |= (lv < 2 ? 1u : 0u) << g;
+            need_last |= (lv == 0 ? 1u : 0u) << g;
+            if (k_levels_out != nullptr && wave == 0 && (lane & 3) == 0)
+                k_levels_out[(int64_t)bh * D + g * 16 + (lane >> 2)] = (uint8_t)lv;
+        }
+        k_score_blocks<D>(ta, k_first_8 + plane_off * 2, k_mid_4 + plane_off, k_last_4 + plane_off, n_blocks, first_blk,
+                          end_blk, qf, need_mid, need_last, ma.scores + (int64_t)bh * ma.row_stride, scale);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+#ifdef AKV_DEBUG_TS
+    if (threadIdx.x == 0) ts[1] = wall_clock64();
+#endif
+    // ---- middle: append, tail scores, softmax, probe, threshold, tail output
+    middle_body<D, NT>(ma, bh);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+#ifdef AKV_DEBUG_TS
+    if (threadIdx.x == 0) ts[2] = wall_clock64();
+#endif
+    // ---- V pass: wave w accumulates tokens [w*tpw, (w+1)*tpw)
+    const int R = ma.R;
+    const unsigned char amin = REF ? 0 : ma.amin[bh];
+    if (!REF && amin_out != nullptr && threadIdx.x == 0) amin_out[bh] = amin;
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    {
+        constexpr int GT = 2 * (D == 256 ? 32 : 64);
+        const int tpw = ((R + NW - 1) / NW + GT - 1) / GT * GT;
+        const int t_begin = wave * tpw;
+        const int t_end = min(t_begin + tpw, R);
+        const int64_t row0 = (int64_t)bh * ma.max_seq_len;
+        v_accumulate_range<D, REF>(v_first_8 + row0 * D, v_mid_4 + row0 * (D / 2), v_last_4 + row0 * (D / 2), R,
+                                   ma.probs + (int64_t)bh * ma.row_stride, amin, t_begin, t_end, acc,
+                                   v_levels_out != nullptr ? v_levels_out + (int64_t)bh * R : nullptr);
+    }
+    v_fold_lanes<D, NW>(acc, wave_part);
+    __syncthreads();
+#ifdef AKV_DEBUG_TS
+    if (threadIdx.x == 0) { ts[3] = wall_clock64(); ts[4] = __smid(); }
+#endif
+    for (int d = threadIdx.x; d < D; d += NT) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += wave_part[w][d];
+        const float o16 = half_bits_to_float(float_to_half_bits(sum));
+        out[(int64_t)bh * D + d] = float_to_half_bits(o16 + half_bits_to_float(ma.otail[(int64_t)bh * D + d]));
+    }
+    (void)H;
 }
 
 // Threshold indexing of the reference expression as written (extension/v_cache_file.py:157-160): entry b*H+h
@@ -590,6 +710,25 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     mark(0, st);
     // the kernel multiplies by the fp16-rounded scale (extension/csrc/K_cache.cu:306)
     const float scale = __half2float(__float2half_rn(1.0f / sqrtf((float)D)));
+    // One launch for the whole step when the (batch, head) pairs alone fill the machine (MI355X: 256 compute
+    // units) and every wave of a 16-wave workgroup gets at least one block; AKV_TUNE_MONO=0/1 overrides.
+    bool mono = (int64_t)B * H >= 192 && n_blocks >= 16 && !(literal_broadcast && !ref);
+    if (const char *e = getenv("AKV_TUNE_MONO")) mono = atoi(e) != 0 && n_blocks >= 1 && !(literal_broadcast && !ref);
+    if (mono) {
+        if (ref)
+            hipLaunchKernelGGL((mono_step_kernel<D, true>), dim3(B * H), dim3(1024), 0, st, kf8, km4, kl4, vf8, vm4, vl4,
+                               ma, reinterpret_cast<unsigned short *>(out), k_levels_out, v_levels_out, amin_out,
+                               n_blocks, n_max_blocks, scale);
+        else
+            hipLaunchKernelGGL((mono_step_kernel<D, false>), dim3(B * H), dim3(1024), 0, st, kf8, km4, kl4, vf8, vm4, vl4,
+                               ma, reinterpret_cast<unsigned short *>(out), k_levels_out, v_levels_out, amin_out,
+                               n_blocks, n_max_blocks, scale);
+        mark(1, st);
+        mark(2, st);
+        mark(3, st);
+        mark(4, st);
+        return check_launch("decode_step(mono)");
+    }
     bool middle_done = false;
     if (n_blocks > 0) {
         const int bpw = k_blocks_per_wave(B, H, n_blocks);
@@ -709,6 +848,8 @@ extern "C" int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_
                     rest_start + rest_len == cur_len,
                 "decode_step: inconsistent state cur_len=%d rest_start=%d rest_len=%d", cur_len, rest_start, rest_len);
     AKV_REQUIRE(cur_len + 1 <= max_seq_len, "decode_step: cache full (%d of %d tokens)", cur_len, max_seq_len);
+    AKV_REQUIRE(rest_start + d_block <= 65536 * 32, "decode_step: at most %d flushed tokens (16-bit group index of the probe)",
+                65536 * 32);
     AKV_REQUIRE((int64_t)n_max_blocks * d_block >= rest_start + (rest_len + 1 == d_block ? d_block : 0),
                 "decode_step: K planes hold %d blocks, %d tokens flushed", n_max_blocks, rest_start);
     AKV_REQUIRE(row_stride % 8 == 0 && row_stride >= rest_start + d_block,
