@@ -92,7 +92,7 @@ template <int D>
 __device__ __forceinline__ void k_score_blocks(KHalfTile<D / 32> &ta, const uint8_t *f8, const uint8_t *m4,
                                                const uint8_t *l4, int n_blocks, int first_blk, int end_blk,
                                                const float *qf, u32 need_mid, u32 need_last, unsigned short *s_row,
-                                               float scale) {
+                                               float scale, int blk_stride = 1) {
     constexpr int CB = 64;
     constexpr int NG = D / 16;
     constexpr int HG = NG / 2;
@@ -109,7 +109,7 @@ __device__ __forceinline__ void k_score_blocks(KHalfTile<D / 32> &ta, const uint
     KHalfTile<HG> tb;
     k_issue_half_ml<D, HG>(ta, rM, rL, first_blk, 0, need_mid, need_last);   // its high bytes: k_prefetch_first
     __builtin_amdgcn_sched_barrier(0);
-    for (int blk = first_blk; blk < end_blk; ++blk) {
+    for (int blk = first_blk; blk < end_blk; blk += blk_stride) {
         float acc[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.f;
@@ -118,7 +118,7 @@ __device__ __forceinline__ void k_score_blocks(KHalfTile<D / 32> &ta, const uint
         k_compute_half<HG>(acc, ta, 0, qf, need_mid, need_last);
         __builtin_amdgcn_sched_barrier(0);
         // past the last block the offsets fall outside the buffer resources: the loads return 0 and fetch nothing
-        k_issue_half<D, HG>(ta, rH, rM, rL, blk + 1 < end_blk ? blk + 1 : n_blocks, 0, need_mid, need_last);
+        k_issue_half<D, HG>(ta, rH, rM, rL, blk + blk_stride < end_blk ? blk + blk_stride : n_blocks, 0, need_mid, need_last);
         __builtin_amdgcn_sched_barrier(0);
         k_compute_half<HG>(acc, tb, HG, qf, need_mid, need_last);
         __builtin_amdgcn_sched_barrier(0);
@@ -295,9 +295,9 @@ __device__ __forceinline__ void v_accumulate(VFirstTile<D> &ft, const uint8_t *f
 template <int D, bool REF>
 __device__ __forceinline__ void v_accumulate_range(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_tokens,
                                                    const unsigned short *s_row, unsigned char amin, int t_begin,
-                                                   int t_end, float *acc, uint8_t *levels_row) {
+                                                   int t_end, float *acc, uint8_t *levels_row, int group_stride = 1) {
     constexpr int GT = 2 * (D == 256 ? 32 : 64);
-    for (int g = t_begin; g < t_end; g += GT) {
+    for (int g = t_begin; g < t_end; g += GT * group_stride) {
         VFirstTile<D> ft;
         v_prefetch_first<D>(ft, f8, n_tokens, g, t_end);
         v_accumulate<D, REF, 2>(ft, f8, m4, l4, n_tokens, s_row, amin, g, min(g + GT, t_end), acc, levels_row);

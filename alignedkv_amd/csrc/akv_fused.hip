@@ -16,8 +16,6 @@
 // run first, exactly as the reference flushes before it computes.
 #include "akv_cores.h"
 
-#include <atomic>
-
 namespace akv {
 
 // defined in akv_k.hip / akv_v.hip
@@ -34,33 +32,8 @@ __device__ __forceinline__ u32 exp_field(u32 half_bits) { return (half_bits >> 1
 static bool g_profile = false;
 static hipEvent_t g_ev[5];
 static bool g_ev_ready = false;
-// epochs of the arrival counters: process-wide, never 0
-static std::atomic<unsigned long long> g_epoch_source{1};
-static inline unsigned long long next_epoch() {
-    unsigned long long e = g_epoch_source.fetch_add(1) & 0xffffffffffffull;
-    return e ? e : (g_epoch_source.fetch_add(1) & 0xffffffffffffull);
-}
 static inline void mark(int i, hipStream_t st) {
     if (g_profile) (void)hipEventRecord(g_ev[i], st);
-}
-
-// Arrival counter that needs no initialisation: a 64-bit word holds (epoch << 16 | arrivals).  Every call of
-// the step uses a fresh epoch (process-wide counter on the host), so whatever an earlier call or an
-// uninitialised workspace left in the word reads as "no arrival yet".  Returns true for the last of
-// `expected` arrivals.  Call with one thread per workgroup, after a __threadfence() + __syncthreads().
-__device__ __forceinline__ bool arrive_and_test_last(unsigned long long *word, unsigned long long epoch, u32 expected) {
-    unsigned long long seen = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    while (true) {
-        const unsigned long long count = (seen >> 16) == epoch ? (seen & 0xffffull) : 0ull;
-        const unsigned long long want = (epoch << 16) | (count + 1);
-        if (__hip_atomic_compare_exchange_strong(word, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
-                                                 __HIP_MEMORY_SCOPE_AGENT)) {
-            if (count + 1 != expected) return false;
-            // leave the word empty: a captured graph replays the step with the epoch it was recorded with
-            __hip_atomic_store(word, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            return true;
-        }
-    }
 }
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -114,8 +87,7 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
     unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, int n_blocks, int n_max_blocks, int H,
-    int row_stride, int blocks_per_wave, float scale, MiddleArgs ma, unsigned long long *done_k,
-    unsigned long long epoch) {
+    int row_stride, int blocks_per_wave, float scale) {
     constexpr int CB = 64;
     constexpr int NG = D / 16;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -153,18 +125,6 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     }
     k_score_blocks<D>(ta, first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
                       need_mid, need_last, scores + (int64_t)bh * row_stride, scale);
-    if (done_k == nullptr) return;
-    // The workgroup that finishes the last chunk of this (batch, head) runs the middle stage for it, while
-    // other workgroups are still streaming their blocks: no separate launch, no idle machine in between.
-    // The scores were stored at device scope; the workgroup-scope fence + barrier below waits until every
-    // wave's stores have completed before one thread reports the arrival, and the middle stage reads the
-    // scores at device scope: no device-wide fence (a whole-L2 write back and invalidate) is needed.
-    __shared__ int is_last;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
-    if (threadIdx.x == 0) is_last = arrive_and_test_last(done_k + bh, epoch, gridDim.x) ? 1 : 0;
-    __syncthreads();
-    if (is_last) middle_body<D, 256>(ma, bh);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -485,9 +445,9 @@ __global__ __launch_bounds__(1024) void mono_step_kernel(
 #endif
     // ---- K pass: wave w scores blocks [w*bpw, (w+1)*bpw)
     {
-        const int bpw = (n_blocks + NW - 1) / NW;
-        const int first_blk = wave * bpw;
-        const int end_blk = min(first_blk + bpw, n_blocks);
+        // wave w takes blocks w, w + 16, ...: at any time the 16 waves stream 16 neighbouring blocks
+        const int first_blk = wave;
+        const int end_blk = n_blocks;
         const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
         KHalfTile<D / 32> ta;
         k_prefetch_first<D>(ta, k_first_8 + plane_off * 2, n_blocks, first_blk);
@@ -515,7 +475,7 @@ __global__ __launch_bounds__(1024) void mono_step_kernel(
                 k_levels_out[(int64_t)bh * D + g * 16 + (lane >> 2)] = (uint8_t)lv;
         }
         k_score_blocks<D>(ta, k_first_8 + plane_off * 2, k_mid_4 + plane_off, k_last_4 + plane_off, n_blocks, first_blk,
-                          end_blk, qf, need_mid, need_last, ma.scores + (int64_t)bh * ma.row_stride, scale);
+                          end_blk, qf, need_mid, need_last, ma.scores + (int64_t)bh * ma.row_stride, scale, NW);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
@@ -537,14 +497,12 @@ __global__ __launch_bounds__(1024) void mono_step_kernel(
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
     {
+        // wave w takes the token groups w, w + 16, ... (128 tokens each): neighbouring waves, neighbouring rows
         constexpr int GT = 2 * (D == 256 ? 32 : 64);
-        const int tpw = ((R + NW - 1) / NW + GT - 1) / GT * GT;
-        const int t_begin = wave * tpw;
-        const int t_end = min(t_begin + tpw, R);
         const int64_t row0 = (int64_t)bh * ma.max_seq_len;
         v_accumulate_range<D, REF>(v_first_8 + row0 * D, v_mid_4 + row0 * (D / 2), v_last_4 + row0 * (D / 2), R,
-                                   ma.probs + (int64_t)bh * ma.row_stride, amin, t_begin, t_end, acc,
-                                   v_levels_out != nullptr ? v_levels_out + (int64_t)bh * R : nullptr);
+                                   ma.probs + (int64_t)bh * ma.row_stride, amin, wave * GT, R, acc,
+                                   v_levels_out != nullptr ? v_levels_out + (int64_t)bh * R : nullptr, NW);
     }
     v_fold_lanes<D, NW>(acc, wave_part);
     __syncthreads();
@@ -583,8 +541,7 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const unsigned short *__restrict__ probs, const uint8_t *__restrict__ amin_u8, float *__restrict__ partial,
     uint8_t *__restrict__ levels_out, uint8_t *__restrict__ amin_out, int H, int max_seq_len, int row_stride,
-    int n_tokens, int tokens_per_wave, int n_chunks, const unsigned short *__restrict__ otail,
-    unsigned short *__restrict__ out, unsigned long long *done_v, unsigned long long epoch) {
+    int n_tokens, int tokens_per_wave, int n_chunks) {
     __shared__ float wave_part[4][D];
     const int wave = threadIdx.x >> 6;
     const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
@@ -603,23 +560,6 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
                               probs + (int64_t)bh * row_stride, amin, t_begin, t_end, acc,
                               levels_out != nullptr ? levels_out + (int64_t)bh * n_tokens : nullptr);
     v_fold_workgroup<D>(acc, wave_part, partial + ((int64_t)bh * n_chunks + chunk) * D);
-    if (done_v == nullptr) return;
-    // The workgroup that delivers the last chunk of this (batch, head) adds the partials up (in chunk order:
-    // the output bits do not depend on which workgroup comes last) and writes the output.
-    __shared__ int is_last;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // partial sums were stored at device scope
-    __syncthreads();
-    if (threadIdx.x == 0) is_last = arrive_and_test_last(done_v + bh, epoch, (u32)n_chunks) ? 1 : 0;
-    __syncthreads();
-    if (is_last) {
-        const __amdgpu_buffer_rsrc_t rP = make_rsrc(partial + (int64_t)bh * n_chunks * D, (u32)n_chunks * D * 4);
-        for (int d = threadIdx.x; d < D; d += 256) {
-            float sum = 0.f;
-            for (int c = 0; c < n_chunks; ++c) sum += load_f32_device(rP, (c * D + d) * 4);
-            const float o16 = half_bits_to_float(float_to_half_bits(sum));
-            out[(int64_t)bh * D + d] = float_to_half_bits(o16 + half_bits_to_float(otail[(int64_t)bh * D + d]));
-        }
-    }
 }
 
 // grid (B*H), D threads: out = fp16(fp16(sum of partials) + tail), the fp16 `o += tail` of the reference.
@@ -635,7 +575,7 @@ __global__ void fused_combine_kernel(const float *__restrict__ partial, const un
 }
 
 struct StepLayout {
-    size_t done_k, done_v, toe, amin, otail, partial, total;
+    size_t toe, amin, otail, partial, total;
 };
 
 static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
@@ -645,10 +585,8 @@ static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
     // the plan for fewer tokens never has more chunks than the plan for max_seq_len has at its finest split
     size_t max_chunks = (size_t)(max_seq_len + 4 * (D == 256 ? 32 : 64) - 1) / (4 * (D == 256 ? 32 : 64));
     (void)p;
-    l.done_k = 0;
-    l.done_v = up((size_t)B * H * 8);
-    l.toe = l.done_v + up((size_t)B * H * 8);
-    l.amin = l.toe + up((size_t)B * H * D);
+    l.toe = 0;
+    l.amin = up((size_t)B * H * D);
     l.otail = l.amin + up((size_t)B * H);
     l.partial = l.otail + up((size_t)B * H * D * 2);
     l.total = l.partial + up((size_t)B * H * max_chunks * D * sizeof(float));
@@ -665,15 +603,6 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     const StepLayout lay = step_layout(B, H, D, max_seq_len);
     uint8_t *toe = ws + lay.toe;
     uint8_t *amin = ws + lay.amin;
-    // Optional fusion of the middle stage into the K pass and of the combine stage into the V pass ("last
-    // workgroup of a (batch, head) does the next stage").  Measured slower than separate launches on MI355X
-    // (every workgroup has to wait for its device-scope stores and the arrival atomic before it can retire),
-    // so it is off unless AKV_TUNE_TAIL_FUSION=1.
-    static const bool no_fusion = getenv("AKV_TUNE_TAIL_FUSION") == nullptr;
-    const unsigned long long epoch = next_epoch();
-    const bool fuse_middle = !no_fusion && !(literal_broadcast && !ref);   // the literal threshold needs every probe first
-    unsigned long long *done_k = fuse_middle ? reinterpret_cast<unsigned long long *>(ws + lay.done_k) : nullptr;
-    unsigned long long *done_v = !no_fusion ? reinterpret_cast<unsigned long long *>(ws + lay.done_v) : nullptr;
     unsigned short *otail = reinterpret_cast<unsigned short *>(ws + lay.otail);
     float *partial = reinterpret_cast<float *>(ws + lay.partial);
     const unsigned short *q16 = reinterpret_cast<const unsigned short *>(q);
@@ -729,27 +658,22 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         mark(4, st);
         return check_launch("decode_step(mono)");
     }
-    bool middle_done = false;
     if (n_blocks > 0) {
         const int bpw = k_blocks_per_wave(B, H, n_blocks);
         dim3 grid((n_blocks + 4 * bpw - 1) / (4 * bpw), H, B);
         if (ref)
             hipLaunchKernelGGL((fused_k_pass_kernel<D, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                               k_levels_out, n_blocks, n_max_blocks, H, row_stride, bpw, scale, ma, done_k, epoch);
+                               k_levels_out, n_blocks, n_max_blocks, H, row_stride, bpw, scale);
         else
             hipLaunchKernelGGL((fused_k_pass_kernel<D, false>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                               k_levels_out, n_blocks, n_max_blocks, H, row_stride, bpw, scale, ma, done_k, epoch);
+                               k_levels_out, n_blocks, n_max_blocks, H, row_stride, bpw, scale);
         int rc = check_launch("decode_step(k_pass)");
         if (rc != AKV_OK) return rc;
-        middle_done = done_k != nullptr;
     }
     mark(1, st);
-    int rc = AKV_OK;
-    if (!middle_done) {
-        hipLaunchKernelGGL((fused_middle_kernel<D>), dim3(B * H), dim3(256), 0, st, ma);
-        rc = check_launch("decode_step(middle)");
-        if (rc != AKV_OK) return rc;
-    }
+    hipLaunchKernelGGL((fused_middle_kernel<D>), dim3(B * H), dim3(256), 0, st, ma);
+    int rc = check_launch("decode_step(middle)");
+    if (rc != AKV_OK) return rc;
     if (literal_broadcast && !ref && R > 0) {
         hipLaunchKernelGGL(fused_amin_literal_kernel, dim3(B * H), dim3(64), 0, st, toe, vcm, amin, H, D);
         rc = check_launch("decode_step(amin)");
@@ -761,8 +685,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         dim3 grid(p.n_chunks, H, B);
 #define AKV_VP(R, N)                                                                                                  \
     hipLaunchKernelGGL((fused_v_pass_kernel<D, R, N>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, amin, partial, \
-                       v_levels_out, amin_out, H, max_seq_len, row_stride, R_tokens, p.tokens_per_wave, p.n_chunks,   \
-                       otail, reinterpret_cast<unsigned short *>(out), done_v, epoch)
+                       v_levels_out, amin_out, H, max_seq_len, row_stride, R_tokens, p.tokens_per_wave, p.n_chunks)
         const int R_tokens = R;
         if (ref) {
             if (p.iters_per_wave == 1) AKV_VP(true, 1);
@@ -778,14 +701,11 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
     }
     mark(3, st);
-    if (p.n_chunks == 0 || done_v == nullptr) {
-        hipLaunchKernelGGL(fused_combine_kernel, dim3(B * H), dim3(D < 256 ? D : 256), 0, st, partial, otail,
-                           reinterpret_cast<unsigned short *>(out), D, p.n_chunks);
-        rc = check_launch("decode_step(combine)");
-    }
+    hipLaunchKernelGGL(fused_combine_kernel, dim3(B * H), dim3(D < 256 ? D : 256), 0, st, partial, otail,
+                       reinterpret_cast<unsigned short *>(out), D, p.n_chunks);
     mark(4, st);
     (void)cur_len;
-    return rc;
+    return check_launch("decode_step(combine)");
 }
 
 }  // namespace akv

@@ -198,3 +198,36 @@ def test_fused_step_rejects_bad_state():
     with pytest.raises(RuntimeError, match="cache full"):
         m.decode_step(*args(128, 128, 0))
     m.decode_step(*args(5, 0, 5))
+
+
+@pytest.mark.parametrize("reference", [False, True])
+def test_one_launch_step_matches_the_four_launch_step(monkeypatch, reference):
+    """AKV_TUNE_MONO=1 runs the whole step as one kernel (one 16-wave workgroup per (batch, head)); it must
+    agree with the four-launch step: identical fetch levels and threshold, outputs within 1e-3."""
+    from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
+    B, H, D, prefill, steps = 2, 8, 128, 1100, 70
+    q, k, v = make_qkv(B, prefill + steps, H, D, seed=123)
+    rng = np.random.default_rng(8)
+    caches = []
+    for _ in range(2):
+        c = QuantizedCache_AlignedKV(cfg(H, D), B, prefill + steps + 64, "cuda", torch.half)
+        c.reference = reference
+        c.key_cache[0].save(dev(k[:, :prefill]), 0, prefill)
+        c.value_cache[0].save(dev(v[:, :prefill]), 0, prefill)
+        c.key_cache[0].record_levels = c.value_cache[0].record_levels = True
+        caches.append(c)
+    for t in range(prefill, prefill + steps):
+        qt = dev(rng.standard_normal((B, 1, H, D)).astype(np.float16))
+        monkeypatch.setenv("AKV_TUNE_MONO", "0")
+        o4 = caches[0].auto_compute(qt, dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None)
+        monkeypatch.setenv("AKV_TUNE_MONO", "1")
+        o1 = caches[1].auto_compute(qt, dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None)
+        assert (o4.float() - o1.float()).abs().max().item() <= 1e-3
+        for name in ("last_levels",):
+            assert torch.equal(caches[0].key_cache[0].last_levels, caches[1].key_cache[0].last_levels)
+            assert torch.equal(caches[0].value_cache[0].last_levels, caches[1].value_cache[0].last_levels)
+        if not reference:
+            assert torch.equal(caches[0].value_cache[0].last_alignment_min, caches[1].value_cache[0].last_alignment_min)
+    k0, k1 = caches[0].key_cache[0], caches[1].key_cache[0]
+    assert torch.equal(k0.k_cache_first_8, k1.k_cache_first_8) and torch.equal(k0.k_cache_last_4, k1.k_cache_last_4)
+    assert k0.reststartpos == k1.reststartpos == (prefill + steps) // 64 * 64
