@@ -36,3 +36,32 @@ def assert_close_fp16(got, want, abs_floor):
     err = np.abs(g - w)
     bad = err > spacing + abs_floor
     assert not bad.any(), f"max err {err.max():.3e} (allowed {float((spacing + abs_floor)[err.argmax()]):.3e}) at {int(bad.sum())} entries"
+
+
+def oracle_decode_step_c(k_planes, v_planes, k_colmax, v_colmax, q, k_new, v_new, R, d_block=64, top_k=32,
+                         reference=False):
+    """One decode step (cache of R flushed tokens, empty rest buffer, one appended token) with the C
+    restatement of the ops + the NumPy host logic.  All arguments are NumPy arrays in the reference layouts.
+    Returns (out [B,1,H,D] float16, k_levels, v_levels, amin, probs)."""
+    import math
+    from oracle import akv_oracle as O
+    from oracle import akv_oracle_c as OC
+    B, _, H, D = q.shape
+    nb = R // d_block
+    kcm2 = O.colmax_update(k_colmax, k_new)
+    vcm2 = O.colmax_update(v_colmax, v_new)
+    ksum, kmax = O.k_sum_and_max(q, kcm2)
+    s, klv = OC.k_cache_compute(*k_planes, ksum, kmax, O.as_bits(q), nb, d_block, 1.0 / math.sqrt(D), reference)
+    s = s.copy()
+    restk = np.zeros((B, d_block, H, D), np.float16)
+    restv = np.zeros((B, d_block, H, D), np.float16)
+    restk[:, :1], restv[:, :1] = k_new, v_new
+    s[:, :, :, R:R + 1] = O.rest_scores(q, restk, 1, D)
+    s[:, :, :, R + 1:] = -np.inf
+    p = O.softmax_fp32_to_half(s)
+    tv, ti = O.bucket_max(p[..., :R], R + 1, top_k)
+    to = OC.v_cache_test_compute(v_planes[0], O.as_bits(tv), ti, top_k)
+    amin = O.alignment_min(O.test_o_exponent(to), vcm2)
+    o, vlv = OC.v_cache_compute(*v_planes, O.as_bits(np.ascontiguousarray(p)), amin, R, reference)
+    o = (o + O.rest_output(p[..., R:R + 1], restv, 1)).astype(np.float16)
+    return o.reshape(B, 1, H, D), klv, vlv, amin, p

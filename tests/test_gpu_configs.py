@@ -1,0 +1,94 @@
+"""The benchmark configurations at their real shapes on the GPU (fused decode step), checked against the
+C restatement of the ops run on the same planes, plus size-independent properties:
+  C1  batch 1, 32 heads x 128, cache 1024, K with 4 outlier channels per head x10
+  C2  batch 8, 32 heads x 128, cache 4096 (+ one appended token)
+  C4  batch 4, 32 heads x 128, cache 32768, K scaled per token by a log-normal factor
+Inputs are generated on the GPU with a seeded generator and copied to the host for the oracle."""
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import akv_oracle as O
+from tests.common import oracle_decode_step_c
+
+pytestmark = pytest.mark.gpu
+
+
+def build(B, H, D, L, k_kind, seed):
+    from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
+    cfg = SimpleNamespace(num_hidden_layers=1, num_attention_heads=H, num_key_value_heads=H, hidden_size=H * D,
+                          max_position_embeddings=L + 64)
+    cache = QuantizedCache_AlignedKV(cfg, B, L + 64, "cuda", torch.half)
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    k = torch.randn((B, L, H, D), device="cuda", generator=g)
+    if k_kind == "outlier":
+        for h in range(H):
+            ch = torch.randperm(D, generator=torch.Generator().manual_seed(1000 + h))[:4].cuda()
+            k[:, :, h, ch] *= 10.0
+    else:
+        k *= torch.exp(torch.randn((B, L, 1, 1), device="cuda", generator=g))
+    k = k.half()
+    v = (0.5 * torch.randn((B, L, H, D), device="cuda", generator=g)).half()
+    cache.key_cache[0].save(k, 0, L)
+    cache.value_cache[0].save(v, 0, L)
+    q = torch.randn((B, 1, H, D), device="cuda", generator=g).half()
+    kn = torch.randn((B, 1, H, D), device="cuda", generator=g).half()
+    vn = (0.5 * torch.randn((B, 1, H, D), device="cuda", generator=g)).half()
+    return cache, k, v, q, kn, vn
+
+
+@pytest.mark.parametrize("name,B,H,D,L,k_kind", [("C1", 1, 32, 128, 1024, "outlier"), ("C2", 8, 32, 128, 4096, "outlier"),
+                                                 ("C4", 4, 32, 128, 32768, "lognormal")])
+def test_config_step_against_c_oracle(name, B, H, D, L, k_kind):
+    cache, k, v, q, kn, vn = build(B, H, D, L, k_kind, seed=17)
+    kc, vc = cache.key_cache[0], cache.value_cache[0]
+    # round trip of the plane format: planes written by the HIP save kernels reconstruct the fp16 input exactly
+    sample = slice(0, L, max(1, L // 256))
+    hi, mid, last = O.v_planes_fields(vc.v_cache_first_8[:, :, sample].cpu().numpy(), vc.v_cache_mid_4[:, :, sample].cpu().numpy(),
+                                      vc.v_cache_last_4[:, :, sample].cpu().numpy(), len(range(L)[sample]))
+    assert np.array_equal(O.reconstruct(hi, mid, last, 0), v[:, sample].transpose(1, 2).cpu().numpy().view(np.uint16))
+    host = dict(k_planes=[t.cpu().numpy() for t in (kc.k_cache_first_8, kc.k_cache_mid_4, kc.k_cache_last_4)],
+                v_planes=[t.cpu().numpy() for t in (vc.v_cache_first_8, vc.v_cache_mid_4, vc.v_cache_last_4)],
+                k_colmax=kc.k_cache_exp_column_max.cpu().numpy(), v_colmax=vc.v_cache_exp_column_max.cpu().numpy())
+    kc.record_levels = vc.record_levels = True
+    out = cache.auto_compute(q, kn, vn, 0, None)
+    want, klv, vlv, amin, p = oracle_decode_step_c(host["k_planes"], host["v_planes"], host["k_colmax"], host["v_colmax"],
+                                                   q.cpu().numpy(), kn.cpu().numpy(), vn.cpu().numpy(), L)
+    assert np.array_equal(kc.last_levels.cpu().numpy(), klv), "K fetch levels differ"
+    got_p = cache._probs[:, :, :L + 1].cpu().numpy()
+    assert np.max(np.abs(got_p.astype(np.float32) - p[:, :, 0, :L + 1].astype(np.float32))) <= 2e-3
+    # V levels: bit exact for the probabilities and threshold the kernels produced; against the oracle's own
+    # probabilities a level can only differ where a probability sits on a rounding boundary
+    got_amin = vc.last_alignment_min.cpu().numpy()
+    got_vlv = vc.last_levels.cpu().numpy()
+    assert np.array_equal(got_vlv, O.v_levels(got_amin, O.as_bits(np.ascontiguousarray(got_p[:, :, :L]))))
+    assert np.array_equal(got_amin, amin)
+    assert (got_vlv != vlv).mean() <= 1e-3
+    err = np.max(np.abs(out.cpu().numpy().astype(np.float32) - want.astype(np.float32)))
+    assert err <= 1e-3, f"{name}: max abs err {err}"
+    # the algorithm has to move fewer bytes than dense fp16 on these distributions
+    moved = L * ((klv < 3).sum() + 0.5 * (klv < 2).sum() + 0.5 * (klv == 0).sum()) \
+        + D * ((vlv < 3).sum() + 0.5 * (vlv < 2).sum() + 0.5 * (vlv == 0).sum())
+    assert moved <= 0.8 * (2 * B * H * L * D * 2), f"{name}: {moved / (2 * B * H * L * D * 2):.3f} of dense"
+
+
+def test_config2_reference_mode_equals_dense_fp32_attention():
+    B, H, D, L = 8, 32, 128, 4096
+    cache, k, v, q, kn, vn = build(B, H, D, L, "outlier", seed=23)
+    cache.reference = True
+    out = cache.auto_compute(q, kn, vn, 0, None)
+    kk = torch.cat([k, kn], 1).float().permute(0, 2, 1, 3)      # [B,H,L+1,D]
+    vv = torch.cat([v, vn], 1).float().permute(0, 2, 1, 3)
+    w = torch.softmax((q.float().permute(0, 2, 1, 3) @ kk.transpose(2, 3)) / D ** 0.5, -1)
+    want = (w @ vv).permute(0, 2, 1, 3)
+    # fp16 scores with an fp16-rounded scale in the plane path: a few 1e-3 on outlier keys
+    assert (out.float() - want).abs().max().item() <= 5e-3
+    # determinism: the same step on the same state gives the same bits
+    kc, vc = cache.key_cache[0], cache.value_cache[0]
+    for c in (kc, vc):
+        c.current_cache_len -= 1
+        c._restlen -= 1
+    out2 = cache.auto_compute(q, kn, vn, 0, None)
+    assert torch.equal(out, out2)
