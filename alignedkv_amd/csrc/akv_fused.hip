@@ -47,6 +47,40 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Shape and per-sequence state of one step.  Query head hq reads the planes of KV head hq / G (grouped-query
+// attention; G == 1 is the reference's multi-head case).  seq_lens (device, may be null) holds the tokens
+// cached before this step per sequence; without it every sequence has cur_len tokens.
+struct StepGeom {
+    int Hq, Hkv, G;
+    int cb, max_seq_len, n_max_blocks, row_stride;
+    int cur_len;
+    const int *seq_lens;
+};
+
+// tokens flushed into the planes / held in the rest buffer once this step's token has been appended
+__device__ __forceinline__ void seq_state(const StepGeom &g, int b, int &R, int &nrest) {
+    const int L = (g.seq_lens != nullptr ? g.seq_lens[b] : g.cur_len) + 1;
+    R = (L / g.cb) * g.cb;
+    nrest = L - R;
+}
+
+// Workgroup -> (chunk, query head of the group).  Workgroups go to the 8 XCDs round-robin by linear index,
+// and each XCD has its own L2: the G workgroups that stream the same plane chunk for the G query heads of a
+// KV head get linear indices 8 apart, i.e. the same XCD at about the same time, so the chunk comes from HBM
+// once and from that L2 G-1 times.  gridDim.x = 8 * ceil(chunks / 8) * G.
+__device__ __forceinline__ void decode_group_block(int G, int &chunk, int &gq) {
+    const int lin = blockIdx.x;
+    if (G == 1) {
+        chunk = lin;
+        gq = 0;
+    } else {
+        const int t = lin >> 3;
+        gq = t % G;
+        chunk = (t / G) * 8 + (lin & 7);
+    }
+}
+static inline int group_grid_x(int chunks, int G) { return G == 1 ? chunks : ((chunks + 7) / 8) * 8 * G; }
+
 // ------------------------------------------------------------------------------------------------
 // persist (flush steps only): token -> rest buffers, column maxima.  grid (B*H), D threads.
 // ------------------------------------------------------------------------------------------------
@@ -64,16 +98,91 @@ __global__ void fused_persist_kernel(const unsigned short *__restrict__ k_new, c
     }
 }
 
+// Ragged mode, first kernel of every step: append the token of every sequence to its rest buffer, update the
+// column maxima and, for the sequences whose rest buffer is full with it, write the 64-token block into the
+// planes (same bytes as k_save_blocks_kernel / v_save_vec8_kernel).  grid (B*Hkv), 256 threads.
+template <int D>
+__global__ __launch_bounds__(256) void fused_pre_kernel(uint8_t *__restrict__ kf8, uint8_t *__restrict__ km4,
+                                                        uint8_t *__restrict__ kl4, uint8_t *__restrict__ vf8,
+                                                        uint8_t *__restrict__ vm4, uint8_t *__restrict__ vl4,
+                                                        const unsigned short *__restrict__ k_new,
+                                                        const unsigned short *__restrict__ v_new,
+                                                        unsigned short *__restrict__ restk, unsigned short *__restrict__ restv,
+                                                        uint8_t *__restrict__ kcm, uint8_t *__restrict__ vcm, StepGeom geo) {
+    constexpr int CB = 64;
+    __shared__ unsigned short tile[CB][D + 2];
+    const int bh = blockIdx.x, b = bh / geo.Hkv, h = bh - b * geo.Hkv;
+    const int cur = geo.seq_lens[b];
+    const int slot = cur % CB;
+    for (int d = threadIdx.x; d < D; d += 256) {
+        const u32 kb = k_new[(int64_t)bh * D + d], vb = v_new[(int64_t)bh * D + d];
+        const int64_t at = (((int64_t)b * CB + slot) * geo.Hkv + h) * D + d;
+        restk[at] = (unsigned short)kb;
+        restv[at] = (unsigned short)vb;
+        kcm[(int64_t)bh * D + d] = (uint8_t)max((u32)kcm[(int64_t)bh * D + d], exp_field(kb));
+        vcm[(int64_t)bh * D + d] = (uint8_t)max((u32)vcm[(int64_t)bh * D + d], exp_field(vb));
+    }
+    if (slot != CB - 1) return;
+    __syncthreads();                          // the token written above is part of the block
+    const int blk = cur / CB;
+    // V rows: 8 channels per thread and token
+    for (int idx = threadIdx.x; idx < CB * (D / 8); idx += 256) {
+        const int j = idx / (D / 8), d8 = idx - j * (D / 8);
+        const u32x4 w = *reinterpret_cast<const u32x4 *>(restv + (((int64_t)b * CB + j) * geo.Hkv + h) * D + d8 * 8);
+        const u32 ww[4] = {w.x, w.y, w.z, w.w};
+        u32 hi0 = 0, hi1 = 0, mid = 0, last = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const u32 e = ww[i] & 0xffffu, o = ww[i] >> 16;
+            const u32 hp = (e >> 8) | ((o >> 8) << 8);
+            if (i < 2) hi0 |= hp << (16 * i); else hi1 |= hp << (16 * (i - 2));
+            mid |= ((e & 0xf0u) | ((o & 0xf0u) >> 4)) << (8 * i);
+            last |= (((e & 0x0fu) << 4) | (o & 0x0fu)) << (8 * i);
+        }
+        const int64_t row = (int64_t)bh * geo.max_seq_len + (int64_t)blk * CB + j;
+        const u32x2 hv = {hi0, hi1};
+        *reinterpret_cast<u32x2 *>(vf8 + row * D + d8 * 8) = hv;
+        *reinterpret_cast<u32 *>(vm4 + row * (D / 2) + d8 * 4) = mid;
+        *reinterpret_cast<u32 *>(vl4 + row * (D / 2) + d8 * 4) = last;
+    }
+    // K block: transpose through LDS
+    for (int idx = threadIdx.x; idx < CB * (D / 2); idx += 256) {
+        const int j = idx / (D / 2), dp = idx - j * (D / 2);
+        const u32 w = *reinterpret_cast<const u32 *>(restk + (((int64_t)b * CB + j) * geo.Hkv + h) * D + dp * 2);
+        tile[j][2 * dp] = (unsigned short)(w & 0xffffu);
+        tile[j][2 * dp + 1] = (unsigned short)(w >> 16);
+    }
+    __syncthreads();
+    const int64_t base = ((int64_t)bh * geo.n_max_blocks + blk) * (int64_t)D * (CB / 2);
+    for (int idx = threadIdx.x; idx < D * (CB / 4); idx += 256) {
+        const int d = idx / (CB / 4), j = (idx - d * (CB / 4)) * 4;
+        const u32 w = (u32)(tile[j][d] >> 8) | ((u32)(tile[j + 1][d] >> 8) << 8) | ((u32)(tile[j + 2][d] >> 8) << 16) |
+                      ((u32)(tile[j + 3][d] >> 8) << 24);
+        *reinterpret_cast<u32 *>(kf8 + base * 2 + (int64_t)d * CB + j) = w;
+    }
+    for (int idx = threadIdx.x; idx < D * (CB / 8); idx += 256) {
+        const int d = idx / (CB / 8), j = (idx - d * (CB / 8)) * 8;
+        u32 mw = 0, lw = 0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const u32 le = tile[j + 2 * i][d] & 0xffu, lo = tile[j + 2 * i + 1][d] & 0xffu;
+            mw |= ((le & 0xf0u) | (lo >> 4)) << (8 * i);
+            lw |= (((le & 0x0fu) << 4) | (lo & 0x0fu)) << (8 * i);
+        }
+        *reinterpret_cast<u32 *>(km4 + base + (int64_t)d * (CB / 2) + (j >> 1)) = mw;
+        *reinterpret_cast<u32 *>(kl4 + base + (int64_t)d * (CB / 2) + (j >> 1)) = lw;
+    }
+}
+
 struct MiddleArgs {
     const unsigned short *q, *k_new, *v_new, *mask;
     unsigned short *restk, *restv, *scores, *probs, *otail;
     uint8_t *kcm, *vcm, *toe, *amin;
     const uint8_t *v_first_8;
-    int H, cb, max_seq_len, row_stride, mask_stride;
-    int R;        // flushed tokens (multiple of cb)
-    int nrest;    // tokens in the rest buffer including the one of this step (0 on a flush step)
+    StepGeom g;
+    int mask_stride;
     int top_k;
-    int persist;  // this kernel appends the token (no flush happened in this step)
+    int persist;  // this kernel appends the token (it is not in the rest buffers / planes yet)
 };
 
 template <int D, int NT>
@@ -86,17 +195,22 @@ template <int D, bool REF>
 __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
-    unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, int n_blocks, int n_max_blocks, int H,
-    int row_stride, int blocks_per_wave, float scale) {
+    unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, StepGeom geo, int blocks_per_wave,
+    float scale) {
     constexpr int CB = 64;
     constexpr int NG = D / 16;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int h = blockIdx.y, b = blockIdx.z;
-    const int bh = b * H + h;
-    const int first_blk = (blockIdx.x * 4 + wave) * blocks_per_wave;   // may lie past the end: the wave then idles
+    int chunk, gq;
+    decode_group_block(geo.G, chunk, gq);
+    const int hkv = blockIdx.y, b = blockIdx.z;
+    const int bh_kv = b * geo.Hkv + hkv, bh = b * geo.Hq + hkv * geo.G + gq;
+    int R, nrest;
+    seq_state(geo, b, R, nrest);
+    const int n_blocks = R / CB;
+    const int first_blk = (chunk * 4 + wave) * blocks_per_wave;   // may lie past the end: the wave then idles
     const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
 
-    const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
+    const int64_t plane_off = (int64_t)bh_kv * geo.n_max_blocks * (D * (CB / 2));
     KHalfTile<D / 32> ta;
     k_prefetch_first<D>(ta, first_8 + plane_off * 2, n_blocks, first_blk);
     float qf[NG];
@@ -108,7 +222,7 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
         const u32 qb = q[(int64_t)bh * D + c];
         qf[g] = half_bits_to_float(qb);
         // column max including the token appended by this step
-        const u32 cm = max((u32)kcm[(int64_t)bh * D + c], exp_field(k_new[(int64_t)bh * D + c]));
+        const u32 cm = max((u32)kcm[(int64_t)bh_kv * D + c], exp_field(k_new[(int64_t)bh_kv * D + c]));
         esum[g] = (exp_field(qb) + cm) & 0xffu;
         mx = max(mx, esum[g]);
     }
@@ -120,11 +234,11 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
         const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)esum[g]);
         need_mid |= (lv < 2 ? 1u : 0u) << g;
         need_last |= (lv == 0 ? 1u : 0u) << g;
-        if (levels_out != nullptr && blockIdx.x == 0 && wave == 0 && (lane & 3) == 0)
+        if (levels_out != nullptr && chunk == 0 && wave == 0 && (lane & 3) == 0)
             levels_out[(int64_t)bh * D + g * 16 + (lane >> 2)] = (uint8_t)lv;
     }
     k_score_blocks<D>(ta, first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
-                      need_mid, need_last, scores + (int64_t)bh * row_stride, scale);
+                      need_mid, need_last, scores + (int64_t)bh * geo.row_stride, scale);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -178,13 +292,19 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     __shared__ int probe_t[32];
     __shared__ u32 red_min[NW];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int b = bh / a.H, h = bh - b * a.H;
-    const int R = a.R, nrest = a.nrest, newest = nrest - 1;
+    // bh indexes (batch, query head); the keys, values, column maxima and rest buffers belong to its KV head
+    const int b = bh / a.g.Hq, hq = bh - b * a.g.Hq, h = hq / a.g.G;
+    const int bh_kv = b * a.g.Hkv + h;
+    const int Hkv = a.g.Hkv, cb = a.g.cb;
+    const bool owner = hq % a.g.G == 0;       // one query head of the group writes the shared state
+    int R, nrest;
+    seq_state(a.g, b, R, nrest);
+    const int newest = nrest - 1;
     const unsigned short *qrow = a.q + (int64_t)bh * D;
-    const unsigned short *knew = a.k_new + (int64_t)bh * D;
-    const unsigned short *vnew = a.v_new + (int64_t)bh * D;
-    unsigned short *srow = a.scores + (int64_t)bh * a.row_stride;
-    unsigned short *prow = a.probs + (int64_t)bh * a.row_stride;
+    const unsigned short *knew = a.k_new + (int64_t)bh_kv * D;
+    const unsigned short *vnew = a.v_new + (int64_t)bh_kv * D;
+    unsigned short *srow = a.scores + (int64_t)bh * a.g.row_stride;
+    unsigned short *prow = a.probs + (int64_t)bh * a.g.row_stride;
     const unsigned short *mrow = a.mask ? a.mask + (int64_t)b * a.mask_stride : nullptr;
     const int nvec = R >> 3;
     const bool in_regs = nvec <= NT * VPT;
@@ -212,16 +332,20 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     //     vcm_mine: this thread's channel of the V column maxima after the update (threads < D).
     u32 vcm_mine = 0;
     for (int d = tid; d < D; d += NT) {
-        u32 kc = a.kcm[(int64_t)bh * D + d], vc = a.vcm[(int64_t)bh * D + d];
+        u32 kc = a.kcm[(int64_t)bh_kv * D + d], vc = a.vcm[(int64_t)bh_kv * D + d];
         if (a.persist) {
+            // every query head of the group derives the updated maxima itself (max is idempotent, so it does
+            // not matter whether it reads them before or after the owner's store); only the owner stores
             const u32 kb = knew[d], vb = vnew[d];
-            const int64_t at = (((int64_t)b * a.cb + newest) * a.H + h) * D + d;
-            a.restk[at] = (unsigned short)kb;
-            a.restv[at] = (unsigned short)vb;
             kc = max(kc, exp_field(kb));
             vc = max(vc, exp_field(vb));
-            a.kcm[(int64_t)bh * D + d] = (uint8_t)kc;
-            a.vcm[(int64_t)bh * D + d] = (uint8_t)vc;
+            if (owner) {
+                const int64_t at = (((int64_t)b * cb + newest) * Hkv + h) * D + d;
+                a.restk[at] = (unsigned short)kb;
+                a.restv[at] = (unsigned short)vb;
+                a.kcm[(int64_t)bh_kv * D + d] = (uint8_t)kc;
+                a.vcm[(int64_t)bh_kv * D + d] = (uint8_t)vc;
+            }
         }
         vcm_mine = vc;
     }
@@ -229,7 +353,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     //     an fp16 division (extension/k_cache_file.py:156)
     const float sqrt_d = sqrtf((float)D);
     for (int r = wave; r < nrest; r += NW) {
-        const unsigned short *krow = (r == newest && a.persist) ? knew : a.restk + (((int64_t)b * a.cb + r) * a.H + h) * D;
+        const unsigned short *krow = (r == newest && a.persist) ? knew : a.restk + (((int64_t)b * cb + r) * Hkv + h) * D;
         float part = 0.f;
         for (int c = lane; c < D; c += 64) part = fmaf(half_bits_to_float(krow[c]), half_bits_to_float(qrow[c]), part);
         part = wave_sum(part);
@@ -378,7 +502,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
             // the 32 gathered bytes first, then the sum: 32 independent loads in flight instead of a chain
             u32 hi[32];
 #pragma unroll
-            for (int i = 0; i < 32; ++i) hi[i] = a.v_first_8[((int64_t)bh * a.max_seq_len + probe_t[i]) * D + d];
+            for (int i = 0; i < 32; ++i) hi[i] = a.v_first_8[((int64_t)bh_kv * a.g.max_seq_len + probe_t[i]) * D + d];
             float acc = 0.f;
 #pragma unroll
             for (int i = 0; i < 32; ++i)
@@ -406,7 +530,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     for (int d = tid; d < D; d += NT) {
         float acc = 0.f;
         for (int r = 0; r < nrest; ++r) {
-            const unsigned short *vrow = (r == newest && a.persist) ? vnew : a.restv + (((int64_t)b * a.cb + r) * a.H + h) * D;
+            const unsigned short *vrow = (r == newest && a.persist) ? vnew : a.restv + (((int64_t)b * cb + r) * Hkv + h) * D;
             acc = fmaf(half_bits_to_float(vrow[d]), tail_p[r], acc);
         }
         a.otail[(int64_t)bh * D + d] = float_to_half_bits(acc);
@@ -438,7 +562,6 @@ __global__ __launch_bounds__(1024) void mono_step_kernel(
     __shared__ float wave_part[NW][D];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int bh = blockIdx.x;
-    const int H = ma.H;
 #ifdef AKV_DEBUG_TS
     unsigned long long *ts = reinterpret_cast<unsigned long long *>(ma.toe) + 1024 * 1024 / 8 + (int64_t)bh * 8;
     if (threadIdx.x == 0) ts[0] = wall_clock64();
@@ -475,7 +598,7 @@ __global__ __launch_bounds__(1024) void mono_step_kernel(
                 k_levels_out[(int64_t)bh * D + g * 16 + (lane >> 2)] = (uint8_t)lv;
         }
         k_score_blocks<D>(ta, k_first_8 + plane_off * 2, k_mid_4 + plane_off, k_last_4 + plane_off, n_blocks, first_blk,
-                          end_blk, qf, need_mid, need_last, ma.scores + (int64_t)bh * ma.row_stride, scale, NW);
+                          end_blk, qf, need_mid, need_last, ma.scores + (int64_t)bh * ma.g.row_stride, scale, NW);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
@@ -490,7 +613,8 @@ __global__ __launch_bounds__(1024) void mono_step_kernel(
     if (threadIdx.x == 0) ts[2] = wall_clock64();
 #endif
     // ---- V pass: wave w accumulates tokens [w*tpw, (w+1)*tpw)
-    const int R = ma.R;
+    int R, nrest_unused;
+    seq_state(ma.g, bh / ma.g.Hq, R, nrest_unused);
     const unsigned char amin = REF ? 0 : ma.amin[bh];
     if (!REF && amin_out != nullptr && threadIdx.x == 0) amin_out[bh] = amin;
     float acc[16];
@@ -499,9 +623,9 @@ __global__ __launch_bounds__(1024) void mono_step_kernel(
     {
         // wave w takes the token groups w, w + 16, ... (128 tokens each): neighbouring waves, neighbouring rows
         constexpr int GT = 2 * (D == 256 ? 32 : 64);
-        const int64_t row0 = (int64_t)bh * ma.max_seq_len;
+        const int64_t row0 = (int64_t)bh * ma.g.max_seq_len;
         v_accumulate_range<D, REF>(v_first_8 + row0 * D, v_mid_4 + row0 * (D / 2), v_last_4 + row0 * (D / 2), R,
-                                   ma.probs + (int64_t)bh * ma.row_stride, amin, wave * GT, R, acc,
+                                   ma.probs + (int64_t)bh * ma.g.row_stride, amin, wave * GT, R, acc,
                                    v_levels_out != nullptr ? v_levels_out + (int64_t)bh * R : nullptr, NW);
     }
     v_fold_lanes<D, NW>(acc, wave_part);
@@ -516,7 +640,6 @@ __global__ __launch_bounds__(1024) void mono_step_kernel(
         const float o16 = half_bits_to_float(float_to_half_bits(sum));
         out[(int64_t)bh * D + d] = float_to_half_bits(o16 + half_bits_to_float(ma.otail[(int64_t)bh * D + d]));
     }
-    (void)H;
 }
 
 // Threshold indexing of the reference expression as written (extension/v_cache_file.py:157-160): entry b*H+h
@@ -540,15 +663,20 @@ template <int D, bool REF, int NIT>
 __global__ __launch_bounds__(256) void fused_v_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const unsigned short *__restrict__ probs, const uint8_t *__restrict__ amin_u8, float *__restrict__ partial,
-    uint8_t *__restrict__ levels_out, uint8_t *__restrict__ amin_out, int H, int max_seq_len, int row_stride,
-    int n_tokens, int tokens_per_wave, int n_chunks) {
+    uint8_t *__restrict__ levels_out, int levels_stride, uint8_t *__restrict__ amin_out, StepGeom geo,
+    int tokens_per_wave, int n_chunks) {
     __shared__ float wave_part[4][D];
     const int wave = threadIdx.x >> 6;
-    const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-    const int bh = b * H + h;
+    int chunk, gq;
+    decode_group_block(geo.G, chunk, gq);
+    const int hkv = blockIdx.y, b = blockIdx.z;
+    const int bh_kv = b * geo.Hkv + hkv, bh = b * geo.Hq + hkv * geo.G + gq;
+    if (chunk >= n_chunks) return;    // padding of the grid (whole workgroup)
+    int n_tokens, nrest;
+    seq_state(geo, b, n_tokens, nrest);
     const int t_begin = (chunk * 4 + wave) * tokens_per_wave;
     const int t_end = min(t_begin + tokens_per_wave, n_tokens);
-    const int64_t row0 = (int64_t)bh * max_seq_len;
+    const int64_t row0 = (int64_t)bh_kv * geo.max_seq_len;
     VFirstTile<D> ft;
     v_prefetch_first<D>(ft, first_8 + row0 * D, n_tokens, t_begin, t_end);
     const unsigned char amin = REF ? 0 : amin_u8[bh];
@@ -557,15 +685,17 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
     v_accumulate<D, REF, NIT>(ft, first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
-                              probs + (int64_t)bh * row_stride, amin, t_begin, t_end, acc,
-                              levels_out != nullptr ? levels_out + (int64_t)bh * n_tokens : nullptr);
+                              probs + (int64_t)bh * geo.row_stride, amin, t_begin, t_end, acc,
+                              levels_out != nullptr ? levels_out + (int64_t)bh * levels_stride : nullptr);
     v_fold_workgroup<D>(acc, wave_part, partial + ((int64_t)bh * n_chunks + chunk) * D);
 }
 
 // grid (B*H), D threads: out = fp16(fp16(sum of partials) + tail), the fp16 `o += tail` of the reference.
 __global__ void fused_combine_kernel(const float *__restrict__ partial, const unsigned short *__restrict__ otail,
-                                     unsigned short *__restrict__ out, int D, int n_chunks) {
+                                     unsigned short *__restrict__ out, int D, int n_chunks, int *seq_lens_rw, int Hq) {
     const int bh = blockIdx.x;
+    // last kernel of the step: the sequence lengths kept on the device advance here
+    if (seq_lens_rw != nullptr && threadIdx.x == 0 && bh % Hq == 0) seq_lens_rw[bh / Hq] += 1;
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
         float acc = 0.f;
         for (int c = 0; c < n_chunks; ++c) acc += partial[((int64_t)bh * n_chunks + c) * D + d];
@@ -598,9 +728,9 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
                     uint8_t *vcm, uint8_t *restk, uint8_t *restv, const uint8_t *q, const uint8_t *k_new,
                     const uint8_t *v_new, const uint8_t *mask, int mask_stride, uint8_t *out, uint8_t *scores,
                     uint8_t *probs, int row_stride, uint8_t *ws, uint8_t *k_levels_out, uint8_t *v_levels_out,
-                    uint8_t *amin_out, int B, int H, int n_max_blocks, int max_seq_len, int cb, int top_k, int cur_len,
-                    int rest_start, int rest_len, bool ref, int literal_broadcast, hipStream_t st) {
-    const StepLayout lay = step_layout(B, H, D, max_seq_len);
+                    uint8_t *amin_out, int B, int Hq, int Hkv, int n_max_blocks, int max_seq_len, int cb, int top_k,
+                    int cur_len, int *seq_lens, bool ref, int literal_broadcast, hipStream_t st) {
+    const StepLayout lay = step_layout(B, Hq, D, max_seq_len);
     uint8_t *toe = ws + lay.toe;
     uint8_t *amin = ws + lay.amin;
     unsigned short *otail = reinterpret_cast<unsigned short *>(ws + lay.otail);
@@ -610,46 +740,61 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     const unsigned short *v16 = reinterpret_cast<const unsigned short *>(v_new);
     unsigned short *s16 = reinterpret_cast<unsigned short *>(scores);
     unsigned short *p16 = reinterpret_cast<unsigned short *>(probs);
+    unsigned short *rk16 = reinterpret_cast<unsigned short *>(restk), *rv16 = reinterpret_cast<unsigned short *>(restv);
+    const bool ragged = seq_lens != nullptr;
 
-    int R = rest_start, nrest = rest_len + 1, persist = 1;
-    if (nrest == cb) {   // the token fills the rest buffer: flush it into the planes before computing
-        hipLaunchKernelGGL(fused_persist_kernel, dim3(B * H), dim3(D < 256 ? D : 256), 0, st, k16, v16,
-                           reinterpret_cast<unsigned short *>(restk), reinterpret_cast<unsigned short *>(restv), kcm,
-                           vcm, H, D, cb, rest_len);
+    StepGeom geo;
+    geo.Hq = Hq; geo.Hkv = Hkv; geo.G = Hq / Hkv;
+    geo.cb = cb; geo.max_seq_len = max_seq_len; geo.n_max_blocks = n_max_blocks; geo.row_stride = row_stride;
+    geo.cur_len = cur_len; geo.seq_lens = seq_lens;
+
+    int persist = 1;
+    if (ragged) {
+        // per-sequence lengths live on the device: one small kernel appends every token and flushes the rest
+        // buffers that fill up with it
+        hipLaunchKernelGGL((fused_pre_kernel<D>), dim3(B * Hkv), dim3(256), 0, st, kf8, km4, kl4, vf8, vm4, vl4, k16, v16,
+                           rk16, rv16, kcm, vcm, geo);
+        int rc = check_launch("decode_step(pre)");
+        if (rc != AKV_OK) return rc;
+        persist = 0;
+    } else if (cur_len % cb + 1 == cb) {
+        // the token fills the rest buffer: flush it into the planes before computing
+        const int rest_start = cur_len / cb * cb;
+        hipLaunchKernelGGL(fused_persist_kernel, dim3(B * Hkv), dim3(D < 256 ? D : 256), 0, st, k16, v16, rk16, rv16, kcm,
+                           vcm, Hkv, D, cb, cur_len % cb);
         int rc = check_launch("decode_step(persist)");
         if (rc != AKV_OK) return rc;
-        rc = launch_k_save_blocks(kf8, km4, kl4, restk, B, H, 1, n_max_blocks, D, cb, rest_start, cb, st);
+        rc = launch_k_save_blocks(kf8, km4, kl4, restk, B, Hkv, 1, n_max_blocks, D, cb, rest_start, cb, st);
         if (rc != AKV_OK) return rc;
-        rc = launch_v_save(vf8, vm4, vl4, restv, B, H, max_seq_len, D, rest_start, cb, cb, st);
+        rc = launch_v_save(vf8, vm4, vl4, restv, B, Hkv, max_seq_len, D, rest_start, cb, cb, st);
         if (rc != AKV_OK) return rc;
-        R = rest_start + cb;
-        nrest = 0;
         persist = 0;
     }
+    // flushed tokens after the append: exact for uniform lengths, an upper bound for ragged ones
+    const int R = (cur_len + 1) / cb * cb;
     const int n_blocks = R / cb;
     MiddleArgs ma;
     ma.q = q16; ma.k_new = k16; ma.v_new = v16;
     ma.mask = reinterpret_cast<const unsigned short *>(mask);
-    ma.restk = reinterpret_cast<unsigned short *>(restk);
-    ma.restv = reinterpret_cast<unsigned short *>(restv);
+    ma.restk = rk16; ma.restv = rv16;
     ma.scores = s16; ma.probs = p16; ma.otail = otail;
     ma.kcm = kcm; ma.vcm = vcm; ma.toe = toe; ma.amin = amin; ma.v_first_8 = vf8;
-    ma.H = H; ma.cb = cb; ma.max_seq_len = max_seq_len; ma.row_stride = row_stride; ma.mask_stride = mask_stride;
-    ma.R = R; ma.nrest = nrest; ma.top_k = top_k; ma.persist = persist;
+    ma.g = geo; ma.mask_stride = mask_stride; ma.top_k = top_k; ma.persist = persist;
     mark(0, st);
     // the kernel multiplies by the fp16-rounded scale (extension/csrc/K_cache.cu:306)
     const float scale = __half2float(__float2half_rn(1.0f / sqrtf((float)D)));
-    // One launch for the whole step when the (batch, head) pairs alone fill the machine (MI355X: 256 compute
-    // units) and every wave of a 16-wave workgroup gets at least one block; AKV_TUNE_MONO=0/1 overrides.
-    bool mono = (int64_t)B * H >= 192 && n_blocks >= 16 && !(literal_broadcast && !ref);
-    if (const char *e = getenv("AKV_TUNE_MONO")) mono = atoi(e) != 0 && n_blocks >= 1 && !(literal_broadcast && !ref);
+    // One launch for the whole step: opt-in (AKV_TUNE_MONO=1), multi-head uniform-length caches only.  It
+    // measures level with the four launches at batch 8 x 32 heads x 4096 tokens on MI355X.
+    bool mono = false;
+    if (const char *e = getenv("AKV_TUNE_MONO")) mono = atoi(e) != 0;
+    mono = mono && n_blocks >= 1 && geo.G == 1 && !ragged && !(literal_broadcast && !ref);
     if (mono) {
         if (ref)
-            hipLaunchKernelGGL((mono_step_kernel<D, true>), dim3(B * H), dim3(1024), 0, st, kf8, km4, kl4, vf8, vm4, vl4,
+            hipLaunchKernelGGL((mono_step_kernel<D, true>), dim3(B * Hq), dim3(1024), 0, st, kf8, km4, kl4, vf8, vm4, vl4,
                                ma, reinterpret_cast<unsigned short *>(out), k_levels_out, v_levels_out, amin_out,
                                n_blocks, n_max_blocks, scale);
         else
-            hipLaunchKernelGGL((mono_step_kernel<D, false>), dim3(B * H), dim3(1024), 0, st, kf8, km4, kl4, vf8, vm4, vl4,
+            hipLaunchKernelGGL((mono_step_kernel<D, false>), dim3(B * Hq), dim3(1024), 0, st, kf8, km4, kl4, vf8, vm4, vl4,
                                ma, reinterpret_cast<unsigned short *>(out), k_levels_out, v_levels_out, amin_out,
                                n_blocks, n_max_blocks, scale);
         mark(1, st);
@@ -659,34 +804,33 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         return check_launch("decode_step(mono)");
     }
     if (n_blocks > 0) {
-        const int bpw = k_blocks_per_wave(B, H, n_blocks);
-        dim3 grid((n_blocks + 4 * bpw - 1) / (4 * bpw), H, B);
+        const int bpw = k_blocks_per_wave(B, Hq, n_blocks);
+        dim3 grid(group_grid_x((n_blocks + 4 * bpw - 1) / (4 * bpw), geo.G), Hkv, B);
         if (ref)
             hipLaunchKernelGGL((fused_k_pass_kernel<D, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                               k_levels_out, n_blocks, n_max_blocks, H, row_stride, bpw, scale);
+                               k_levels_out, geo, bpw, scale);
         else
             hipLaunchKernelGGL((fused_k_pass_kernel<D, false>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                               k_levels_out, n_blocks, n_max_blocks, H, row_stride, bpw, scale);
+                               k_levels_out, geo, bpw, scale);
         int rc = check_launch("decode_step(k_pass)");
         if (rc != AKV_OK) return rc;
     }
     mark(1, st);
-    hipLaunchKernelGGL((fused_middle_kernel<D>), dim3(B * H), dim3(256), 0, st, ma);
+    hipLaunchKernelGGL((fused_middle_kernel<D>), dim3(B * Hq), dim3(256), 0, st, ma);
     int rc = check_launch("decode_step(middle)");
     if (rc != AKV_OK) return rc;
     if (literal_broadcast && !ref && R > 0) {
-        hipLaunchKernelGGL(fused_amin_literal_kernel, dim3(B * H), dim3(64), 0, st, toe, vcm, amin, H, D);
+        hipLaunchKernelGGL(fused_amin_literal_kernel, dim3(B * Hq), dim3(64), 0, st, toe, vcm, amin, Hq, D);
         rc = check_launch("decode_step(amin)");
         if (rc != AKV_OK) return rc;
     }
     mark(2, st);
-    const VPlan p = v_plan(B, H, D, R);
+    const VPlan p = v_plan(B, Hq, D, R);
     if (p.n_chunks > 0) {
-        dim3 grid(p.n_chunks, H, B);
-#define AKV_VP(R, N)                                                                                                  \
-    hipLaunchKernelGGL((fused_v_pass_kernel<D, R, N>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, amin, partial, \
-                       v_levels_out, amin_out, H, max_seq_len, row_stride, R_tokens, p.tokens_per_wave, p.n_chunks)
-        const int R_tokens = R;
+        dim3 grid(group_grid_x(p.n_chunks, geo.G), Hkv, B);
+#define AKV_VP(RF, N)                                                                                                  \
+    hipLaunchKernelGGL((fused_v_pass_kernel<D, RF, N>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, amin, partial,     \
+                       v_levels_out, R, amin_out, geo, p.tokens_per_wave, p.n_chunks)
         if (ref) {
             if (p.iters_per_wave == 1) AKV_VP(true, 1);
             else if (p.iters_per_wave == 2) AKV_VP(true, 2);
@@ -701,10 +845,9 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
     }
     mark(3, st);
-    hipLaunchKernelGGL(fused_combine_kernel, dim3(B * H), dim3(D < 256 ? D : 256), 0, st, partial, otail,
-                       reinterpret_cast<unsigned short *>(out), D, p.n_chunks);
+    hipLaunchKernelGGL(fused_combine_kernel, dim3(B * Hq), dim3(D < 256 ? D : 256), 0, st, partial, otail,
+                       reinterpret_cast<unsigned short *>(out), D, p.n_chunks, seq_lens, Hq);
     mark(4, st);
-    (void)cur_len;
     return check_launch("decode_step(combine)");
 }
 
@@ -741,9 +884,61 @@ extern "C" int akv_profile_read(float *phase_ms) {
     return AKV_OK;
 }
 
-extern "C" size_t akv_decode_step_workspace_bytes(int bsz, int n_kv_heads, int head_dim, int max_seq_len) {
-    if (bsz <= 0 || n_kv_heads <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
-    return step_layout(bsz, n_kv_heads, head_dim, max_seq_len).total;
+extern "C" size_t akv_decode_step_workspace_bytes(int bsz, int n_q_heads, int head_dim, int max_seq_len) {
+    if (bsz <= 0 || n_q_heads <= 0 || head_dim <= 0 || max_seq_len <= 0) return 0;
+    return step_layout(bsz, n_q_heads, head_dim, max_seq_len).total;
+}
+
+extern "C" int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,
+                                   uint8_t *v_mid_4, uint8_t *v_last_4, uint8_t *k_exp_column_max,
+                                   uint8_t *v_exp_column_max, uint8_t *restk, uint8_t *restv, const uint8_t *q,
+                                   const uint8_t *k_new, const uint8_t *v_new, const uint8_t *mask, int mask_stride,
+                                   uint8_t *out, uint8_t *scores, uint8_t *probs, int row_stride, void *workspace,
+                                   size_t workspace_bytes, uint8_t *k_levels_out, uint8_t *v_levels_out,
+                                   uint8_t *amin_out, int bsz, int n_q_heads, int n_kv_heads, int n_max_blocks,
+                                   int max_seq_len, int head_dim, int d_block, int top_max_k, int cur_len,
+                                   int *seq_lens, int reference, int literal_broadcast, akv_stream_t stream) {
+    AKV_REQUIRE(k_first_8 && k_mid_4 && k_last_4 && v_first_8 && v_mid_4 && v_last_4 && k_exp_column_max &&
+                    v_exp_column_max && restk && restv && q && k_new && v_new && out && scores && probs && workspace,
+                "decode_step: null pointer");
+    AKV_REQUIRE(bsz > 0 && n_q_heads > 0 && n_kv_heads > 0 && n_max_blocks > 0 && max_seq_len > 0,
+                "decode_step: non-positive dimension");
+    AKV_REQUIRE(n_q_heads % n_kv_heads == 0, "decode_step: %d query heads are not a multiple of %d KV heads", n_q_heads,
+                n_kv_heads);
+    AKV_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256,
+                "decode_step: head_dim %d not supported by the fused step (64, 128, 256); use the five ops", head_dim);
+    AKV_REQUIRE(d_block == 64, "decode_step: d_block %d not supported by the fused step (64); use the five ops", d_block);
+    AKV_REQUIRE(top_max_k == 32, "decode_step: top_max_k %d not supported by the fused step (32)", top_max_k);
+    AKV_REQUIRE(bsz <= 65535 && n_kv_heads <= 65535, "decode_step: bsz/heads exceed the grid limit 65535");
+    AKV_REQUIRE(cur_len >= 0 && cur_len + 1 <= max_seq_len, "decode_step: cache full (%d of %d tokens)", cur_len, max_seq_len);
+    AKV_REQUIRE(!literal_broadcast || (n_q_heads == n_kv_heads && seq_lens == nullptr),
+                "decode_step: literal_broadcast is defined for multi-head caches of uniform length only");
+    const int flushed = (cur_len + 1) / d_block * d_block;
+    AKV_REQUIRE(flushed + d_block <= 65536 * 32, "decode_step: at most %d flushed tokens (16-bit group index of the probe)",
+                65536 * 32);
+    AKV_REQUIRE((int64_t)n_max_blocks * d_block >= flushed, "decode_step: K planes hold %d blocks, %d tokens flushed",
+                n_max_blocks, flushed);
+    AKV_REQUIRE(row_stride % 8 == 0 && row_stride >= flushed + d_block,
+                "decode_step: row_stride %d must be a multiple of 8 and >= %d", row_stride, flushed + d_block);
+    AKV_REQUIRE(mask == nullptr || mask_stride == 0 || mask_stride >= cur_len + 1,
+                "decode_step: mask row stride %d shorter than %d (0 = one row for all sequences)", mask_stride, cur_len + 1);
+    AKV_REQUIRE((int64_t)max_seq_len * head_dim < (int64_t)1 << 31 && (int64_t)n_max_blocks * head_dim * d_block < (int64_t)1 << 31,
+                "decode_step: one (batch, head) slice of a high-byte plane must stay below 2 GiB");
+    const size_t need = akv_decode_step_workspace_bytes(bsz, n_q_heads, head_dim, max_seq_len);
+    AKV_REQUIRE(workspace_bytes >= need, "decode_step: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+    AKV_REQUIRE(((uintptr_t)workspace & 255) == 0 && ((uintptr_t)scores & 15) == 0 && ((uintptr_t)probs & 15) == 0,
+                "decode_step: workspace must be 256-byte aligned, scores/probs 16-byte aligned");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    uint8_t *ws = static_cast<uint8_t *>(workspace);
+#define AKV_STEP(DD)                                                                                                  \
+    return run_step<DD>(k_first_8, k_mid_4, k_last_4, v_first_8, v_mid_4, v_last_4, k_exp_column_max, v_exp_column_max, \
+                        restk, restv, q, k_new, v_new, mask, mask_stride, out, scores, probs, row_stride, ws,          \
+                        k_levels_out, v_levels_out, amin_out, bsz, n_q_heads, n_kv_heads, n_max_blocks, max_seq_len,   \
+                        d_block, top_max_k, cur_len, seq_lens, reference != 0, literal_broadcast, st);
+    if (head_dim == 64) { AKV_STEP(64) }
+    if (head_dim == 128) { AKV_STEP(128) }
+    AKV_STEP(256)
+#undef AKV_STEP
 }
 
 extern "C" int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,
@@ -755,42 +950,12 @@ extern "C" int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_
                                int bsz, int n_kv_heads, int n_max_blocks, int max_seq_len, int head_dim, int d_block,
                                int top_max_k, int cur_len, int rest_start, int rest_len, int reference,
                                int literal_broadcast, akv_stream_t stream) {
-    AKV_REQUIRE(k_first_8 && k_mid_4 && k_last_4 && v_first_8 && v_mid_4 && v_last_4 && k_exp_column_max &&
-                    v_exp_column_max && restk && restv && q && k_new && v_new && out && scores && probs && workspace,
-                "decode_step: null pointer");
-    AKV_REQUIRE(bsz > 0 && n_kv_heads > 0 && n_max_blocks > 0 && max_seq_len > 0, "decode_step: non-positive dimension");
-    AKV_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256,
-                "decode_step: head_dim %d not supported by the fused step (64, 128, 256); use the five ops", head_dim);
-    AKV_REQUIRE(d_block == 64, "decode_step: d_block %d not supported by the fused step (64); use the five ops", d_block);
-    AKV_REQUIRE(top_max_k == 32, "decode_step: top_max_k %d not supported by the fused step (32)", top_max_k);
-    AKV_REQUIRE(bsz <= 65535 && n_kv_heads <= 65535, "decode_step: bsz/heads exceed the grid limit 65535");
-    AKV_REQUIRE(cur_len >= 0 && rest_start >= 0 && rest_len >= 0 && rest_len < d_block && rest_start % d_block == 0 &&
-                    rest_start + rest_len == cur_len,
+    AKV_REQUIRE(d_block > 0 && cur_len >= 0 && rest_start >= 0 && rest_len >= 0 && rest_len < d_block &&
+                    rest_start % d_block == 0 && rest_start + rest_len == cur_len,
                 "decode_step: inconsistent state cur_len=%d rest_start=%d rest_len=%d", cur_len, rest_start, rest_len);
-    AKV_REQUIRE(cur_len + 1 <= max_seq_len, "decode_step: cache full (%d of %d tokens)", cur_len, max_seq_len);
-    AKV_REQUIRE(rest_start + d_block <= 65536 * 32, "decode_step: at most %d flushed tokens (16-bit group index of the probe)",
-                65536 * 32);
-    AKV_REQUIRE((int64_t)n_max_blocks * d_block >= rest_start + (rest_len + 1 == d_block ? d_block : 0),
-                "decode_step: K planes hold %d blocks, %d tokens flushed", n_max_blocks, rest_start);
-    AKV_REQUIRE(row_stride % 8 == 0 && row_stride >= rest_start + d_block,
-                "decode_step: row_stride %d must be a multiple of 8 and >= %d", row_stride, rest_start + d_block);
-    AKV_REQUIRE(mask == nullptr || mask_stride == 0 || mask_stride >= cur_len + 1,
-                "decode_step: mask row stride %d shorter than %d (0 = one row for all sequences)", mask_stride, cur_len + 1);
-    AKV_REQUIRE((int64_t)max_seq_len * head_dim < (int64_t)1 << 31 && (int64_t)n_max_blocks * head_dim * d_block < (int64_t)1 << 31,
-                "decode_step: one (batch, head) slice of a high-byte plane must stay below 2 GiB");
-    const size_t need = akv_decode_step_workspace_bytes(bsz, n_kv_heads, head_dim, max_seq_len);
-    AKV_REQUIRE(workspace_bytes >= need, "decode_step: workspace of %zu bytes, %zu needed", workspace_bytes, need);
-    AKV_REQUIRE(((uintptr_t)workspace & 255) == 0 && ((uintptr_t)scores & 15) == 0 && ((uintptr_t)probs & 15) == 0,
-                "decode_step: workspace must be 256-byte aligned, scores/probs 16-byte aligned");
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    uint8_t *ws = static_cast<uint8_t *>(workspace);
-#define AKV_STEP(DD)                                                                                                  \
-    return run_step<DD>(k_first_8, k_mid_4, k_last_4, v_first_8, v_mid_4, v_last_4, k_exp_column_max, v_exp_column_max, \
-                        restk, restv, q, k_new, v_new, mask, mask_stride, out, scores, probs, row_stride, ws,          \
-                        k_levels_out, v_levels_out, amin_out, bsz, n_kv_heads, n_max_blocks, max_seq_len, d_block,     \
-                        top_max_k, cur_len, rest_start, rest_len, reference != 0, literal_broadcast, st);
-    if (head_dim == 64) { AKV_STEP(64) }
-    if (head_dim == 128) { AKV_STEP(128) }
-    AKV_STEP(256)
-#undef AKV_STEP
+    return akv_decode_step_gqa(k_first_8, k_mid_4, k_last_4, v_first_8, v_mid_4, v_last_4, k_exp_column_max,
+                               v_exp_column_max, restk, restv, q, k_new, v_new, mask, mask_stride, out, scores, probs,
+                               row_stride, workspace, workspace_bytes, k_levels_out, v_levels_out, amin_out, bsz,
+                               n_kv_heads, n_kv_heads, n_max_blocks, max_seq_len, head_dim, d_block, top_max_k, cur_len,
+                               nullptr, reference, literal_broadcast, stream);
 }

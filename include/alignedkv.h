@@ -142,7 +142,7 @@ AKV_API int akv_v_cache_compute(const uint8_t *first_8, const uint8_t *mid_4, co
  * (extension/v_cache_file.py:157-160 broadcasts [B,H,1,D] against [B,1,H,D]).
  * Supported: head_dim 64/128/256, d_block 64, top_max_k 32; other shapes go through the five ops.
  */
-AKV_API size_t akv_decode_step_workspace_bytes(int bsz, int n_kv_heads, int head_dim, int max_seq_len);
+AKV_API size_t akv_decode_step_workspace_bytes(int bsz, int n_q_heads, int head_dim, int max_seq_len);
 AKV_API int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,
                             uint8_t *v_mid_4, uint8_t *v_last_4, uint8_t *k_exp_column_max,
                             uint8_t *v_exp_column_max, uint8_t *restk, uint8_t *restv, const uint8_t *q,
@@ -152,6 +152,28 @@ AKV_API int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_las
                             int bsz, int n_kv_heads, int n_max_blocks, int max_seq_len, int head_dim, int d_block,
                             int top_max_k, int cur_len, int rest_start, int rest_len, int reference,
                             int literal_broadcast, akv_stream_t stream);
+
+/*
+ * The fused decode step for grouped-query attention and per-sequence lengths; beyond the reference, which
+ * asserts multi-head attention and keeps one scalar length per layer (model/KVCache_AlignedKV.py:32,
+ * extension/k_cache_file.py:133, extension/v_cache_file.py:146).  Per query head the algorithm is the
+ * reference's, on the planes of KV head (query head / group size): q, out [bsz,1,n_q_heads,head_dim];
+ * k_new, v_new, planes, column maxima, rest buffers per KV head; scores / probs [bsz, n_q_heads, row_stride];
+ * k_levels_out [bsz,n_q_heads,head_dim], v_levels_out [bsz,n_q_heads,(cur_len+1)/64*64], amin_out [bsz,n_q_heads].
+ * seq_lens == NULL: every sequence holds cur_len tokens (akv_decode_step is this case with n_q_heads ==
+ * n_kv_heads).  seq_lens != NULL: device int32 [bsz], tokens cached per sequence before the step; cur_len is
+ * then an upper bound of them (it sizes the launches), a sequence flushes its rest buffer on the step that
+ * fills it, and the step increments every entry of seq_lens on the device.
+ */
+AKV_API int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,
+                                uint8_t *v_mid_4, uint8_t *v_last_4, uint8_t *k_exp_column_max,
+                                uint8_t *v_exp_column_max, uint8_t *restk, uint8_t *restv, const uint8_t *q,
+                                const uint8_t *k_new, const uint8_t *v_new, const uint8_t *mask, int mask_stride,
+                                uint8_t *out, uint8_t *scores, uint8_t *probs, int row_stride, void *workspace,
+                                size_t workspace_bytes, uint8_t *k_levels_out, uint8_t *v_levels_out, uint8_t *amin_out,
+                                int bsz, int n_q_heads, int n_kv_heads, int n_max_blocks, int max_seq_len, int head_dim,
+                                int d_block, int top_max_k, int cur_len, int *seq_lens, int reference,
+                                int literal_broadcast, akv_stream_t stream);
 
 /*
  * Dense fp16 decode attention, the baseline of the benchmark (semantics of the reference's dense branch,
