@@ -206,5 +206,56 @@ class _AlignedKVModule:
                                       top_max_k, cur_len, rest_start, rest_len, int(bool(reference)),
                                       int(bool(literal_broadcast)), _stream_ptr(dev)), lib)
 
+    def decode_step_gqa(self, k_planes, v_planes, k_exp_column_max, v_exp_column_max, restk, restv, q, k_new, v_new,
+                        mask, out, scores, probs, bsz, n_q_heads, n_kv_heads, n_max_blocks, max_seq_len, head_dim,
+                        d_block, top_max_k, cur_len, seq_lens, reference, k_levels_out=None, v_levels_out=None,
+                        amin_out=None):
+        """Fused step with grouped-query heads and optional per-sequence lengths (seq_lens: int32 device tensor
+        [bsz], incremented by the step; cur_len then bounds them).  See akv_decode_step_gqa in include/alignedkv.h."""
+        lib = load_library()
+        dev = q.device
+        kplane = bsz * n_kv_heads * n_max_blocks * head_dim * d_block
+        vplane = bsz * n_kv_heads * max_seq_len * head_dim
+        tok_q, tok_kv = bsz * n_q_heads * head_dim * 2, bsz * n_kv_heads * head_dim * 2
+        for name, t, n in (("k_first_8", k_planes[0], kplane), ("k_mid_4", k_planes[1], kplane // 2),
+                           ("k_last_4", k_planes[2], kplane // 2), ("v_first_8", v_planes[0], vplane),
+                           ("v_mid_4", v_planes[1], vplane // 2), ("v_last_4", v_planes[2], vplane // 2),
+                           ("k_exp_column_max", k_exp_column_max, tok_kv // 2),
+                           ("v_exp_column_max", v_exp_column_max, tok_kv // 2), ("restk", restk, tok_kv * d_block),
+                           ("restv", restv, tok_kv * d_block), ("q", q, tok_q), ("k_new", k_new, tok_kv),
+                           ("v_new", v_new, tok_kv), ("out", out, tok_q)):
+            _require(name, t, n, dev)
+        row_stride = scores.shape[-1] // 2
+        _require("scores", scores, bsz * n_q_heads * row_stride * 2, dev)
+        _require("probs", probs, bsz * n_q_heads * row_stride * 2, dev)
+        if seq_lens is not None:
+            if seq_lens.dtype != torch.int32 or not seq_lens.is_cuda or seq_lens.numel() != bsz or not seq_lens.is_contiguous():
+                raise RuntimeError("seq_lens: expected a contiguous int32 tensor [bsz] on the GPU")
+        mask_stride = 0
+        if mask is not None:
+            if mask.dtype != torch.uint8 or mask.dim() != 2 or mask.stride(-1) != 1 or not mask.is_cuda:
+                raise RuntimeError("mask: expected a 2-d uint8 view [rows, 2*len] of an fp16 mask on the GPU")
+            if mask.shape[0] not in (1, bsz) or mask.shape[1] < 2 * (cur_len + 1):
+                raise RuntimeError(f"mask: shape {tuple(mask.shape)} does not cover {bsz} x {cur_len + 1} halves")
+            mask_stride = 0 if mask.shape[0] == 1 else mask.stride(0) // 2
+        flushed = (cur_len + 1) // d_block * d_block
+        if k_levels_out is not None:
+            _require("k_levels_out", k_levels_out, bsz * n_q_heads * head_dim, dev)
+        if v_levels_out is not None:
+            _require("v_levels_out", v_levels_out, bsz * n_q_heads * flushed, dev)
+        if amin_out is not None:
+            _require("amin_out", amin_out, bsz * n_q_heads, dev)
+        need = lib.akv_decode_step_workspace_bytes(bsz, n_q_heads, head_dim, max_seq_len)
+        ws = self._workspace(dev, need)
+        with torch.cuda.device(dev):
+            check(lib.akv_decode_step_gqa(_ptr(k_planes[0]), _ptr(k_planes[1]), _ptr(k_planes[2]), _ptr(v_planes[0]),
+                                          _ptr(v_planes[1]), _ptr(v_planes[2]), _ptr(k_exp_column_max),
+                                          _ptr(v_exp_column_max), _ptr(restk), _ptr(restv), _ptr(q), _ptr(k_new),
+                                          _ptr(v_new), _ptr(mask), mask_stride, _ptr(out), _ptr(scores), _ptr(probs),
+                                          row_stride, _ptr(ws), ws.numel(), _ptr(k_levels_out), _ptr(v_levels_out),
+                                          _ptr(amin_out), bsz, n_q_heads, n_kv_heads, n_max_blocks, max_seq_len,
+                                          head_dim, d_block, top_max_k, cur_len, _ptr(seq_lens),
+                                          int(bool(reference)), 0, _stream_ptr(dev)), lib)
+
 
 cuda_module = _AlignedKVModule()
