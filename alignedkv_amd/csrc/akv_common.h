@@ -60,9 +60,12 @@ __device__ __forceinline__ int v_level(unsigned char amin_u8, unsigned short s_b
 // bytes (M = 0x88888888, L = 0 for level 2; L = 0x88888888 for level 1), which reproduces
 // hi<<8|0x80 and hi<<8|mid<<4|0x8 (reference: extension/csrc/K_cache.cu:201-205,249-252).
 // acc[i] += value(element i) * x.
-__device__ __forceinline__ void fma8(float *acc, u32 Ha, u32 Hb, u32 M, u32 L, float x) {
-    u32 E = (M & 0xF0F0F0F0u) | ((L >> 4) & 0x0F0F0F0Fu);   // low bytes of elements 0,2,4,6
-    u32 O = ((M << 4) & 0xF0F0F0F0u) | (L & 0x0F0F0F0Fu);   // low bytes of elements 1,3,5,7
+// E / O: the low bytes of the even / odd elements of 8 elements, from their 4 mid and 4 last bytes.
+__device__ __forceinline__ void split_even_odd(u32 M, u32 L, u32 &E, u32 &O) {
+    E = (M & 0xF0F0F0F0u) | ((L >> 4) & 0x0F0F0F0Fu);   // low bytes of elements 0,2,4,6
+    O = ((M << 4) & 0xF0F0F0F0u) | (L & 0x0F0F0F0Fu);   // low bytes of elements 1,3,5,7
+}
+__device__ __forceinline__ void fma8_even_odd(float *acc, u32 Ha, u32 Hb, u32 E, u32 O, float x) {
     u32 w02 = __builtin_amdgcn_perm(Ha, E, 0x06010400u);
     u32 w13 = __builtin_amdgcn_perm(Ha, O, 0x07010500u);
     u32 w46 = __builtin_amdgcn_perm(Hb, E, 0x06030402u);
@@ -75,6 +78,18 @@ __device__ __forceinline__ void fma8(float *acc, u32 Ha, u32 Hb, u32 M, u32 L, f
     acc[6] = fmaf(hi_half_to_float(w46), x, acc[6]);
     acc[5] = fmaf(lo_half_to_float(w57), x, acc[5]);
     acc[7] = fmaf(hi_half_to_float(w57), x, acc[7]);
+}
+__device__ __forceinline__ void fma8(float *acc, u32 Ha, u32 Hb, u32 M, u32 L, float x) {
+    u32 E, O;
+    split_even_odd(M, L, E, O);
+    fma8_even_odd(acc, Ha, Hb, E, O, x);
+}
+// A fetch level as a pair (keep, put) applied to the even/odd low bytes of fully fetched planes:
+// low = (low & keep) | put gives low (level 0), (mid << 4) | 0x8 (level 1), 0x80 (level 2).  Used where
+// several query heads with different levels share one fetched tile.
+__device__ __forceinline__ void level_masks(int level, u32 &keep, u32 &put) {
+    keep = level == 0 ? 0xFFFFFFFFu : (level == 1 ? 0xF0F0F0F0u : 0u);
+    put = level == 0 ? 0u : (level == 1 ? 0x08080808u : 0x80808080u);
 }
 
 // Scalar reconstruction used by the generic (any-shape) kernels.

@@ -14,7 +14,7 @@
 //   combine  adds the chunk partials in a fixed order, rounds to fp16 and adds the fp16 tail part
 // On a step that fills the rest buffer (64 tokens) a persist kernel and the two plane-write kernels
 // run first, exactly as the reference flushes before it computes.
-#include "akv_cores.h"
+#include "akv_step.h"
 
 namespace akv {
 
@@ -24,8 +24,6 @@ int launch_k_save_blocks(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, cons
                          hipStream_t st);
 int launch_v_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *v_new, int bsz, int heads,
                   int max_seq_len, int head_dim, int start_pos, int seq_len, int v_new_seq, hipStream_t st);
-
-__device__ __forceinline__ u32 exp_field(u32 half_bits) { return (half_bits >> 10) & 0x1fu; }
 
 // Optional per-phase timing of the fused step (benchmark aid): when enabled, events are recorded on the
 // step's stream around the K pass, the middle kernel, the V pass and the combine kernel.
@@ -46,40 +44,6 @@ __device__ __forceinline__ float wave_max(float v) {
     for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
     return v;
 }
-
-// Shape and per-sequence state of one step.  Query head hq reads the planes of KV head hq / G (grouped-query
-// attention; G == 1 is the reference's multi-head case).  seq_lens (device, may be null) holds the tokens
-// cached before this step per sequence; without it every sequence has cur_len tokens.
-struct StepGeom {
-    int Hq, Hkv, G;
-    int cb, max_seq_len, n_max_blocks, row_stride;
-    int cur_len;
-    const int *seq_lens;
-};
-
-// tokens flushed into the planes / held in the rest buffer once this step's token has been appended
-__device__ __forceinline__ void seq_state(const StepGeom &g, int b, int &R, int &nrest) {
-    const int L = (g.seq_lens != nullptr ? g.seq_lens[b] : g.cur_len) + 1;
-    R = (L / g.cb) * g.cb;
-    nrest = L - R;
-}
-
-// Workgroup -> (chunk, query head of the group).  Workgroups go to the 8 XCDs round-robin by linear index,
-// and each XCD has its own L2: the G workgroups that stream the same plane chunk for the G query heads of a
-// KV head get linear indices 8 apart, i.e. the same XCD at about the same time, so the chunk comes from HBM
-// once and from that L2 G-1 times.  gridDim.x = 8 * ceil(chunks / 8) * G.
-__device__ __forceinline__ void decode_group_block(int G, int &chunk, int &gq) {
-    const int lin = blockIdx.x;
-    if (G == 1) {
-        chunk = lin;
-        gq = 0;
-    } else {
-        const int t = lin >> 3;
-        gq = t % G;
-        chunk = (t / G) * 8 + (lin & 7);
-    }
-}
-static inline int group_grid_x(int chunks, int G) { return G == 1 ? chunks : ((chunks + 7) / 8) * 8 * G; }
 
 // ------------------------------------------------------------------------------------------------
 // persist (flush steps only): token -> rest buffers, column maxima.  grid (B*H), D threads.
@@ -803,7 +767,12 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         mark(4, st);
         return check_launch("decode_step(mono)");
     }
-    if (n_blocks > 0) {
+    // grouped-query heads: one workgroup per plane chunk serves 2 or 4 query heads (AKV_TUNE_GROUP: see group_heads)
+    const bool grouped = group_heads(geo.G) > 1;
+    if (n_blocks > 0 && grouped) {
+        int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo, B, n_blocks, ref, scale, st);
+        if (rc != AKV_OK) return rc;
+    } else if (n_blocks > 0) {
         const int bpw = k_blocks_per_wave(B, Hq, n_blocks);
         dim3 grid(group_grid_x((n_blocks + 4 * bpw - 1) / (4 * bpw), geo.G), Hkv, B);
         if (ref)
@@ -825,8 +794,11 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
     }
     mark(2, st);
-    const VPlan p = v_plan(B, Hq, D, R);
-    if (p.n_chunks > 0) {
+    const VPlan p = v_plan(B, grouped ? Hq / group_heads(geo.G) : Hq, D, R);
+    if (p.n_chunks > 0 && grouped) {
+        rc = launch_group_v_pass<D>(vf8, vm4, vl4, p16, amin, partial, v_levels_out, R, amin_out, geo, B, p, ref, st);
+        if (rc != AKV_OK) return rc;
+    } else if (p.n_chunks > 0) {
         dim3 grid(group_grid_x(p.n_chunks, geo.G), Hkv, B);
 #define AKV_VP(RF, N)                                                                                                  \
     hipLaunchKernelGGL((fused_v_pass_kernel<D, RF, N>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, amin, partial,     \

@@ -1,0 +1,57 @@
+// Shape and per-sequence state of the fused decode step, shared by its kernels.
+#pragma once
+
+#include "akv_cores.h"
+
+namespace akv {
+
+__device__ __forceinline__ u32 exp_field(u32 half_bits) { return (half_bits >> 10) & 0x1fu; }
+
+// Shape and per-sequence state of one step.  Query head hq reads the planes of KV head hq / G (grouped-query
+// attention; G == 1 is the reference's multi-head case).  seq_lens (device, may be null) holds the tokens
+// cached before this step per sequence; without it every sequence has cur_len tokens.
+struct StepGeom {
+    int Hq, Hkv, G;
+    int cb, max_seq_len, n_max_blocks, row_stride;
+    int cur_len;
+    const int *seq_lens;
+};
+
+// tokens flushed into the planes / held in the rest buffer once this step's token has been appended
+__device__ __forceinline__ void seq_state(const StepGeom &g, int b, int &R, int &nrest) {
+    const int L = (g.seq_lens != nullptr ? g.seq_lens[b] : g.cur_len) + 1;
+    R = (L / g.cb) * g.cb;
+    nrest = L - R;
+}
+
+// Workgroup -> (chunk, query head of the group).  Workgroups go to the 8 XCDs round-robin by linear index,
+// and each XCD has its own L2: the G workgroups that stream the same plane chunk for the G query heads of a
+// KV head get linear indices 8 apart, i.e. the same XCD at about the same time, so the chunk comes from HBM
+// once and from that L2 G-1 times.  gridDim.x = 8 * ceil(chunks / 8) * G.
+__device__ __forceinline__ void decode_group_block(int G, int &chunk, int &gq) {
+    const int lin = blockIdx.x;
+    if (G == 1) {
+        chunk = lin;
+        gq = 0;
+    } else {
+        const int t = lin >> 3;
+        gq = t % G;
+        chunk = (t / G) * 8 + (lin & 7);
+    }
+}
+static inline int group_grid_x(int chunks, int G) { return G == 1 ? chunks : ((chunks + 7) / 8) * 8 * G; }
+
+
+// Grouped-query passes (akv_gqa.hip): one workgroup serves group_heads(G) query heads of a KV head.
+int group_heads(int G);
+template <int D>
+int launch_group_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *kcm,
+                        const unsigned short *q, const unsigned short *k_new, unsigned short *scores,
+                        uint8_t *levels_out, const StepGeom &geo, int B, int n_blocks, bool ref, float scale,
+                        hipStream_t st);
+template <int D>
+int launch_group_v_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const unsigned short *probs,
+                        const uint8_t *amin, float *partial, uint8_t *levels_out, int levels_stride, uint8_t *amin_out,
+                        const StepGeom &geo, int B, const VPlan &p, bool ref, hipStream_t st);
+
+}  // namespace akv

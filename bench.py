@@ -44,8 +44,11 @@ def parse():
     ap.add_argument("--layers", type=int, default=4, help="caches the steps rotate over")
     ap.add_argument("--k-kind", default="outlier", choices=["outlier", "lognormal"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-steps", type=int, default=3)
+    ap.add_argument("--cpu-steps", type=int, default=10)
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3"],
+                    help="c2: the headline configuration (shape flags apply); c3: grouped-query heads (32 over 8), batch 32, "
+                         "lengths uniform in [2048, 8192] -- an extra line, not the headline metric")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB copy kernel (known size, for scaling hardware byte counters)")
     return ap.parse_args()
@@ -183,11 +186,101 @@ def cpu_baseline(torch, cache, q, k_new, v_new, n_steps):
     return min(times), out.reshape(B, 1, H, D), klv, vlv, OC.num_threads()
 
 
+def bench_c3(a):
+    """Grouped-query, ragged-length decode step (akv_decode_step_gqa) at batch 32, 32 query heads over 8 KV
+    heads x 128, lengths uniform in [2048, 8192].  The lengths are reset before every step so that each step
+    sees the same state."""
+    import numpy as np
+    import torch
+    import alignedkv_amd
+    from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
+    lib = alignedkv_amd.load_library()
+    B, Hq, Hkv, D, cb = 32, 32, 8, 128, 64
+    Lmax = 8192 + cb
+    lens = np.random.default_rng(a.seed + 3).integers(2048, 8193, B)
+    cache = RaggedGQACache(a.layers, B, Lmax, Hq, Hkv, D)
+    for layer in range(a.layers):
+        for b in range(B):
+            k, v = make_layer_inputs(torch, 1, int(lens[b]), Hkv, D, a.seed + 100 * layer + b, "outlier")
+            cache.prefill(layer, b, k, v)
+    g = torch.Generator(device="cuda").manual_seed(a.seed + 999)
+    q = torch.randn((B, 1, Hq, D), device="cuda", generator=g).half()
+    k_new = torch.randn((B, 1, Hkv, D), device="cuda", generator=g).half()
+    v_new = (0.5 * torch.randn((B, 1, Hkv, D), device="cuda", generator=g)).half()
+    lens0 = torch.from_numpy(lens.astype(np.int32)).cuda()
+    bound = int(lens.max())
+    cache.record_levels = True
+
+    def run(reference, steps, warmup):
+        cache.reference = reference
+        t0 = 0.0
+        for i in range(warmup + steps):
+            if i == warmup:
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+            layer = i % a.layers
+            cache.seq_lens[layer].copy_(lens0)
+            cache.len_bound[layer] = bound
+            cache.decode(layer, q, k_new, v_new)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps
+
+    cache.record_levels = True
+    cache.seq_lens[0].copy_(lens0)
+    cache.len_bound[0] = bound
+    cache.decode(0, q, k_new, v_new)
+    klv = cache.last_k_levels.cpu().numpy()
+    vlv = cache.last_v_levels.cpu().numpy()
+    cache.record_levels = False
+    kv_bytes = dense = 0.0
+    for b in range(B):
+        R = (int(lens[b]) + 1) // cb * cb
+        # a KV element is fetched at the finest level any query head of its group asks for
+        kl = klv[b].reshape(Hkv, Hq // Hkv, D).min(1)
+        vl = vlv[b, :, :R].reshape(Hkv, Hq // Hkv, R).min(1)
+        kv_bytes += R * (kl.size + 0.5 * (kl < 2).sum() + 0.5 * (kl == 0).sum())
+        kv_bytes += D * (vl.size + 0.5 * (vl < 2).sum() + 0.5 * (vl == 0).sum())
+        dense += 2 * Hkv * (int(lens[b]) + 1) * D * 2
+    sec = run(False, a.steps, a.warmup)
+    sec_ref = run(True, max(a.steps // 2, 20), 10)
+    cache.reference = False
+    lib.akv_profile_enable(1)
+    import ctypes
+    buf = (ctypes.c_float * 4)()
+    acc = [0.0] * 4
+    n = min(a.steps, 100)
+    for i in range(n + 4):
+        layer = i % a.layers
+        cache.seq_lens[layer].copy_(lens0)
+        cache.len_bound[layer] = bound
+        cache.decode(layer, q, k_new, v_new)
+        lib.akv_profile_read(buf)
+        if i >= 4:
+            for j in range(4):
+                acc[j] += buf[j] * 1e3 / n
+    lib.akv_profile_enable(0)
+    res = {"metric": "decode-attn us/step, grouped-query 32 over 8 heads x 128, batch 32, lengths U[2048,8192]",
+           "value": round(sec * 1e6, 2), "unit": "us/step", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+           "ms_per_step": round(sec * 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+           "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "C3: batch 32, 32 query heads over 8 KV heads x 128, %d cached tokens in total, "
+                                  "%d layers rotated" % (int(lens.sum()), a.layers)},
+           "kv_plane_bytes_union_of_group_levels": int(kv_bytes), "dense_fp16_bytes": int(dense),
+           "bytes_vs_dense": round(kv_bytes / dense, 4),
+           "effective_hbm_gbps": round(kv_bytes / sec / 1e9, 1), "pct_hbm_peak": round(100 * kv_bytes / sec / 1e9 / HBM_PEAK_GBPS, 1),
+           "kernel_us": {"k_pass": round(acc[0], 2), "middle": round(acc[1], 2), "v_pass": round(acc[2], 2),
+                         "combine": round(acc[3], 2)},
+           "dense_in_planes_us": round(sec_ref * 1e6, 2), "speedup_vs_dense_in_planes": round(sec_ref / sec, 3)}
+    print(json.dumps(res))
+
+
 def main():
     a = parse()
     if a.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
+    if a.workload == "c3":
+        return bench_c3(a)
     import numpy as np
     import torch
     import alignedkv_amd

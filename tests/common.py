@@ -39,10 +39,11 @@ def assert_close_fp16(got, want, abs_floor):
 
 
 def oracle_decode_step_c(k_planes, v_planes, k_colmax, v_colmax, q, k_new, v_new, R, d_block=64, top_k=32,
-                         reference=False):
-    """One decode step (cache of R flushed tokens, empty rest buffer, one appended token) with the C
-    restatement of the ops + the NumPy host logic.  All arguments are NumPy arrays in the reference layouts.
-    Returns (out [B,1,H,D] float16, k_levels, v_levels, amin, probs)."""
+                         reference=False, rest_k=None, rest_v=None):
+    """One decode step with the C restatement of the ops + the NumPy host logic: R tokens in the planes and,
+    after the append, the rest buffer given by rest_k/rest_v [B, n_rest, H, D] (default: only the appended
+    token; n_rest may be 0 when the append completed a block that the planes already hold).  All arguments
+    are NumPy arrays in the reference layouts.  Returns (out [B,1,H,D] float16, k_levels, v_levels, amin, probs)."""
     import math
     from oracle import akv_oracle as O
     from oracle import akv_oracle_c as OC
@@ -53,15 +54,20 @@ def oracle_decode_step_c(k_planes, v_planes, k_colmax, v_colmax, q, k_new, v_new
     ksum, kmax = O.k_sum_and_max(q, kcm2)
     s, klv = OC.k_cache_compute(*k_planes, ksum, kmax, O.as_bits(q), nb, d_block, 1.0 / math.sqrt(D), reference)
     s = s.copy()
+    if rest_k is None:
+        rest_k, rest_v = k_new, v_new
+    n_rest = rest_k.shape[1]
     restk = np.zeros((B, d_block, H, D), np.float16)
     restv = np.zeros((B, d_block, H, D), np.float16)
-    restk[:, :1], restv[:, :1] = k_new, v_new
-    s[:, :, :, R:R + 1] = O.rest_scores(q, restk, 1, D)
-    s[:, :, :, R + 1:] = -np.inf
+    restk[:, :n_rest], restv[:, :n_rest] = rest_k, rest_v
+    if n_rest:
+        s[:, :, :, R:R + n_rest] = O.rest_scores(q, restk, n_rest, D)
+    s[:, :, :, R + n_rest:] = -np.inf
     p = O.softmax_fp32_to_half(s)
-    tv, ti = O.bucket_max(p[..., :R], R + 1, top_k)
+    tv, ti = O.bucket_max(p[..., :R], R + n_rest, top_k)
     to = OC.v_cache_test_compute(v_planes[0], O.as_bits(tv), ti, top_k)
     amin = O.alignment_min(O.test_o_exponent(to), vcm2)
     o, vlv = OC.v_cache_compute(*v_planes, O.as_bits(np.ascontiguousarray(p)), amin, R, reference)
-    o = (o + O.rest_output(p[..., R:R + 1], restv, 1)).astype(np.float16)
+    if n_rest:
+        o = (o + O.rest_output(p[..., R:R + n_rest], restv, n_rest)).astype(np.float16)
     return o.reshape(B, 1, H, D), klv, vlv, amin, p

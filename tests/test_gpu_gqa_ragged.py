@@ -88,3 +88,79 @@ def test_gqa_reads_each_kv_chunk_for_all_query_heads_consistently():
     mha.value_cache[0].save(dev(vr[:, :L]), 0, L)
     out_m = mha.auto_compute(dev(q), dev(kr[:, L:]), dev(vr[:, L:]), 0, None)
     assert torch.equal(out_g, out_m)
+
+
+def test_config3_full_size_against_c_oracle():
+    """C3: 32 query heads over 8 KV heads, head_dim 128, batch 32, lengths uniform in [2048, 8192], K with 4
+    outlier channels per KV head x10, V ~ N(0, 0.5).  Every sequence is checked against the C restatement of
+    the ops run on its own planes with the KV heads repeated."""
+    from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
+    from tests.common import oracle_decode_step_c
+    B, Hq, Hkv, D, cb = 32, 32, 8, 128, 64
+    G = Hq // Hkv
+    Lmax = 8192 + cb
+    lens = np.random.default_rng(3).integers(2048, 8193, B)
+    lens[:4] = [2048, 8191, 4159, 8192]          # block-aligned, two that complete a block with the append, the maximum
+    cache = RaggedGQACache(1, B, Lmax, Hq, Hkv, D)
+    cache.record_levels = True
+    gen = torch.Generator(device="cuda").manual_seed(33)
+    tails = []
+    for b in range(B):
+        S = int(lens[b])
+        k = torch.randn((1, S, Hkv, D), device="cuda", generator=gen)
+        for h in range(Hkv):
+            ch = torch.randperm(D, generator=torch.Generator().manual_seed(1000 + h))[:4].cuda()
+            k[:, :, h, ch] *= 10.0
+        k = k.half()
+        v = (0.5 * torch.randn((1, S, Hkv, D), device="cuda", generator=gen)).half()
+        cache.prefill(0, b, k, v)
+        t = S % cb
+        tails.append((k[:, S - t:].cpu().numpy(), v[:, S - t:].cpu().numpy()))
+    colmax_k = cache.k_colmax[0].cpu().numpy()
+    colmax_v = cache.v_colmax[0].cpu().numpy()
+    q = torch.randn((B, 1, Hq, D), device="cuda", generator=gen).half()
+    kn = torch.randn((B, 1, Hkv, D), device="cuda", generator=gen).half()
+    vn = (0.5 * torch.randn((B, 1, Hkv, D), device="cuda", generator=gen)).half()
+    out = cache.decode(0, q, kn, vn).cpu().numpy()
+    assert cache.seq_lens[0].cpu().tolist() == [int(l) + 1 for l in lens]
+    qh, knh, vnh = q.cpu().numpy(), kn.cpu().numpy(), vn.cpu().numpy()
+    worst = 0.0
+    flips = total = 0
+    moved = dense = 0.0
+    for b in range(B):
+        L = int(lens[b]) + 1
+        R = L // cb * cb
+        rk = np.concatenate([tails[b][0], knh[b:b + 1]], axis=1)
+        rv = np.concatenate([tails[b][1], vnh[b:b + 1]], axis=1)
+        kpl = [p[b:b + 1, :, :R // cb].cpu().numpy() for p in cache.k_planes[0]]
+        vpl = [p[b:b + 1, :, :R].cpu().numpy() for p in cache.v_planes[0]]
+        if rk.shape[1] == cb:
+            # the append completed a block: what the step wrote into the planes must be the NumPy split of it
+            blk = R // cb - 1
+            ref_k = O.k_planes_alloc(1, Hkv, cb, D)
+            O.k_cache_save(*ref_k, O.as_bits(rk), 1, cb, 0, cb)
+            ref_v = O.v_planes_alloc(1, Hkv, cb, D)
+            O.v_cache_save(*ref_v, O.as_bits(rv), 0, cb)
+            for i in range(3):
+                assert np.array_equal(kpl[i][:, :, blk], ref_k[i][:, :, 0]), f"flushed K block, plane {i}, sequence {b}"
+                assert np.array_equal(vpl[i][:, :, R - cb:], ref_v[i]), f"flushed V block, plane {i}, sequence {b}"
+            rk, rv = rk[:, :0], rv[:, :0]
+        rep = lambda a, ax: np.ascontiguousarray(np.repeat(a, G, axis=ax))
+        want, klv, vlv, amin, p = oracle_decode_step_c([rep(x, 1) for x in kpl], [rep(x, 1) for x in vpl],
+                                                       rep(colmax_k[b:b + 1], 2), rep(colmax_v[b:b + 1], 2), qh[b:b + 1],
+                                                       rep(knh[b:b + 1], 2), rep(vnh[b:b + 1], 2), R,
+                                                       rest_k=rep(rk, 2), rest_v=rep(rv, 2))
+        assert np.array_equal(cache.last_k_levels[b].cpu().numpy(), klv[0]), f"K levels, sequence {b}"
+        assert np.array_equal(cache.last_alignment_min[b].cpu().numpy(), amin.reshape(-1)), f"threshold, sequence {b}"
+        got_v = cache.last_v_levels[b, :, :R].cpu().numpy()
+        got_p = cache.probs[b, :, :R].cpu().numpy()
+        assert np.array_equal(got_v, O.v_levels(amin.reshape(1, Hq), O.as_bits(got_p)[None])[0])
+        flips += int((got_v != vlv[0]).sum())
+        total += got_v.size
+        worst = max(worst, float(np.max(np.abs(out[b:b + 1].astype(np.float32) - want.astype(np.float32)))))
+        moved += R * ((klv < 3).sum() + 0.5 * (klv < 2).sum() + 0.5 * (klv == 0).sum()) / G \
+            + D * ((vlv < 3).sum() + 0.5 * (vlv < 2).sum() + 0.5 * (vlv == 0).sum()) / G
+        dense += 2 * Hkv * R * D * 2
+    assert worst <= 1e-3, f"max abs err {worst}"
+    assert flips <= 1e-3 * total
+    print(f"C3: max err {worst:.2e}, V level flips {flips}/{total}, plane bytes per query group {moved / dense:.3f} of dense")
