@@ -255,6 +255,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     __shared__ float probe_p[32];
     __shared__ int probe_t[32];
     __shared__ u32 red_min[NW];
+    __shared__ float tail_o[NW][D];           // per-wave sums of the tail's share of the output
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // bh indexes (batch, query head); the keys, values, column maxima and rest buffers belong to its KV head
     const int b = bh / a.g.Hq, hq = bh - b * a.g.Hq, h = hq / a.g.G;
@@ -314,14 +315,29 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
         vcm_mine = vc;
     }
     // (b) scores of the tail: fp16(fp16(q.k) / sqrt(D)), the two roundings of an fp16 matmul followed by
-    //     an fp16 division (extension/k_cache_file.py:156)
+    //     an fp16 division (extension/k_cache_file.py:156).  LPT lanes per tail token, 8 channels per 16-byte load:
+    //     all rows are in flight at once (a real decode step has 32 tail tokens on average).
     const float sqrt_d = sqrtf((float)D);
-    for (int r = wave; r < nrest; r += NW) {
-        const unsigned short *krow = (r == newest && a.persist) ? knew : a.restk + (((int64_t)b * cb + r) * Hkv + h) * D;
+    {
+        constexpr int LPT = NT / 64;          // lanes per token (the rest buffer holds at most 64 tokens)
+        const int r = tid / LPT, j = tid % LPT;
         float part = 0.f;
-        for (int c = lane; c < D; c += 64) part = fmaf(half_bits_to_float(krow[c]), half_bits_to_float(qrow[c]), part);
-        part = wave_sum(part);
-        if (lane == 0) {
+        if (r < nrest) {
+            const unsigned short *krow = (r == newest && a.persist) ? knew : a.restk + (((int64_t)b * cb + r) * Hkv + h) * D;
+            for (int v8 = j; v8 < D / 8; v8 += LPT) {
+                const u32x4 kw = *reinterpret_cast<const u32x4 *>(krow + v8 * 8);
+                const u32x4 qw = *reinterpret_cast<const u32x4 *>(qrow + v8 * 8);
+                const u32 kk[4] = {kw.x, kw.y, kw.z, kw.w}, qq[4] = {qw.x, qw.y, qw.z, qw.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    part = fmaf(lo_half_to_float(kk[i]), lo_half_to_float(qq[i]), part);
+                    part = fmaf(hi_half_to_float(kk[i]), hi_half_to_float(qq[i]), part);
+                }
+            }
+        }
+#pragma unroll
+        for (int mk = 1; mk < LPT; mk <<= 1) part += __shfl_xor(part, mk, 64);
+        if (r < nrest && j == 0) {
             const float dot16 = half_bits_to_float(float_to_half_bits(part));
             const unsigned short sc = float_to_half_bits(dot16 / sqrt_d);
             tail_s[r] = sc;
@@ -490,14 +506,44 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
         lds_barrier();
     }
     AKV_MTS(7)
-    // (f) the tail's share of the output, an fp16 matmul result (extension/v_cache_file.py:189)
-    for (int d = tid; d < D; d += NT) {
-        float acc = 0.f;
-        for (int r = 0; r < nrest; ++r) {
+    // (f) the tail's share of the output, an fp16 matmul result (extension/v_cache_file.py:189): a thread takes 8
+    //     channels of every NRG-th tail token, lanes of a wave that share the channels fold by shuffles, waves by LDS
+    {
+        constexpr int VPR = D / 8;            // 16-byte vectors per row
+        constexpr int NRG = NT / VPR;         // row groups
+        constexpr int RGW = 64 / VPR;         // row groups inside a wave
+        static_assert(VPR <= 32, "head_dim above 256 needs another tail mapping");
+        const int c8 = tid % VPR, rg = tid / VPR;
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+        for (int r = rg; r < nrest; r += NRG) {
             const unsigned short *vrow = (r == newest && a.persist) ? vnew : a.restv + (((int64_t)b * cb + r) * Hkv + h) * D;
-            acc = fmaf(half_bits_to_float(vrow[d]), tail_p[r], acc);
+            const u32x4 vw = *reinterpret_cast<const u32x4 *>(vrow + c8 * 8);
+            const u32 vv[4] = {vw.x, vw.y, vw.z, vw.w};
+            const float pr = tail_p[r];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[2 * i] = fmaf(lo_half_to_float(vv[i]), pr, acc[2 * i]);
+                acc[2 * i + 1] = fmaf(hi_half_to_float(vv[i]), pr, acc[2 * i + 1]);
+            }
         }
-        a.otail[(int64_t)bh * D + d] = float_to_half_bits(acc);
+#pragma unroll
+        for (int mk = VPR; mk < 64; mk <<= 1)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] += __shfl_xor(acc[i], mk, 64);
+        (void)RGW;
+        if (lane < VPR) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) tail_o[wave][c8 * 8 + i] = acc[i];
+        }
+        lds_barrier();
+        for (int d = tid; d < D; d += NT) {
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) sum += tail_o[w][d];
+            a.otail[(int64_t)bh * D + d] = float_to_half_bits(sum);
+        }
     }
 }
 
