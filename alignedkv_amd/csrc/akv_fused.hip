@@ -715,7 +715,7 @@ __global__ void fused_combine_kernel(const float *__restrict__ partial, const un
 }
 
 struct StepLayout {
-    size_t toe, amin, otail, partial, total;
+    size_t toe, amin, otail, partial, prep, total;
 };
 
 static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
@@ -729,7 +729,8 @@ static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
     l.amin = up((size_t)B * H * D);
     l.otail = l.amin + up((size_t)B * H);
     l.partial = l.otail + up((size_t)B * H * D * 2);
-    l.total = l.partial + up((size_t)B * H * max_chunks * D * sizeof(float));
+    l.prep = l.partial + up((size_t)B * H * max_chunks * D * sizeof(float));
+    l.total = l.prep + up((size_t)B * H * mfma_k_prep_words(D) * sizeof(u32));   // B * Hkv <= B * H rows are used
     return l;
 }
 
@@ -815,7 +816,13 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     }
     // grouped-query heads: one workgroup per plane chunk serves 2 or 4 query heads (AKV_TUNE_GROUP: see group_heads)
     const bool grouped = group_heads(geo.G) > 1;
-    if (n_blocks > 0 && grouped) {
+    bool matrix = geo.G >= 2 && geo.G <= 16;
+    if (const char *e = getenv("AKV_TUNE_MFMA")) matrix = matrix && atoi(e) != 0;
+    if (n_blocks > 0 && matrix) {
+        int rc = launch_mfma_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, reinterpret_cast<u32 *>(ws + lay.prep),
+                                       geo, B, n_blocks, ref, scale, st);
+        if (rc != AKV_OK) return rc;
+    } else if (n_blocks > 0 && grouped) {
         int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo, B, n_blocks, ref, scale, st);
         if (rc != AKV_OK) return rc;
     } else if (n_blocks > 0) {

@@ -1,0 +1,359 @@
+// Grouped-query K and V passes on the matrix cores.
+//
+// With G query heads per KV head the passes are skinny matrix products (tokens x channels times channels x G):
+// on the vector ALUs every query head repeats the unpack-and-multiply of the shared tile (2.5 vector operations
+// per query-head element), which makes the pass ALU-bound from G = 4 on.  Here the shared tile is unpacked ONCE
+// into fp16 MFMA operands and v_mfma_f32_16x16x16_f16 does the multiply for up to 16 query heads (columns) with
+// fp32 accumulation: fp16 x fp16 products are exact in fp32, so results differ from the vector kernels only in
+// summation order.
+//
+// Per-head fetch levels (K: extension/csrc/K_cache.cu:211,249-252; V: extension/csrc/V_cache.cu:195-197,250-253)
+// stay exact.  A plane row is fetched at the finest level any head of the group asks for ("union level"); the
+// operand A holds the values at that level.  A head with a coarser level needs the value with its low bits
+// replaced (0x8 / 0x80): value_at_level = A - C1 (level 1) or A - C2 (level 2) with C1 = A - sub1(A),
+// C2 = A - sub2(A).  Both differences are exact in fp16 (same sign, exponent and upper mantissa), so two more
+// MFMAs with the operands (C1, -q [level == 1]) and (C2, -q [level == 2]) give every head exactly its own levels.
+#include "akv_step.h"
+
+namespace akv {
+
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f16x4 as_f16x4(u32 lo, u32 hi) {
+    union { u32 u[2]; f16x4 v; } x;
+    x.u[0] = lo;
+    x.u[1] = hi;
+    return x.v;
+}
+__device__ __forceinline__ f16x2 as_f16x2(u32 w) {
+    union { u32 u; f16x2 v; } x;
+    x.u = w;
+    return x.v;
+}
+__device__ __forceinline__ u32 as_u32(f16x2 v) {
+    union { u32 u; f16x2 v; } x;
+    x.v = v;
+    return x.u;
+}
+// packed pair of fp16 values minus the same pair with the low bits replaced: exact
+__device__ __forceinline__ u32 low_bits_excess(u32 w, u32 keep, u32 put) {
+    return as_u32(as_f16x2(w) - as_f16x2((w & keep) | put));
+}
+
+// acc += A x B0  (+ C1 x B1 + C2 x B2 unless every plane is read)
+template <bool REF>
+__device__ __forceinline__ void mfma_levels(f32x4 &acc, u32 a_lo, u32 a_hi, f16x4 b0, f16x4 b1, f16x4 b2) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x16f16(as_f16x4(a_lo, a_hi), b0, acc, 0, 0, 0);
+    if (!REF) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x16f16(
+            as_f16x4(low_bits_excess(a_lo, 0xFFF0FFF0u, 0x00080008u), low_bits_excess(a_hi, 0xFFF0FFF0u, 0x00080008u)), b1,
+            acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x16f16(
+            as_f16x4(low_bits_excess(a_lo, 0xFF00FF00u, 0x00800080u), low_bits_excess(a_hi, 0xFF00FF00u, 0x00800080u)), b2,
+            acc, 0, 0, 0);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// K pass.  A wave takes tasks of SL/4 blocks (SL = slots per lane: 16, 8 or 4).  Lane l: token set ts = l % 16 =
+// (block of the task, piece of SL slots of its 64), channel residue cs = l / 16; per channel group kg (16
+// channels) it loads the SL slots of the channels 16 kg + 4 r + cs (r < 4).  In the MFMA the token sets are the
+// rows, (cs, r) the contraction index, the query heads the columns: the partial sums over channels that the
+// vector kernel folds with 15 shuffles per head are summed inside the instruction.  Lane (j, ig) ends up with
+// the scores of token sets 4 ig .. 4 ig + 3 for query head j.
+// Smaller SL: fewer accumulators (4 SL registers) and smaller tiles, hence more waves per SIMD and more tiles in
+// flight per wave at the same register budget -- what hides the several-microsecond loaded HBM latency -- at the
+// price of narrower loads.
+// grid (ceil(tasks / (4 * tasks_per_wave)), Hkv, B), 256 threads.
+// ------------------------------------------------------------------------------------------------
+template <int SL>
+struct KTaskTile {   // one channel group: 4 channels x SL slots per lane
+    u32 h[4][SL / 4];
+    u32 m[4][(SL + 7) / 8], l[4][(SL + 7) / 8];
+};
+
+template <int NB>
+__device__ __forceinline__ void load_bytes(u32 *dst, const __amdgpu_buffer_rsrc_t r, int off) {
+    if constexpr (NB == 16) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+        dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+    } else if constexpr (NB == 8) {
+        const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+        dst[0] = v.x; dst[1] = v.y;
+    } else if constexpr (NB == 4) {
+        dst[0] = __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0);
+    } else {
+        dst[0] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0);
+    }
+}
+
+template <int D, int SL>
+__device__ __forceinline__ void kt_issue(KTaskTile<SL> &t, const __amdgpu_buffer_rsrc_t rH, const __amdgpu_buffer_rsrc_t rM,
+                                         const __amdgpu_buffer_rsrc_t rL, int blk, int kg, u32 need_mid, u32 need_last) {
+    constexpr int PB = 64 / SL;   // pieces per block
+    const int lane = threadIdx.x & 63;
+    const int piece = (lane & 15) % PB, cs = lane >> 4;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int c = 16 * kg + 4 * r + cs;
+        load_bytes<SL>(t.h[r], rH, blk * (D * 64) + c * 64 + piece * SL);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int c = 16 * kg + 4 * r + cs;
+        const int off = blk * (D * 32) + c * 32 + piece * (SL / 2);
+        load_bytes<SL / 2>(t.m[r], rM, ((need_mid >> (4 * kg + r)) & 1u) ? off : kSkip);
+        load_bytes<SL / 2>(t.l[r], rL, ((need_last >> (4 * kg + r)) & 1u) ? off : kSkip);
+    }
+}
+
+template <bool REF, int SL>
+__device__ __forceinline__ void kt_compute(f32x4 *acc, const KTaskTile<SL> &t, int kg, u32 need_mid, u32 need_last, f16x4 b0,
+                                           f16x4 b1, f16x4 b2) {
+    constexpr int NX = (SL + 7) / 8;       // units of 8 slots (one unit of 4 for SL == 4)
+    constexpr int NP = SL == 4 ? 2 : 4;    // slot pairs per unit
+#pragma unroll
+    for (int x = 0; x < NX; ++x) {
+        u32 w[4][4];                 // [r][pair]: slots 8x + (0,2), (1,3), (4,6), (5,7) of channel r
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const bool mid = (need_mid >> (4 * kg + r)) & 1u, last = (need_last >> (4 * kg + r)) & 1u;
+            const u32 cm = mid ? 0u : 0x88888888u;               // union level 2: low byte 0x80
+            const u32 cl = (mid && !last) ? 0x88888888u : 0u;    // union level 1: last nibble 0x8
+            u32 E, O;
+            split_even_odd(t.m[r][x] | cm, t.l[r][x] | cl, E, O);
+            const u32 Ha = t.h[r][SL == 4 ? 0 : 2 * x];
+            w[r][0] = __builtin_amdgcn_perm(Ha, E, 0x06010400u);
+            w[r][1] = __builtin_amdgcn_perm(Ha, O, 0x07010500u);
+            if constexpr (SL != 4) {
+                const u32 Hb = t.h[r][2 * x + 1];
+                w[r][2] = __builtin_amdgcn_perm(Hb, E, 0x06030402u);
+                w[r][3] = __builtin_amdgcn_perm(Hb, O, 0x07030502u);
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int s0 = 8 * x + (p & 1) + 4 * (p >> 1);        // the pair holds slots s0 and s0 + 2
+            // 2x2 transposes: (channel r, slot pair) -> (slot, channel pair)
+            const u32 a01_s0 = __builtin_amdgcn_perm(w[1][p], w[0][p], 0x05040100u);
+            const u32 a23_s0 = __builtin_amdgcn_perm(w[3][p], w[2][p], 0x05040100u);
+            const u32 a01_s2 = __builtin_amdgcn_perm(w[1][p], w[0][p], 0x07060302u);
+            const u32 a23_s2 = __builtin_amdgcn_perm(w[3][p], w[2][p], 0x07060302u);
+            mfma_levels<REF>(acc[s0], a01_s0, a23_s0, b0, b1, b2);
+            mfma_levels<REF>(acc[s0 + 2], a01_s2, a23_s2, b0, b1, b2);
+        }
+    }
+}
+
+// Set-up of the K pass, once per (batch, KV head) instead of once per wave: lane (j, kq) = (l % 16, l / 16) takes
+// query head j of the group at the channels 16 kg + 4 r + kq and leaves, for the K-pass lane of the same index,
+// 2 KG words of q (packed fp16 pairs r = 0,1 / 2,3 per channel group) and 4 words of level bits (bit 4 kg + r):
+// this head's level is 1 / is 2, and -- OR-ed over the heads of the group -- the mid / last plane row of the
+// channel is fetched.  grid (B * Hkv), 64 threads.
+template <int D, bool REF>
+__global__ __launch_bounds__(64) void mfma_k_prepare_kernel(const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q,
+                                                           const unsigned short *__restrict__ k_new, u32 *__restrict__ prep,
+                                                           uint8_t *__restrict__ levels_out, StepGeom geo) {
+    constexpr int KG = D / 16;
+    const int lane = threadIdx.x;
+    const int bh_kv = blockIdx.x, b = bh_kv / geo.Hkv, hkv = bh_kv - b * geo.Hkv;
+    const int G = geo.G;
+    const int64_t bh0 = (int64_t)b * geo.Hq + hkv * G;
+    const int j = lane & 15, kq = lane >> 4;
+    const bool head = j < G;
+    u32 *out = prep + ((int64_t)bh_kv * 64 + lane) * (2 * KG + 4);
+    u32 lv1 = 0, lv2 = 0;
+    u32 esum[KG][4];
+    u32 mx = 0;
+#pragma unroll
+    for (int kg = 0; kg < KG; ++kg) {
+        u32 qb[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int c = 16 * kg + 4 * r + kq;
+            qb[r] = head ? (u32)q[(bh0 + j) * D + c] : 0u;
+            // column max including the token appended by this step
+            const u32 cm = max((u32)kcm[(int64_t)bh_kv * D + c], exp_field(k_new[(int64_t)bh_kv * D + c]));
+            esum[kg][r] = (exp_field(qb[r]) + cm) & 0xffu;
+            mx = max(mx, esum[kg][r]);
+        }
+        out[2 * kg] = qb[0] | (qb[1] << 16);
+        out[2 * kg + 1] = qb[2] | (qb[3] << 16);
+    }
+    mx = max(mx, (u32)__shfl_xor((int)mx, 16, 64));
+    mx = max(mx, (u32)__shfl_xor((int)mx, 32, 64));
+#pragma unroll
+    for (int kg = 0; kg < KG; ++kg)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)esum[kg][r]);
+            if (head) {
+                lv1 |= (lv == 1 ? 1u : 0u) << (4 * kg + r);
+                lv2 |= (lv == 2 ? 1u : 0u) << (4 * kg + r);
+                if (levels_out != nullptr) levels_out[(bh0 + j) * D + 16 * kg + 4 * r + kq] = (uint8_t)lv;
+            }
+        }
+    // a plane row is fetched if any head of the group reads it: OR over the 16 lanes that share kq
+    u32 need_mid = head ? ~lv2 : 0u;
+    u32 need_last = head ? ~(lv1 | lv2) : 0u;
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) {
+        need_mid |= (u32)__shfl_xor((int)need_mid, m, 64);
+        need_last |= (u32)__shfl_xor((int)need_last, m, 64);
+    }
+    out[2 * KG] = lv1;
+    out[2 * KG + 1] = lv2;
+    out[2 * KG + 2] = need_mid;
+    out[2 * KG + 3] = need_last;
+}
+
+template <int D, bool REF, int SL, int AHEAD>
+__global__ __launch_bounds__(256) void mfma_k_pass_kernel(
+    const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
+    const u32 *__restrict__ prep, unsigned short *__restrict__ scores, StepGeom geo, int tasks_per_wave, float scale,
+    u32 scores_bytes) {
+    constexpr int CB = 64;
+    constexpr int KG = D / 16;     // channel groups
+    constexpr int PB = 64 / SL;    // pieces (token sets) per block
+    constexpr int NBT = 16 / PB;   // blocks per task
+    static_assert(KG % (AHEAD + 1) == 0, "the tile ring is rotated by unrolling");
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int chunk = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z;
+    const int G = geo.G;
+    const int bh_kv = b * geo.Hkv + hkv;
+    const int64_t bh0 = (int64_t)b * geo.Hq + hkv * G;
+    int R, nrest;
+    seq_state(geo, b, R, nrest);
+    const int n_blocks = R / CB;
+    const int n_tasks = (n_blocks + NBT - 1) / NBT;
+    const int first_task = (chunk * 4 + wave) * tasks_per_wave;
+    const int end_task = min(first_task + tasks_per_wave, n_tasks);
+    if (first_task >= n_tasks) return;     // past the end of this sequence (no barrier in this kernel)
+
+    const int64_t plane_off = (int64_t)bh_kv * geo.n_max_blocks * (D * (CB / 2));
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(first_8 + plane_off * 2, (u32)n_blocks * (D * CB));
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(mid_4 + plane_off, (u32)n_blocks * (D * CB / 2));
+    const __amdgpu_buffer_rsrc_t rL = make_rsrc(last_4 + plane_off, (u32)n_blocks * (D * CB / 2));
+    const __amdgpu_buffer_rsrc_t rS = make_rsrc(scores, scores_bytes);
+    const int blk_sel = (lane & 15) / PB;
+
+    // what mfma_k_prepare_kernel left for this lane
+    const int j = lane & 15;
+    const bool head = j < G;
+    u32 qp[KG][2];
+    u32 lv1, lv2, need_mid, need_last;
+    {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(prep + ((int64_t)bh_kv * 64 + lane) * (2 * KG + 4));
+#pragma unroll
+        for (int i = 0; i < KG / 2; ++i) {
+            const u32x4 v = src[i];
+            qp[2 * i][0] = v.x; qp[2 * i][1] = v.y; qp[2 * i + 1][0] = v.z; qp[2 * i + 1][1] = v.w;
+        }
+        const u32x4 v = src[KG / 2];
+        lv1 = v.x; lv2 = v.y; need_mid = v.z; need_last = v.w;
+    }
+
+    // Software pipeline: AHEAD channel-group tiles in flight while one is multiplied.
+    KTaskTile<SL> t[AHEAD + 1];
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) kt_issue<D, SL>(t[i], rH, rM, rL, first_task * NBT + blk_sel, i, need_mid, need_last);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int task = first_task; task < end_task; ++task) {
+        f32x4 acc[SL];
+#pragma unroll
+        for (int i = 0; i < SL; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        // the masks derived from these words are cheap to rebuild and would otherwise be kept in ~100 registers
+        // across the loop: hide their loop invariance from the compiler
+        asm volatile("" : "+v"(need_mid), "+v"(need_last), "+v"(lv1), "+v"(lv2));
+        const int blk = task * NBT + blk_sel;
+        const int next_blk = (task + 1 < end_task ? task + 1 : n_tasks) * NBT + blk_sel;   // past the end: nothing is fetched
+#pragma unroll
+        for (int kg = 0; kg < KG; ++kg) {
+            const int kn = kg + AHEAD;
+            kt_issue<D, SL>(t[kn % (AHEAD + 1)], rH, rM, rL, kn < KG ? blk : next_blk, kn % KG, need_mid, need_last);
+            __builtin_amdgcn_sched_barrier(0);
+            const u32 m1a = ((lv1 >> (4 * kg)) & 1u ? 0xFFFFu : 0u) | ((lv1 >> (4 * kg + 1)) & 1u ? 0xFFFF0000u : 0u);
+            const u32 m1b = ((lv1 >> (4 * kg + 2)) & 1u ? 0xFFFFu : 0u) | ((lv1 >> (4 * kg + 3)) & 1u ? 0xFFFF0000u : 0u);
+            const u32 m2a = ((lv2 >> (4 * kg)) & 1u ? 0xFFFFu : 0u) | ((lv2 >> (4 * kg + 1)) & 1u ? 0xFFFF0000u : 0u);
+            const u32 m2b = ((lv2 >> (4 * kg + 2)) & 1u ? 0xFFFFu : 0u) | ((lv2 >> (4 * kg + 3)) & 1u ? 0xFFFF0000u : 0u);
+            const u32 na = qp[kg][0] ^ 0x80008000u, nb = qp[kg][1] ^ 0x80008000u;     // -q
+            kt_compute<REF, SL>(acc, t[kg % (AHEAD + 1)], kg, need_mid, need_last, as_f16x4(qp[kg][0], qp[kg][1]),
+                                as_f16x4(na & m1a, nb & m1b), as_f16x4(na & m2a, nb & m2b));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // lane (j, ig): acc[s][r] = score of slot s of token set 4 ig + r for query head j
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int ts = 4 * (lane >> 4) + r;
+            const int out_blk = task * NBT + ts / PB;
+            const bool store = head && out_blk < n_blocks;
+            u32 pk[SL / 2];
+#pragma unroll
+            for (int sl = 0; sl < SL; sl += 2)
+                pk[sl >> 1] = (u32)float_to_half_bits(acc[sl][r] * scale) | ((u32)float_to_half_bits(acc[sl + 1][r] * scale) << 16);
+            const int off = store ? (int)(((bh0 + j) * geo.row_stride + out_blk * CB + (ts % PB) * SL) * 2) : kSkip;
+            // device scope: the workgroup that runs the softmax for this (batch, head) may sit on another XCD
+            if constexpr (SL == 4) {
+                __builtin_amdgcn_raw_buffer_store_b64((u32x2){pk[0], pk[1]}, rS, off, 0, kDeviceScope);
+            } else {
+                __builtin_amdgcn_raw_buffer_store_b128((u32x4){pk[0], pk[1], pk[2], pk[3]}, rS, off, 0, kDeviceScope);
+                if constexpr (SL == 16)
+                    __builtin_amdgcn_raw_buffer_store_b128((u32x4){pk[4], pk[5], pk[6], pk[7]}, rS, store ? off + 16 : kSkip, 0,
+                                                           kDeviceScope);
+            }
+        }
+    }
+}
+
+// ---- host ------------------------------------------------------------------------------------------
+template <int D>
+int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *kcm,
+                       const unsigned short *q, const unsigned short *k_new, unsigned short *scores,
+                       uint8_t *levels_out, u32 *prep, const StepGeom &geo, int B, int n_blocks, bool ref, float scale,
+                       hipStream_t st) {
+    int sl = 8;
+    if (const char *e = getenv("AKV_TUNE_K_SL")) sl = atoi(e) == 16 ? 16 : (atoi(e) == 4 ? 4 : 8);
+    const int nbt = sl / 4;
+    const int n_tasks = (n_blocks + nbt - 1) / nbt;
+    int tpw = 1;
+    while (tpw < 8 && (int64_t)B * geo.Hkv * ((n_tasks + 8 * tpw - 1) / (8 * tpw)) * 4 >= 8192) tpw *= 2;
+    if (const char *e = getenv("AKV_TUNE_K_TPW")) tpw = atoi(e) > 0 ? atoi(e) : tpw;
+    const int64_t scores_bytes = (int64_t)B * geo.Hq * geo.row_stride * 2;
+    if (scores_bytes >= ((int64_t)1 << 31)) {
+        set_error("decode_step: score rows of %lld bytes exceed the 2 GiB the grouped K pass addresses", (long long)scores_bytes);
+        return AKV_ERR_INVALID;
+    }
+    if (ref)
+        hipLaunchKernelGGL((mfma_k_prepare_kernel<D, true>), dim3(B * geo.Hkv), dim3(64), 0, st, kcm, q, k_new, prep, levels_out, geo);
+    else
+        hipLaunchKernelGGL((mfma_k_prepare_kernel<D, false>), dim3(B * geo.Hkv), dim3(64), 0, st, kcm, q, k_new, prep, levels_out, geo);
+    int rc = check_launch("decode_step(mfma k_prepare)");
+    if (rc != AKV_OK) return rc;
+    dim3 grid((n_tasks + 4 * tpw - 1) / (4 * tpw), geo.Hkv, B);
+#define AKV_MK(RF, SLL, AH)                                                                                          \
+    hipLaunchKernelGGL((mfma_k_pass_kernel<D, RF, SLL, AH>), grid, dim3(256), 0, st, f8, m4, l4, prep, scores, geo, tpw, \
+                       scale, (u32)scores_bytes)
+    int ahead = 3;
+    if (const char *e = getenv("AKV_TUNE_K_AHEAD")) ahead = atoi(e);
+    constexpr int DEEP = (D / 16) % 8 == 0 ? 7 : 3;
+    if (sl == 16) { if (ref) AKV_MK(true, 16, 1); else AKV_MK(false, 16, 1); }
+    else if (sl == 8 && ahead == 7) { if (ref) AKV_MK(true, 8, DEEP); else AKV_MK(false, 8, DEEP); }
+    else if (sl == 8) { if (ref) AKV_MK(true, 8, 3); else AKV_MK(false, 8, 3); }
+    else if (ahead == 7) { if (ref) AKV_MK(true, 4, DEEP); else AKV_MK(false, 4, DEEP); }
+    else { if (ref) AKV_MK(true, 4, 3); else AKV_MK(false, 4, 3); }
+#undef AKV_MK
+    return check_launch("decode_step(mfma k_pass)");
+}
+
+#define AKV_INST(DD)                                                                                                  \
+    template int launch_mfma_k_pass<DD>(const uint8_t *, const uint8_t *, const uint8_t *, const uint8_t *,           \
+                                        const unsigned short *, const unsigned short *, unsigned short *, uint8_t *, \
+                                        u32 *, const StepGeom &, int, int, bool, float, hipStream_t);
+AKV_INST(64)
+AKV_INST(128)
+AKV_INST(256)
+#undef AKV_INST
+
+}  // namespace akv

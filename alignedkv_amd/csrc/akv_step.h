@@ -54,4 +54,14 @@ int launch_group_v_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4,
                         const uint8_t *amin, float *partial, uint8_t *levels_out, int levels_stride, uint8_t *amin_out,
                         const StepGeom &geo, int B, const VPlan &p, bool ref, hipStream_t st);
 
+
+// Grouped-query passes on the matrix cores (akv_gqa_mfma.hip): 2 to 16 query heads per KV head.
+template <int D>
+int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *kcm,
+                       const unsigned short *q, const unsigned short *k_new, unsigned short *scores,
+                       uint8_t *levels_out, u32 *prep, const StepGeom &geo, int B, int n_blocks, bool ref, float scale,
+                       hipStream_t st);
+// words of set-up data per (batch, KV head) that launch_mfma_k_pass needs in `prep`
+inline size_t mfma_k_prep_words(int D) { return (size_t)64 * (2 * (D / 16) + 4); }
+
 }  // namespace akv

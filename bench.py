@@ -49,6 +49,8 @@ def parse():
     ap.add_argument("--workload", default="c2", choices=["c2", "c3"],
                     help="c2: the headline configuration (shape flags apply); c3: grouped-query heads (32 over 8), batch 32, "
                          "lengths uniform in [2048, 8192] -- an extra line, not the headline metric")
+    ap.add_argument("--c3-q-heads", type=int, default=32, help="c3 only: query heads over the 8 KV heads")
+    ap.add_argument("--c3-len", type=int, default=0, help="c3 only: one length for every sequence instead of U[2048, 8192]")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB copy kernel (known size, for scaling hardware byte counters)")
     return ap.parse_args()
@@ -195,9 +197,11 @@ def bench_c3(a):
     import alignedkv_amd
     from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
     lib = alignedkv_amd.load_library()
-    B, Hq, Hkv, D, cb = 32, 32, 8, 128, 64
+    B, Hq, Hkv, D, cb = 32, a.c3_q_heads, 8, 128, 64
     Lmax = 8192 + cb
     lens = np.random.default_rng(a.seed + 3).integers(2048, 8193, B)
+    if a.c3_len:
+        lens[:] = a.c3_len
     cache = RaggedGQACache(a.layers, B, Lmax, Hq, Hkv, D)
     for layer in range(a.layers):
         for b in range(B):
