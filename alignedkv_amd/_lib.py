@@ -31,6 +31,7 @@ SIGNATURES = {
     "akv_profile_enable": (c_int, [_I]),
     "akv_copy_probe": (c_int, [_P, _P, c_size_t, _P]),
     "akv_profile_read": (c_int, [_P]),
+    "akv_profile_read_empty": (c_int, [_P]),
     "akv_decode_step_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "akv_decode_step": (c_int, [_P] * 14 + [_I] + [_P] * 3 + [_I, _P, c_size_t] + [_P] * 3 + [_I] * 12 + [_P]),
 }

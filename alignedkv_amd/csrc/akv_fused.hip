@@ -28,7 +28,7 @@ int launch_v_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8
 // Optional per-phase timing of the fused step (benchmark aid): when enabled, events are recorded on the
 // step's stream around the K pass, the middle kernel, the V pass and the combine kernel.
 static bool g_profile = false;
-static hipEvent_t g_ev[5];
+static hipEvent_t g_ev[7];   // 0..4 around the four phases, 5 and 6 back to back (interval of an empty phase)
 static bool g_ev_ready = false;
 static inline void mark(int i, hipStream_t st) {
     if (g_profile) (void)hipEventRecord(g_ev[i], st);
@@ -812,6 +812,8 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         mark(2, st);
         mark(3, st);
         mark(4, st);
+        mark(5, st);
+        mark(6, st);
         return check_launch("decode_step(mono)");
     }
     // grouped-query heads: one workgroup per plane chunk serves 2 or 4 query heads (AKV_TUNE_GROUP: see group_heads)
@@ -873,6 +875,8 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     hipLaunchKernelGGL(fused_combine_kernel, dim3(B * Hq), dim3(D < 256 ? D : 256), 0, st, partial, otail,
                        reinterpret_cast<unsigned short *>(out), D, p.n_chunks, seq_lens, Hq);
     mark(4, st);
+    mark(5, st);
+    mark(6, st);
     return check_launch("decode_step(combine)");
 }
 
@@ -882,7 +886,7 @@ using namespace akv;
 
 extern "C" int akv_profile_enable(int enable) {
     if (enable && !g_ev_ready) {
-        for (int i = 0; i < 5; ++i) {
+        for (int i = 0; i < 7; ++i) {
             if (hipEventCreate(&g_ev[i]) != hipSuccess) {
                 set_error("profile_enable: hipEventCreate failed");
                 return AKV_ERR_LAUNCH;
@@ -905,6 +909,15 @@ extern "C" int akv_profile_read(float *phase_ms) {
             set_error("profile_read: hipEventElapsedTime failed");
             return AKV_ERR_LAUNCH;
         }
+    }
+    return AKV_OK;
+}
+
+extern "C" int akv_profile_read_empty(float *empty_ms) {
+    AKV_REQUIRE(empty_ms != nullptr && g_ev_ready, "profile_read_empty: profiling was never enabled");
+    if (hipEventSynchronize(g_ev[6]) != hipSuccess || hipEventElapsedTime(empty_ms, g_ev[5], g_ev[6]) != hipSuccess) {
+        set_error("profile_read_empty: no completed step to read");
+        return AKV_ERR_LAUNCH;
     }
     return AKV_OK;
 }

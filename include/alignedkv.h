@@ -196,6 +196,9 @@ AKV_API int akv_profile_enable(int enable);
 /* Plain device copy of `bytes` bytes (multiple of 16): the known-size kernel hardware byte counters are scaled against. */
 AKV_API int akv_copy_probe(void *dst, const void *src, size_t bytes, akv_stream_t stream);
 AKV_API int akv_profile_read(float *phase_ms /* [4] */);
+/* Interval between two events recorded back to back after the last step: what an event pair measures around
+ * nothing.  Subtract it from a phase of akv_profile_read to get the kernel's own duration. */
+AKV_API int akv_profile_read_empty(float *empty_ms /* [1] */);
 
 #ifdef __cplusplus
 }
