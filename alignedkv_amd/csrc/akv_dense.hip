@@ -65,13 +65,15 @@ __global__ __launch_bounds__(256) void dense_k_pass_kernel(const unsigned short 
     }
     const __amdgpu_buffer_rsrc_t rK = make_rsrc(k_cache + (int64_t)bh * max_seq_len * D, (u32)n_tokens * D * 2);
     unsigned short *s_row = scores + (int64_t)bh * row_stride;
-    for (int base = t_begin; base < t_end; base += 32) {
-        u32x4 kv[8];
+    // software pipeline: the 8 loads of the next 32 tokens are in flight while the current ones are multiplied
+    auto issue = [&](u32x4 *kv, int base) {
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int t = base + u * 4 + tl;
             kv[u] = __builtin_amdgcn_raw_buffer_load_b128(rK, t < t_end ? t * (D * 2) + cl * 16 : kSkip, 0, 0);
         }
+    };
+    auto finish = [&](const u32x4 *kv, int base) {
         float acc[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) acc[u] = dot8(kv[u], qf, 0.f);
@@ -85,6 +87,19 @@ __global__ __launch_bounds__(256) void dense_k_pass_kernel(const unsigned short 
         // fp16 matmul result, then the fp16 division by sqrt(D) (model/Llama_AlignedKV.py:130)
         if ((lane & 8) == 0 && t < t_end)
             s_row[t] = float_to_half_bits(half_bits_to_float(float_to_half_bits(acc[0])) / sqrt_d);
+    };
+    u32x4 ka[8], kb[8];
+    issue(ka, t_begin);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int base = t_begin; base < t_end; base += 64) {
+        issue(kb, base + 32);
+        __builtin_amdgcn_sched_barrier(0);
+        finish(ka, base);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(ka, base + 64);
+        __builtin_amdgcn_sched_barrier(0);
+        finish(kb, base + 32);
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -122,15 +137,62 @@ __global__ __launch_bounds__(256) void dense_middle_kernel(DenseMiddleArgs a) {
         }
     }
     __syncthreads();
-    const int total = n + 1;
-    float m = -INFINITY;
-    for (int t = tid; t < total; t += 256) m = fmaxf(m, t < n ? half_bits_to_float(srow[t]) : s_new);
+    // scores of the cached tokens as 16-byte vectors; rows of up to 8192 tokens stay in registers between the passes
+    constexpr int VPT = 4;
+    const int nvec = n >> 3;
+    const bool in_regs = nvec <= 256 * VPT;
+    u32x4 sv[VPT];
+    auto vec = [&](int v) -> u32x4 { return in_regs ? sv[v] : *reinterpret_cast<const u32x4 *>(srow + (tid + 256 * v) * 8); };
+    const int nv = in_regs ? VPT : (nvec + 255) / 256;
+    if (in_regs) {
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int i = tid + 256 * v;
+            sv[v] = i < nvec ? *reinterpret_cast<const u32x4 *>(srow + i * 8) : (u32x4){0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u, 0xfc00fc00u};
+        }
+    }
+    auto each = [&](auto &&f) {   // f(vector index, 8 floats) over this thread's vectors
+        if (in_regs) {
+#pragma unroll
+            for (int v = 0; v < VPT; ++v) {
+                const int i = tid + 256 * v;
+                if (i < nvec) f(i, sv[v]);
+            }
+        } else {
+            for (int v = 0; v < nv; ++v) {
+                const int i = tid + 256 * v;
+                if (i < nvec) f(i, *reinterpret_cast<const u32x4 *>(srow + i * 8));
+            }
+        }
+    };
+    (void)vec;
+    // the tokens after the last whole vector and the new one: scalar
+    const int t_tail = (nvec << 3) + tid;
+    const float x_tail = t_tail < n ? half_bits_to_float(srow[t_tail]) : (t_tail == n ? s_new : -INFINITY);
+    float m = x_tail;
+    each([&](int, const u32x4 w) {
+        const u32 ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) m = fmaxf(m, fmaxf(lo_half_to_float(ww[j]), hi_half_to_float(ww[j])));
+    });
     m = d_block_reduce(m, true, red);
-    float sum = 0.f;
-    for (int t = tid; t < total; t += 256) sum += expf((t < n ? half_bits_to_float(srow[t]) : s_new) - m);
+    float sum = t_tail <= n ? expf(x_tail - m) : 0.f;
+    each([&](int, const u32x4 w) {
+        const u32 ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) sum += expf(lo_half_to_float(ww[j]) - m) + expf(hi_half_to_float(ww[j]) - m);
+    });
     sum = d_block_reduce(sum, false, red);
-    for (int t = tid; t < total; t += 256)
-        prow[t] = float_to_half_bits(expf((t < n ? half_bits_to_float(srow[t]) : s_new) - m) / sum);
+    each([&](int i, const u32x4 w) {
+        const u32 ww[4] = {w.x, w.y, w.z, w.w};
+        u32 o[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            o[j] = (u32)float_to_half_bits(expf(lo_half_to_float(ww[j]) - m) / sum) |
+                   ((u32)float_to_half_bits(expf(hi_half_to_float(ww[j]) - m) / sum) << 16);
+        *reinterpret_cast<u32x4 *>(prow + i * 8) = (u32x4){o[0], o[1], o[2], o[3]};
+    });
+    if (t_tail <= n) prow[t_tail] = float_to_half_bits(expf(x_tail - m) / sum);
 }
 
 // V pass, head_dim 128: lane = 8 channels of one token, 4 tokens per wave-wide load, 8 loads in flight.
@@ -152,26 +214,42 @@ __global__ __launch_bounds__(256) void dense_v_pass_kernel(const unsigned short 
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-    for (int base = t_begin; base < t_end; base += 32) {
-        u32x4 vv[8];
-        float sf[8];
+    auto issue = [&](u32x4 *vv, u32 *sb, int base) {
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int t = base + u * 4 + tl;
             vv[u] = __builtin_amdgcn_raw_buffer_load_b128(rV, t < t_end ? t * (D * 2) + cl * 16 : kSkip, 0, 0);
-            sf[u] = half_bits_to_float((u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < t_end ? t * 2 : kSkip, 0, 0));
+            sb[u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < t_end ? t * 2 : kSkip, 0, 0);
         }
+    };
+    auto finish = [&](const u32x4 *vv, const u32 *sb) {
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-            acc[0] = fmaf(lo_half_to_float(vv[u].x), sf[u], acc[0]);
-            acc[1] = fmaf(hi_half_to_float(vv[u].x), sf[u], acc[1]);
-            acc[2] = fmaf(lo_half_to_float(vv[u].y), sf[u], acc[2]);
-            acc[3] = fmaf(hi_half_to_float(vv[u].y), sf[u], acc[3]);
-            acc[4] = fmaf(lo_half_to_float(vv[u].z), sf[u], acc[4]);
-            acc[5] = fmaf(hi_half_to_float(vv[u].z), sf[u], acc[5]);
-            acc[6] = fmaf(lo_half_to_float(vv[u].w), sf[u], acc[6]);
-            acc[7] = fmaf(hi_half_to_float(vv[u].w), sf[u], acc[7]);
+            const float sf = half_bits_to_float(sb[u]);
+            acc[0] = fmaf(lo_half_to_float(vv[u].x), sf, acc[0]);
+            acc[1] = fmaf(hi_half_to_float(vv[u].x), sf, acc[1]);
+            acc[2] = fmaf(lo_half_to_float(vv[u].y), sf, acc[2]);
+            acc[3] = fmaf(hi_half_to_float(vv[u].y), sf, acc[3]);
+            acc[4] = fmaf(lo_half_to_float(vv[u].z), sf, acc[4]);
+            acc[5] = fmaf(hi_half_to_float(vv[u].z), sf, acc[5]);
+            acc[6] = fmaf(lo_half_to_float(vv[u].w), sf, acc[6]);
+            acc[7] = fmaf(hi_half_to_float(vv[u].w), sf, acc[7]);
         }
+    };
+    // software pipeline: the next 32 token rows are in flight while the current ones are multiplied
+    u32x4 va[8], vb[8];
+    u32 sa[8], sbb[8];
+    issue(va, sa, t_begin);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int base = t_begin; base < t_end; base += 64) {
+        issue(vb, sbb, base + 32);
+        __builtin_amdgcn_sched_barrier(0);
+        finish(va, sa);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(va, sa, base + 64);
+        __builtin_amdgcn_sched_barrier(0);
+        finish(vb, sbb);
+        __builtin_amdgcn_sched_barrier(0);
     }
     // fold the 4 token lanes (lane bits 4, 5): 8 sums -> 2 per lane
     int ch = cl * 8;
@@ -223,7 +301,9 @@ extern "C" int akv_dense_decode_step(uint8_t *k_cache, uint8_t *v_cache, const u
     AKV_REQUIRE(head_dim == 128, "dense_decode_step: the dense baseline is written for head_dim 128 (got %d)", head_dim);
     AKV_REQUIRE(bsz > 0 && n_heads > 0 && bsz <= 65535 && n_heads <= 65535, "dense_decode_step: bad bsz/heads");
     AKV_REQUIRE(cur_len >= 0 && cur_len + 1 <= max_seq_len, "dense_decode_step: cache full (%d of %d)", cur_len, max_seq_len);
-    AKV_REQUIRE(row_stride >= cur_len + 1, "dense_decode_step: row_stride %d shorter than %d", row_stride, cur_len + 1);
+    AKV_REQUIRE(row_stride >= cur_len + 1 && row_stride % 8 == 0 && ((uintptr_t)scores & 15) == 0 && ((uintptr_t)probs & 15) == 0,
+                "dense_decode_step: row_stride %d must be a multiple of 8 and >= %d, scores/probs 16-byte aligned", row_stride,
+                cur_len + 1);
     AKV_REQUIRE((int64_t)max_seq_len * head_dim * 2 < (int64_t)1 << 31, "dense_decode_step: one (batch, head) slice must stay below 2 GiB");
     AKV_REQUIRE(workspace_bytes >= akv_dense_decode_step_workspace_bytes(bsz, n_heads, head_dim, max_seq_len),
                 "dense_decode_step: workspace too small");
