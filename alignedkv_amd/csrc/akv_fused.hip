@@ -62,6 +62,58 @@ __global__ void fused_persist_kernel(const unsigned short *__restrict__ k_new, c
     }
 }
 
+// Task maps of a step with per-sequence lengths (see step_block): for each of the two streaming passes the
+// workgroups that have tokens to read, ordered by (batch, head index, chunk) with the chunk fastest, then kNoTask
+// up to the size of the grid; v_chunks[b] = V-pass chunks of sequence b, for the combine kernel (the lengths
+// themselves advance while it runs).  One workgroup of 256 threads; scratch: 2 * 257 ints of LDS.
+struct TaskMaps {
+    u32 *map_k, *map_v;      // null: no map for that pass
+    int *v_chunks;
+    PassShape k, v;
+};
+
+__device__ __forceinline__ void build_task_map(const StepGeom &geo, u32 *map, const PassShape &sh, int B, int *v_chunks,
+                                               int *part) {
+    const int tid = threadIdx.x;
+    const int per = (B + 255) / 256, b0 = tid * per, b1 = min(b0 + per, B);
+    int mine = 0;
+    for (int b = b0; b < b1; ++b) {
+        int R, nrest;
+        seq_state(geo, b, R, nrest);
+        const int n = (R + sh.tokens_per_wg - 1) / sh.tokens_per_wg;
+        if (v_chunks != nullptr) v_chunks[b] = n;
+        mine += n * sh.grid_y;
+    }
+    part[tid] = mine;
+    __syncthreads();
+    if (tid == 0) {
+        int run = 0;
+        for (int i = 0; i < 256; ++i) {
+            const int v = part[i];
+            part[i] = run;
+            run += v;
+        }
+        part[256] = run;
+    }
+    __syncthreads();
+    int at = part[tid];
+    for (int b = b0; b < b1; ++b) {
+        int R, nrest;
+        seq_state(geo, b, R, nrest);
+        const int n = (R + sh.tokens_per_wg - 1) / sh.tokens_per_wg;
+        for (int y = 0; y < sh.grid_y; ++y)
+            for (int x = 0; x < n; ++x) map[at++] = pack_task(x, y, b);
+    }
+    const int total = part[256], grid = sh.grid_x * sh.grid_y * B;
+    for (int i = total + tid; i < grid; i += 256) map[i] = kNoTask;
+    __syncthreads();
+}
+
+__device__ __forceinline__ void build_task_maps(const StepGeom &geo, const TaskMaps &m, int B, int *part) {
+    if (m.map_k != nullptr) build_task_map(geo, m.map_k, m.k, B, nullptr, part);
+    if (m.map_v != nullptr) build_task_map(geo, m.map_v, m.v, B, m.v_chunks, part);
+}
+
 // Ragged mode, first kernel of every step: append the token of every sequence to its rest buffer, update the
 // column maxima and, for the sequences whose rest buffer is full with it, write the 64-token block into the
 // planes (same bytes as k_save_blocks_kernel / v_save_vec8_kernel).  grid (B*Hkv), 256 threads.
@@ -72,9 +124,14 @@ __global__ __launch_bounds__(256) void fused_pre_kernel(uint8_t *__restrict__ kf
                                                         const unsigned short *__restrict__ k_new,
                                                         const unsigned short *__restrict__ v_new,
                                                         unsigned short *__restrict__ restk, unsigned short *__restrict__ restv,
-                                                        uint8_t *__restrict__ kcm, uint8_t *__restrict__ vcm, StepGeom geo) {
+                                                        uint8_t *__restrict__ kcm, uint8_t *__restrict__ vcm, StepGeom geo,
+                                                        TaskMaps maps, int B) {
     constexpr int CB = 64;
     __shared__ unsigned short tile[CB][D + 2];
+    if ((int)blockIdx.x == B * geo.Hkv) {   // the extra workgroup: task maps of the K and the V pass
+        build_task_maps(geo, maps, B, reinterpret_cast<int *>(&tile[0][0]));
+        return;
+    }
     const int bh = blockIdx.x, b = bh / geo.Hkv, h = bh - b * geo.Hkv;
     const int cur = geo.seq_lens[b];
     const int slot = cur % CB;
@@ -164,9 +221,9 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     constexpr int CB = 64;
     constexpr int NG = D / 16;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    int chunk, gq;
-    decode_group_block(geo.G, chunk, gq);
-    const int hkv = blockIdx.y, b = blockIdx.z;
+    int bx, hkv, b, chunk, gq;
+    if (!step_block(geo, bx, hkv, b)) return;
+    decode_group_block(geo.G, bx, chunk, gq);
     const int bh_kv = b * geo.Hkv + hkv, bh = b * geo.Hq + hkv * geo.G + gq;
     int R, nrest;
     seq_state(geo, b, R, nrest);
@@ -677,9 +734,9 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
     int tokens_per_wave, int n_chunks) {
     __shared__ float wave_part[4][D];
     const int wave = threadIdx.x >> 6;
-    int chunk, gq;
-    decode_group_block(geo.G, chunk, gq);
-    const int hkv = blockIdx.y, b = blockIdx.z;
+    int bx, hkv, b, chunk, gq;
+    if (!step_block(geo, bx, hkv, b)) return;
+    decode_group_block(geo.G, bx, chunk, gq);
     const int bh_kv = b * geo.Hkv + hkv, bh = b * geo.Hq + hkv * geo.G + gq;
     if (chunk >= n_chunks) return;    // padding of the grid (whole workgroup)
     int n_tokens, nrest;
@@ -702,20 +759,23 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
 
 // grid (B*H), D threads: out = fp16(fp16(sum of partials) + tail), the fp16 `o += tail` of the reference.
 __global__ void fused_combine_kernel(const float *__restrict__ partial, const unsigned short *__restrict__ otail,
-                                     unsigned short *__restrict__ out, int D, int n_chunks, int *seq_lens_rw, int Hq) {
+                                     unsigned short *__restrict__ out, int D, int n_chunks, int *seq_lens_rw, int Hq,
+                                     const int *__restrict__ v_chunks) {
     const int bh = blockIdx.x;
+    // with a task map only the chunks of this sequence were written
+    const int n_sum = v_chunks != nullptr ? v_chunks[bh / Hq] : n_chunks;
     // last kernel of the step: the sequence lengths kept on the device advance here
     if (seq_lens_rw != nullptr && threadIdx.x == 0 && bh % Hq == 0) seq_lens_rw[bh / Hq] += 1;
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
         float acc = 0.f;
-        for (int c = 0; c < n_chunks; ++c) acc += partial[((int64_t)bh * n_chunks + c) * D + d];
+        for (int c = 0; c < n_sum; ++c) acc += partial[((int64_t)bh * n_chunks + c) * D + d];
         const float o16 = half_bits_to_float(float_to_half_bits(acc));
         out[(int64_t)bh * D + d] = float_to_half_bits(o16 + half_bits_to_float(otail[(int64_t)bh * D + d]));
     }
 }
 
 struct StepLayout {
-    size_t toe, amin, otail, partial, prep, total;
+    size_t toe, amin, otail, partial, prep, map_k, map_v, v_chunks, total;
 };
 
 static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
@@ -730,7 +790,11 @@ static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
     l.otail = l.amin + up((size_t)B * H);
     l.partial = l.otail + up((size_t)B * H * D * 2);
     l.prep = l.partial + up((size_t)B * H * max_chunks * D * sizeof(float));
-    l.total = l.prep + up((size_t)B * H * mfma_k_prep_words(D) * sizeof(u32));   // B * Hkv <= B * H rows are used
+    l.map_k = l.prep + up((size_t)B * H * mfma_k_prep_words(D) * sizeof(u32));   // B * Hkv <= B * H rows are used
+    // task maps: a pass has at most B * H * (max_chunks + 1) workgroups
+    l.map_v = l.map_k + up((size_t)B * H * (max_chunks + 1) * sizeof(u32));
+    l.v_chunks = l.map_v + up((size_t)B * H * (max_chunks + 1) * sizeof(u32));
+    l.total = l.v_chunks + up((size_t)B * sizeof(int));
     return l;
 }
 
@@ -758,13 +822,59 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     geo.Hq = Hq; geo.Hkv = Hkv; geo.G = Hq / Hkv;
     geo.cb = cb; geo.max_seq_len = max_seq_len; geo.n_max_blocks = n_max_blocks; geo.row_stride = row_stride;
     geo.cur_len = cur_len; geo.seq_lens = seq_lens;
+    geo.task_map = nullptr;
+
+    // flushed tokens after the append: exact for uniform lengths, an upper bound for ragged ones
+    const int R = (cur_len + 1) / cb * cb;
+    const int n_blocks = R / cb;
+    // the kernel multiplies by the fp16-rounded scale (extension/csrc/K_cache.cu:306)
+    const float scale = __half2float(__float2half_rn(1.0f / sqrtf((float)D)));
+    // grouped-query heads: one workgroup per plane chunk serves 2 or 4 query heads (AKV_TUNE_GROUP: see group_heads),
+    // or up to 16 on the matrix cores (K pass)
+    const bool grouped = group_heads(geo.G) > 1;
+    bool matrix = geo.G >= 2 && geo.G <= 16;
+    if (const char *e = getenv("AKV_TUNE_MFMA")) matrix = matrix && atoi(e) != 0;
+    const int bpw = k_blocks_per_wave(B, Hq, n_blocks);
+    const VPlan p = v_plan(B, grouped ? Hq / group_heads(geo.G) : Hq, D, R);
+    // launch shapes of the two streaming passes
+    PassShape ks = {0, 0, 0}, vs = {0, 0, 0};
+    if (n_blocks > 0) {
+        if (matrix) {
+            int rc = launch_mfma_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, nullptr, geo, B, n_blocks, ref, scale,
+                                           st, &ks);
+            if (rc != AKV_OK) return rc;
+        } else if (grouped) {
+            int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo, B, n_blocks, ref, scale, st, &ks);
+            if (rc != AKV_OK) return rc;
+        } else {
+            ks = PassShape{group_grid_x((n_blocks + 4 * bpw - 1) / (4 * bpw), geo.G), Hkv, 4 * bpw * cb};
+        }
+        vs = PassShape{grouped ? p.n_chunks : group_grid_x(p.n_chunks, geo.G), grouped ? Hkv * (geo.G / group_heads(geo.G)) : Hkv,
+                       p.chunk_tokens};
+    }
+    // task maps (per-sequence lengths): not for the swizzled grids of ungrouped multi-query heads
+    const bool mapped = ragged && n_blocks > 0 && (geo.G == 1 || grouped || matrix) && task_map_fits(ks, B) && task_map_fits(vs, B);
+    const bool v_mapped = mapped && (geo.G == 1 || grouped);
+    StepGeom geo_k = geo, geo_v = geo;
+    int *v_chunks = nullptr;
+    if (mapped) geo_k.task_map = reinterpret_cast<const u32 *>(ws + lay.map_k);
+    if (v_mapped) {
+        geo_v.task_map = reinterpret_cast<const u32 *>(ws + lay.map_v);
+        v_chunks = reinterpret_cast<int *>(ws + lay.v_chunks);
+    }
 
     int persist = 1;
     if (ragged) {
         // per-sequence lengths live on the device: one small kernel appends every token and flushes the rest
-        // buffers that fill up with it
-        hipLaunchKernelGGL((fused_pre_kernel<D>), dim3(B * Hkv), dim3(256), 0, st, kf8, km4, kl4, vf8, vm4, vl4, k16, v16,
-                           rk16, rv16, kcm, vcm, geo);
+        // buffers that fill up with it; its last workgroup writes the task maps
+        TaskMaps maps;
+        maps.map_k = mapped ? reinterpret_cast<u32 *>(ws + lay.map_k) : nullptr;
+        maps.map_v = v_mapped ? reinterpret_cast<u32 *>(ws + lay.map_v) : nullptr;
+        maps.v_chunks = v_chunks;
+        maps.k = ks;
+        maps.v = vs;
+        hipLaunchKernelGGL((fused_pre_kernel<D>), dim3(B * Hkv + (mapped ? 1 : 0)), dim3(256), 0, st, kf8, km4, kl4, vf8, vm4,
+                           vl4, k16, v16, rk16, rv16, kcm, vcm, geo, maps, B);
         int rc = check_launch("decode_step(pre)");
         if (rc != AKV_OK) return rc;
         persist = 0;
@@ -781,9 +891,6 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
         persist = 0;
     }
-    // flushed tokens after the append: exact for uniform lengths, an upper bound for ragged ones
-    const int R = (cur_len + 1) / cb * cb;
-    const int n_blocks = R / cb;
     MiddleArgs ma;
     ma.q = q16; ma.k_new = k16; ma.v_new = v16;
     ma.mask = reinterpret_cast<const unsigned short *>(mask);
@@ -792,8 +899,6 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     ma.kcm = kcm; ma.vcm = vcm; ma.toe = toe; ma.amin = amin; ma.v_first_8 = vf8;
     ma.g = geo; ma.mask_stride = mask_stride; ma.top_k = top_k; ma.persist = persist;
     mark(0, st);
-    // the kernel multiplies by the fp16-rounded scale (extension/csrc/K_cache.cu:306)
-    const float scale = __half2float(__float2half_rn(1.0f / sqrtf((float)D)));
     // One launch for the whole step: opt-in (AKV_TUNE_MONO=1), multi-head uniform-length caches only.  It
     // measures level with the four launches at batch 8 x 32 heads x 4096 tokens on MI355X.
     bool mono = false;
@@ -816,26 +921,21 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         mark(6, st);
         return check_launch("decode_step(mono)");
     }
-    // grouped-query heads: one workgroup per plane chunk serves 2 or 4 query heads (AKV_TUNE_GROUP: see group_heads)
-    const bool grouped = group_heads(geo.G) > 1;
-    bool matrix = geo.G >= 2 && geo.G <= 16;
-    if (const char *e = getenv("AKV_TUNE_MFMA")) matrix = matrix && atoi(e) != 0;
     if (n_blocks > 0 && matrix) {
         int rc = launch_mfma_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, reinterpret_cast<u32 *>(ws + lay.prep),
-                                       geo, B, n_blocks, ref, scale, st);
+                                       geo_k, B, n_blocks, ref, scale, st);
         if (rc != AKV_OK) return rc;
     } else if (n_blocks > 0 && grouped) {
-        int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo, B, n_blocks, ref, scale, st);
+        int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo_k, B, n_blocks, ref, scale, st);
         if (rc != AKV_OK) return rc;
     } else if (n_blocks > 0) {
-        const int bpw = k_blocks_per_wave(B, Hq, n_blocks);
-        dim3 grid(group_grid_x((n_blocks + 4 * bpw - 1) / (4 * bpw), geo.G), Hkv, B);
+        dim3 grid(ks.grid_x, ks.grid_y, B);
         if (ref)
             hipLaunchKernelGGL((fused_k_pass_kernel<D, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                               k_levels_out, geo, bpw, scale);
+                               k_levels_out, geo_k, bpw, scale);
         else
             hipLaunchKernelGGL((fused_k_pass_kernel<D, false>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                               k_levels_out, geo, bpw, scale);
+                               k_levels_out, geo_k, bpw, scale);
         int rc = check_launch("decode_step(k_pass)");
         if (rc != AKV_OK) return rc;
     }
@@ -849,15 +949,14 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
     }
     mark(2, st);
-    const VPlan p = v_plan(B, grouped ? Hq / group_heads(geo.G) : Hq, D, R);
     if (p.n_chunks > 0 && grouped) {
-        rc = launch_group_v_pass<D>(vf8, vm4, vl4, p16, amin, partial, v_levels_out, R, amin_out, geo, B, p, ref, st);
+        rc = launch_group_v_pass<D>(vf8, vm4, vl4, p16, amin, partial, v_levels_out, R, amin_out, geo_v, B, p, ref, st);
         if (rc != AKV_OK) return rc;
     } else if (p.n_chunks > 0) {
         dim3 grid(group_grid_x(p.n_chunks, geo.G), Hkv, B);
 #define AKV_VP(RF, N)                                                                                                  \
     hipLaunchKernelGGL((fused_v_pass_kernel<D, RF, N>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, amin, partial,     \
-                       v_levels_out, R, amin_out, geo, p.tokens_per_wave, p.n_chunks)
+                       v_levels_out, R, amin_out, geo_v, p.tokens_per_wave, p.n_chunks)
         if (ref) {
             if (p.iters_per_wave == 1) AKV_VP(true, 1);
             else if (p.iters_per_wave == 2) AKV_VP(true, 2);
@@ -873,7 +972,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     }
     mark(3, st);
     hipLaunchKernelGGL(fused_combine_kernel, dim3(B * Hq), dim3(D < 256 ? D : 256), 0, st, partial, otail,
-                       reinterpret_cast<unsigned short *>(out), D, p.n_chunks, seq_lens, Hq);
+                       reinterpret_cast<unsigned short *>(out), D, p.n_chunks, seq_lens, Hq, v_chunks);
     mark(4, st);
     mark(5, st);
     mark(6, st);

@@ -42,10 +42,11 @@ __global__ __launch_bounds__(256) void group_k_pass_kernel(
     constexpr int NG = D / 16;
     constexpr int HG = NG / 2;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int chunk = blockIdx.x, b = blockIdx.z;
+    int chunk, by, b;
+    if (!step_block(geo, chunk, by, b)) return;
     const int n_sub = geo.G / GH;
-    const int hkv = blockIdx.y / n_sub;
-    const int hq0 = hkv * geo.G + (blockIdx.y - hkv * n_sub) * GH;   // first query head of this workgroup
+    const int hkv = by / n_sub;
+    const int hq0 = hkv * geo.G + (by - hkv * n_sub) * GH;   // first query head of this workgroup
     const int bh_kv = b * geo.Hkv + hkv;
     const int64_t bh0 = (int64_t)b * geo.Hq + hq0;
     int R, nrest;
@@ -214,17 +215,18 @@ __global__ __launch_bounds__(256) void group_v_pass_kernel(
     constexpr int ST = U * TPL;               // tokens per step of two half tiles
     __shared__ float wave_part[4][D];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int chunk = blockIdx.x, b = blockIdx.z;
+    int chunk, by, b;
+    if (!step_block(geo, chunk, by, b)) return;
     const int n_sub = geo.G / GH;
-    const int hkv = blockIdx.y / n_sub;
-    const int hq0 = hkv * geo.G + (blockIdx.y - hkv * n_sub) * GH;
+    const int hkv = by / n_sub;
+    const int hq0 = hkv * geo.G + (by - hkv * n_sub) * GH;
     const int bh_kv = b * geo.Hkv + hkv;
     const int64_t bh0 = (int64_t)b * geo.Hq + hq0;
     int n_tokens, nrest;
     seq_state(geo, b, n_tokens, nrest);
     const int t_begin = (chunk * 4 + wave) * tokens_per_wave;
     const int t_end = min(t_begin + tokens_per_wave, n_tokens);
-    if (chunk * 4 * tokens_per_wave >= n_tokens && chunk > 0) {
+    if (chunk * 4 * tokens_per_wave >= n_tokens && chunk > 0) {   // (cannot happen with a task map)
         // the grid covers the longest sequence: a workgroup past the end of this one only clears its partial sums
         for (int i = threadIdx.x; i < GH * D; i += 256) partial[((bh0 + i / D) * n_chunks + chunk) * D + i % D] = 0.f;
         return;
@@ -300,13 +302,17 @@ template <int D>
 int launch_group_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *kcm,
                         const unsigned short *q, const unsigned short *k_new, unsigned short *scores,
                         uint8_t *levels_out, const StepGeom &geo, int B, int n_blocks, bool ref, float scale,
-                        hipStream_t st) {
+                        hipStream_t st, PassShape *shape_only) {
     const int GH = group_heads(geo.G);
     // a wave's set-up (q, levels and masks of GH heads) costs about half a block: several blocks per wave
     int bpw = 1;
     while (bpw < 8 && (int64_t)B * geo.Hkv * (geo.G / GH) * ((n_blocks + 8 * bpw - 1) / (8 * bpw)) * 4 >= 6144) bpw *= 2;
     if (const char *e = getenv("AKV_TUNE_K_BPW")) bpw = atoi(e) > 0 ? atoi(e) : bpw;
     dim3 grid((n_blocks + 4 * bpw - 1) / (4 * bpw), geo.Hkv * (geo.G / GH), B);
+    if (shape_only != nullptr) {
+        *shape_only = PassShape{(int)grid.x, (int)grid.y, 4 * bpw * 64};
+        return AKV_OK;
+    }
 #define AKV_GK(RF, GG)                                                                                              \
     hipLaunchKernelGGL((group_k_pass_kernel<D, RF, GG>), grid, dim3(256), 0, st, f8, m4, l4, kcm, q, k_new, scores, \
                        levels_out, geo, bpw, scale)
@@ -334,7 +340,7 @@ int launch_group_v_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4,
 #define AKV_INST(DD)                                                                                                     \
     template int launch_group_k_pass<DD>(const uint8_t *, const uint8_t *, const uint8_t *, const uint8_t *,             \
                                          const unsigned short *, const unsigned short *, unsigned short *, uint8_t *,    \
-                                         const StepGeom &, int, int, bool, float, hipStream_t);                          \
+                                         const StepGeom &, int, int, bool, float, hipStream_t, PassShape *);                          \
     template int launch_group_v_pass<DD>(const uint8_t *, const uint8_t *, const uint8_t *, const unsigned short *,      \
                                          const uint8_t *, float *, uint8_t *, int, uint8_t *, const StepGeom &, int,     \
                                          const VPlan &, bool, hipStream_t);

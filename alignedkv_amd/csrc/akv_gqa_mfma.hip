@@ -220,7 +220,8 @@ __global__ __launch_bounds__(256) void mfma_k_pass_kernel(
     constexpr int NBT = 16 / PB;   // blocks per task
     static_assert(KG % (AHEAD + 1) == 0, "the tile ring is rotated by unrolling");
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int chunk = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z;
+    int chunk, hkv, b;
+    if (!step_block(geo, chunk, hkv, b)) return;
     const int G = geo.G;
     const int bh_kv = b * geo.Hkv + hkv;
     const int64_t bh0 = (int64_t)b * geo.Hq + hkv * G;
@@ -312,7 +313,7 @@ template <int D>
 int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *kcm,
                        const unsigned short *q, const unsigned short *k_new, unsigned short *scores,
                        uint8_t *levels_out, u32 *prep, const StepGeom &geo, int B, int n_blocks, bool ref, float scale,
-                       hipStream_t st) {
+                       hipStream_t st, PassShape *shape_only) {
     int sl = 8;
     if (const char *e = getenv("AKV_TUNE_K_SL")) sl = atoi(e) == 16 ? 16 : (atoi(e) == 4 ? 4 : 8);
     const int nbt = sl / 4;
@@ -320,6 +321,10 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
     int tpw = 1;
     while (tpw < 8 && (int64_t)B * geo.Hkv * ((n_tasks + 8 * tpw - 1) / (8 * tpw)) * 4 >= 8192) tpw *= 2;
     if (const char *e = getenv("AKV_TUNE_K_TPW")) tpw = atoi(e) > 0 ? atoi(e) : tpw;
+    if (shape_only != nullptr) {
+        *shape_only = PassShape{(n_tasks + 4 * tpw - 1) / (4 * tpw), geo.Hkv, 4 * tpw * nbt * 64};
+        return AKV_OK;
+    }
     const int64_t scores_bytes = (int64_t)B * geo.Hq * geo.row_stride * 2;
     if (scores_bytes >= ((int64_t)1 << 31)) {
         set_error("decode_step: score rows of %lld bytes exceed the 2 GiB the grouped K pass addresses", (long long)scores_bytes);
@@ -350,7 +355,7 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
 #define AKV_INST(DD)                                                                                                  \
     template int launch_mfma_k_pass<DD>(const uint8_t *, const uint8_t *, const uint8_t *, const uint8_t *,           \
                                         const unsigned short *, const unsigned short *, unsigned short *, uint8_t *, \
-                                        u32 *, const StepGeom &, int, int, bool, float, hipStream_t);
+                                        u32 *, const StepGeom &, int, int, bool, float, hipStream_t, PassShape *);
 AKV_INST(64)
 AKV_INST(128)
 AKV_INST(256)

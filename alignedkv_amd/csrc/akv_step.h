@@ -15,7 +15,16 @@ struct StepGeom {
     int cb, max_seq_len, n_max_blocks, row_stride;
     int cur_len;
     const int *seq_lens;
+    const u32 *task_map;   // per-sequence lengths: workgroup -> (chunk, head index, batch) of this launch, or null
 };
+
+// Launch shape of a pass: grid (grid_x, grid_y, batch), a workgroup covers tokens_per_wg tokens of one sequence.
+struct PassShape {
+    int grid_x, grid_y, tokens_per_wg;
+};
+constexpr u32 kNoTask = 0xffffffffu;
+__host__ __device__ inline u32 pack_task(int x, int y, int z) { return (u32)x | ((u32)y << 12) | ((u32)z << 20); }
+inline bool task_map_fits(const PassShape &s, int B) { return s.grid_x <= 4096 && s.grid_y <= 256 && B <= 4096; }
 
 // tokens flushed into the planes / held in the rest buffer once this step's token has been appended
 __device__ __forceinline__ void seq_state(const StepGeom &g, int b, int &R, int &nrest) {
@@ -24,12 +33,31 @@ __device__ __forceinline__ void seq_state(const StepGeom &g, int b, int &R, int 
     nrest = L - R;
 }
 
+// Workgroup -> (chunk x, head index y, batch z) of a launch with grid (chunks, heads, batch); false: nothing to do.
+// With per-sequence lengths the grid covers the longest sequence, and in dispatch order (x fastest) the workgroups
+// past the end of the shorter ones would be scattered between the working ones, each holding a workgroup slot for
+// a microsecond or two (measured: +22 % on the K pass with two such out of three).  The step's first kernel
+// therefore writes a map from the linear workgroup index to the tasks that exist, in the same order; what is left
+// over gathers at the end of the launch and leaves at once.
+__device__ __forceinline__ bool step_block(const StepGeom &g, int &x, int &y, int &z) {
+    x = blockIdx.x;
+    y = blockIdx.y;
+    z = blockIdx.z;
+    if (g.task_map != nullptr) {
+        const u32 e = g.task_map[blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)];
+        if (e == kNoTask) return false;
+        x = (int)(e & 0xfffu);
+        y = (int)((e >> 12) & 0xffu);
+        z = (int)(e >> 20);
+    }
+    return true;
+}
+
 // Workgroup -> (chunk, query head of the group).  Workgroups go to the 8 XCDs round-robin by linear index,
 // and each XCD has its own L2: the G workgroups that stream the same plane chunk for the G query heads of a
 // KV head get linear indices 8 apart, i.e. the same XCD at about the same time, so the chunk comes from HBM
 // once and from that L2 G-1 times.  gridDim.x = 8 * ceil(chunks / 8) * G.
-__device__ __forceinline__ void decode_group_block(int G, int &chunk, int &gq) {
-    const int lin = blockIdx.x;
+__device__ __forceinline__ void decode_group_block(int G, int lin, int &chunk, int &gq) {
     if (G == 1) {
         chunk = lin;
         gq = 0;
@@ -48,7 +76,7 @@ template <int D>
 int launch_group_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *kcm,
                         const unsigned short *q, const unsigned short *k_new, unsigned short *scores,
                         uint8_t *levels_out, const StepGeom &geo, int B, int n_blocks, bool ref, float scale,
-                        hipStream_t st);
+                        hipStream_t st, PassShape *shape_only = nullptr);
 template <int D>
 int launch_group_v_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const unsigned short *probs,
                         const uint8_t *amin, float *partial, uint8_t *levels_out, int levels_stride, uint8_t *amin_out,
@@ -60,7 +88,7 @@ template <int D>
 int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *kcm,
                        const unsigned short *q, const unsigned short *k_new, unsigned short *scores,
                        uint8_t *levels_out, u32 *prep, const StepGeom &geo, int B, int n_blocks, bool ref, float scale,
-                       hipStream_t st);
+                       hipStream_t st, PassShape *shape_only = nullptr);
 // words of set-up data per (batch, KV head) that launch_mfma_k_pass needs in `prep`
 inline size_t mfma_k_prep_words(int D) { return (size_t)64 * (2 * (D / 16) + 4); }
 
