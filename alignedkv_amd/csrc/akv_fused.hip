@@ -835,7 +835,12 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     bool matrix = geo.G >= 2 && geo.G <= 16;
     if (const char *e = getenv("AKV_TUNE_MFMA")) matrix = matrix && atoi(e) != 0;
     const int bpw = k_blocks_per_wave(B, Hq, n_blocks);
-    const VPlan p = v_plan(B, grouped ? Hq / group_heads(geo.G) : Hq, D, R);
+    bool matrix_v = matrix && D <= 128;
+    if (const char *e = getenv("AKV_TUNE_MFMA_V")) matrix_v = matrix_v && atoi(e) != 0;
+    VPlan p = v_plan(B, grouped ? Hq / group_heads(geo.G) : Hq, D, R);
+    if constexpr (D <= 128) {
+        if (matrix_v) p = mfma_v_plan<D>(B, Hkv, R);
+    }
     // launch shapes of the two streaming passes
     PassShape ks = {0, 0, 0}, vs = {0, 0, 0};
     if (n_blocks > 0) {
@@ -849,12 +854,13 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         } else {
             ks = PassShape{group_grid_x((n_blocks + 4 * bpw - 1) / (4 * bpw), geo.G), Hkv, 4 * bpw * cb};
         }
-        vs = PassShape{grouped ? p.n_chunks : group_grid_x(p.n_chunks, geo.G), grouped ? Hkv * (geo.G / group_heads(geo.G)) : Hkv,
-                       p.chunk_tokens};
+        if (matrix_v) vs = PassShape{p.n_chunks, Hkv, p.chunk_tokens};
+        else vs = PassShape{grouped ? p.n_chunks : group_grid_x(p.n_chunks, geo.G), grouped ? Hkv * (geo.G / group_heads(geo.G)) : Hkv,
+                            p.chunk_tokens};
     }
     // task maps (per-sequence lengths): not for the swizzled grids of ungrouped multi-query heads
     const bool mapped = ragged && n_blocks > 0 && (geo.G == 1 || grouped || matrix) && task_map_fits(ks, B) && task_map_fits(vs, B);
-    const bool v_mapped = mapped && (geo.G == 1 || grouped);
+    const bool v_mapped = mapped && (geo.G == 1 || grouped || matrix_v);
     StepGeom geo_k = geo, geo_v = geo;
     int *v_chunks = nullptr;
     if (mapped) geo_k.task_map = reinterpret_cast<const u32 *>(ws + lay.map_k);
@@ -949,7 +955,11 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
     }
     mark(2, st);
-    if (p.n_chunks > 0 && grouped) {
+    if (p.n_chunks > 0 && matrix_v) {
+        if constexpr (D <= 128)
+            rc = launch_mfma_v_pass<D>(vf8, vm4, vl4, p16, amin, partial, v_levels_out, R, amin_out, geo_v, B, p, ref, st);
+        if (rc != AKV_OK) return rc;
+    } else if (p.n_chunks > 0 && grouped) {
         rc = launch_group_v_pass<D>(vf8, vm4, vl4, p16, amin, partial, v_levels_out, R, amin_out, geo_v, B, p, ref, st);
         if (rc != AKV_OK) return rc;
     } else if (p.n_chunks > 0) {

@@ -209,6 +209,40 @@ __global__ __launch_bounds__(64) void mfma_k_prepare_kernel(const uint8_t *__res
     out[2 * KG + 3] = need_last;
 }
 
+// The same for a tile whose rows are all used at level 2 by every head (only the high bytes were fetched): the low
+// byte is the constant 0x80 and there is nothing to correct.
+template <int SL>
+__device__ __forceinline__ void kt_compute_coarse(f32x4 *acc, const KTaskTile<SL> &t, f16x4 b0) {
+    constexpr int NX = (SL + 7) / 8;
+    constexpr int NP = SL == 4 ? 2 : 4;
+    const u32 c80 = 0x80808080u;
+#pragma unroll
+    for (int x = 0; x < NX; ++x) {
+        u32 w[4][4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const u32 Ha = t.h[r][SL == 4 ? 0 : 2 * x];
+            w[r][0] = __builtin_amdgcn_perm(Ha, c80, 0x06010400u);
+            w[r][1] = __builtin_amdgcn_perm(Ha, c80, 0x07010500u);
+            if constexpr (SL != 4) {
+                const u32 Hb = t.h[r][2 * x + 1];
+                w[r][2] = __builtin_amdgcn_perm(Hb, c80, 0x06030402u);
+                w[r][3] = __builtin_amdgcn_perm(Hb, c80, 0x07030502u);
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int s0 = 8 * x + (p & 1) + 4 * (p >> 1);
+            const u32 a01_s0 = __builtin_amdgcn_perm(w[1][p], w[0][p], 0x05040100u);
+            const u32 a23_s0 = __builtin_amdgcn_perm(w[3][p], w[2][p], 0x05040100u);
+            const u32 a01_s2 = __builtin_amdgcn_perm(w[1][p], w[0][p], 0x07060302u);
+            const u32 a23_s2 = __builtin_amdgcn_perm(w[3][p], w[2][p], 0x07060302u);
+            acc[s0] = __builtin_amdgcn_mfma_f32_16x16x16f16(as_f16x4(a01_s0, a23_s0), b0, acc[s0], 0, 0, 0);
+            acc[s0 + 2] = __builtin_amdgcn_mfma_f32_16x16x16f16(as_f16x4(a01_s2, a23_s2), b0, acc[s0 + 2], 0, 0, 0);
+        }
+    }
+}
+
 template <int D, bool REF, int SL, int AHEAD>
 __global__ __launch_bounds__(256) void mfma_k_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
@@ -352,13 +386,264 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
     return check_launch("decode_step(mfma k_pass)");
 }
 
-#define AKV_INST(DD)                                                                                                  \
+// ------------------------------------------------------------------------------------------------
+// V pass.  out[j][c] = sum over tokens of p_j[t] * v_level_j(t)[t][c]: rows = channels, contraction = tokens,
+// columns = query heads.  Lane l: channel piece i = l % 16 (D/16 channels), token residue tg = l / 16; a step is
+// 16 tokens (token = step base + 4 tg + u, u < 4 loads), a tile is the lane's D/16 channels of its 4 tokens -- the
+// same register shape as a K tile with slots and channels exchanged, so the unpacking (kt_compute) is shared.
+// The fetch level depends on the token: lane (j, tg) holds the probabilities of head j for the 4 tokens of its
+// lane group and works out their levels; the OR over the 16 lanes of the group gives the planes to fetch for
+// exactly the tokens the group's lanes load.  Lane (j, ig) ends up with 4 x D/16 output channels of head j.
+// A wave walks tokens_per_wave tokens in macro steps of 64 (4 tiles, three in flight while one is multiplied);
+// the probabilities are requested two macro steps ahead so that waiting for them never waits for a tile.
+// grid (n_chunks, Hkv, B), 256 threads.
+// ------------------------------------------------------------------------------------------------
+template <int D>
+__device__ __forceinline__ void vt_issue(KTaskTile<D / 16> &t, const __amdgpu_buffer_rsrc_t rH, const __amdgpu_buffer_rsrc_t rM,
+                                         const __amdgpu_buffer_rsrc_t rL, int lane_h, int lane_m, int step_base, bool valid,
+                                         bool fine, u32 need_mid, u32 need_last) {
+    // lane_h / lane_m: byte offsets of the lane's piece in the row of token 4 tg; step_base and valid are wave-uniform
+    constexpr int CPP = D / 16;
+    const int oh = valid ? lane_h + step_base * D : kSkip, om = lane_m + step_base * (D / 2);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) load_bytes<CPP>(t.h[u], rH, oh + u * D);
+    if (!fine) return;   // wave-uniform: no lane of the wave fetches a nibble row of this step
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        load_bytes<CPP / 2>(t.m[u], rM, (valid && ((need_mid >> u) & 1u)) ? om + u * (D / 2) : kSkip);
+        load_bytes<CPP / 2>(t.l[u], rL, (valid && ((need_last >> u) & 1u)) ? om + u * (D / 2) : kSkip);
+    }
+}
+
+// What a lane needs for one macro step (64 tokens = 4 steps of 16): the probabilities of its head for its 16
+// tokens (4 per step), their levels as bit sets (bit 4 s + u), and the planes its lane group fetches.
+struct VMacroOps {
+    u32x2 p[4];           // step s: tokens 4 kq + 0..3 of the step, packed fp16 pairs
+    u32 lv1, lv2;         // this head's level of the token is 1 / 2
+    u32 need;             // bits 0..15: mid row fetched, bits 16..31: last row fetched (union over the heads)
+};
+
+typedef short i16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+// packed 16-bit a - b with wrap-around, read as signed
+__device__ __forceinline__ i16x2 wrap_diff16(u16x2 a, u32 b) {
+    union { u32 u; u16x2 v; } x;
+    x.u = b;
+    union { u16x2 u; i16x2 s; } d;
+    d.u = a - x.v;
+    return d.s;
+}
+
+template <bool REF>
+__device__ __forceinline__ void v_macro_ops(VMacroOps &o, const u32x2 *p, unsigned char amin, bool head) {
+    u32 mid = 0, last = 0;
+    o.lv1 = 0;
+    o.lv2 = head ? 0xffffu : 0u;
+#pragma unroll
+    for (int sidx = 0; sidx < 4; ++sidx) o.p[sidx] = head ? p[sidx] : (u32x2){0u, 0u};
+    if (REF) {
+        mid = last = head ? 0xffffu : 0u;
+        o.lv2 = 0;
+    } else {
+        // most tokens are at level 2 for every head: first the smallest 16-bit difference of the lane's 16 tokens
+        // (the differences wrap like the reference's `short` arithmetic, extension/csrc/V_cache.cu:195-197,211)
+        const unsigned short a16 = (unsigned short)((unsigned)amin << 10);
+        const u16x2 a2 = {a16, a16};
+        i16x2 mn = {32767, 32767};
+#pragma unroll
+        for (int sidx = 0; sidx < 4; ++sidx) {
+            const i16x2 d0 = wrap_diff16(a2, p[sidx].x), d1 = wrap_diff16(a2, p[sidx].y);
+            mn = __builtin_elementwise_min(mn, __builtin_elementwise_min(d0, d1));
+        }
+        if (head && min(mn.x, mn.y) < 0x0800) {   // some token of this lane is at level 0 or 1: classify all
+            o.lv2 = 0;
+#pragma unroll
+            for (int sidx = 0; sidx < 4; ++sidx)
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const u32 bits = ((u < 2 ? p[sidx].x : p[sidx].y) >> (16 * (u & 1))) & 0xffffu;
+                    const int lv = v_level(amin, (unsigned short)bits);
+                    mid |= (lv < 2 ? 1u : 0u) << (4 * sidx + u);
+                    last |= (lv == 0 ? 1u : 0u) << (4 * sidx + u);
+                    o.lv1 |= (lv == 1 ? 1u : 0u) << (4 * sidx + u);
+                    o.lv2 |= (lv == 2 ? 1u : 0u) << (4 * sidx + u);
+                }
+        }
+    }
+    // union over the heads: OR over the 16 lanes of the lane group
+    u32 both = mid | (last << 16);
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) both |= (u32)__shfl_xor((int)both, m, 64);
+    o.need = both;
+}
+
+template <int D, bool REF>
+__global__ __launch_bounds__(256) void mfma_v_pass_kernel(
+    const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
+    const unsigned short *__restrict__ probs, const uint8_t *__restrict__ amin_u8, float *__restrict__ partial,
+    uint8_t *__restrict__ levels_out, int levels_stride, uint8_t *__restrict__ amin_out, StepGeom geo,
+    int tokens_per_wave, int n_chunks, u32 probs_bytes) {
+    constexpr int CPP = D / 16;        // channels per lane
+    constexpr int MACRO = 64;          // tokens per macro step: 4 tiles of 16 tokens
+    __shared__ float fold[4][4][D];    // [wave][head of the pass][channel]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int chunk, hkv, b;
+    if (!step_block(geo, chunk, hkv, b)) return;
+    const int G = geo.G;
+    const int bh_kv = b * geo.Hkv + hkv;
+    const int64_t bh0 = (int64_t)b * geo.Hq + hkv * G;
+    int n_tokens, nrest;
+    seq_state(geo, b, n_tokens, nrest);
+    if (chunk * 4 * tokens_per_wave >= n_tokens && chunk > 0) {
+        // (without a task map) a workgroup past the end of this sequence only clears its partial sums
+        for (int i = threadIdx.x; i < G * D; i += 256) partial[((bh0 + i / D) * n_chunks + chunk) * D + i % D] = 0.f;
+        return;
+    }
+    // all of these are multiples of 64: a step of 16 tokens is inside [t_begin, t_end) or outside as a whole
+    const int t_begin = (chunk * 4 + wave) * tokens_per_wave;
+    const int t_end = min(t_begin + tokens_per_wave, n_tokens);
+    const int64_t row0 = (int64_t)bh_kv * geo.max_seq_len;
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(first_8 + row0 * D, (u32)n_tokens * D);
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(mid_4 + row0 * (D / 2), (u32)n_tokens * (D / 2));
+    const __amdgpu_buffer_rsrc_t rL = make_rsrc(last_4 + row0 * (D / 2), (u32)n_tokens * (D / 2));
+    const __amdgpu_buffer_rsrc_t rP = make_rsrc(probs, probs_bytes);
+    const int j = lane & 15, kq = lane >> 4;
+    const bool head = j < G;
+    const unsigned char amin = (REF || !head) ? 0 : amin_u8[bh0 + j];
+    if (!REF && head && amin_out != nullptr && chunk == 0 && wave == 0 && kq == 0) amin_out[bh0 + j] = amin;
+    const int lane_p = (int)((bh0 + (head ? j : 0)) * geo.row_stride + 4 * kq) * 2;
+    const int lane_h = (4 * kq) * D + (lane & 15) * CPP, lane_m = (4 * kq) * (D / 2) + (lane & 15) * (CPP / 2);
+
+    // probabilities of the lane's head for a macro step: 4 steps x 4 tokens (base + 16 s + 4 kq + r)
+    auto load_probs = [&](u32x2 *dst, int base) {
+        const int o = base < t_end ? lane_p + base * 2 : kSkip;
+#pragma unroll
+        for (int sidx = 0; sidx < 4; ++sidx) dst[sidx] = __builtin_amdgcn_raw_buffer_load_b64(rP, o + 32 * sidx, 0, 0);
+    };
+    // fine(o, s): some lane of the wave fetches a nibble row in step s of the macro step (wave-uniform)
+    auto fine = [&](const VMacroOps &o, int sidx) -> bool {
+        return __builtin_amdgcn_ballot_w64(((o.need >> (4 * sidx)) & 0x000f000fu) != 0u) != 0ull;
+    };
+    auto issue = [&](KTaskTile<CPP> &tile, const VMacroOps &o, int macro_base, int sidx) {
+        vt_issue<D>(tile, rH, rM, rL, lane_h, lane_m, macro_base + 16 * sidx, macro_base < t_end, fine(o, sidx),
+                    (o.need >> (4 * sidx)) & 0xfu, (o.need >> (16 + 4 * sidx)) & 0xfu);
+    };
+    f32x4 acc[CPP];
+#pragma unroll
+    for (int i = 0; i < CPP; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    u32x2 pn[4], pnn[4];
+    VMacroOps oc, on;
+    {
+        u32x2 pc[4];
+        load_probs(pc, t_begin);
+        load_probs(pn, t_begin + MACRO);
+        v_macro_ops<REF>(oc, pc, amin, head);
+    }
+    KTaskTile<CPP> t[4];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) issue(t[i], oc, t_begin, i);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int base = t_begin; base < t_end; base += MACRO) {
+        load_probs(pnn, base + 2 * MACRO);
+        v_macro_ops<REF>(on, pn, amin, head);     // levels and fetch masks of the next macro step
+#pragma unroll
+        for (int si = 0; si < 4; ++si) {
+            if (si == 0) issue(t[3], oc, base, 3);
+            else issue(t[si - 1], on, base + MACRO, si - 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (fine(oc, si)) {
+                const u32 l1 = (oc.lv1 >> (4 * si)) & 0xfu, l2 = (oc.lv2 >> (4 * si)) & 0xfu;
+                const u32 na = oc.p[si].x ^ 0x80008000u, nb = oc.p[si].y ^ 0x80008000u;     // -p
+                const u32 n1a = na & ((l1 & 1u ? 0xFFFFu : 0u) | (l1 & 2u ? 0xFFFF0000u : 0u));
+                const u32 n1b = nb & ((l1 & 4u ? 0xFFFFu : 0u) | (l1 & 8u ? 0xFFFF0000u : 0u));
+                const u32 n2a = na & ((l2 & 1u ? 0xFFFFu : 0u) | (l2 & 2u ? 0xFFFF0000u : 0u));
+                const u32 n2b = nb & ((l2 & 4u ? 0xFFFFu : 0u) | (l2 & 8u ? 0xFFFF0000u : 0u));
+                kt_compute<REF, CPP>(acc, t[si], 0, (oc.need >> (4 * si)) & 0xfu, (oc.need >> (16 + 4 * si)) & 0xfu,
+                                     as_f16x4(oc.p[si].x, oc.p[si].y), as_f16x4(n1a, n1b), as_f16x4(n2a, n2b));
+            } else {
+                kt_compute_coarse<CPP>(acc, t[si], as_f16x4(oc.p[si].x, oc.p[si].y));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        oc = on;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pn[i] = pnn[i];
+    }
+    // optional record of the levels, outside the pipeline
+    if (levels_out != nullptr) {
+        for (int tt = t_begin + lane; tt < t_end; tt += 64)
+            for (int h = 0; h < G; ++h)
+                levels_out[(bh0 + h) * levels_stride + tt] =
+                    (uint8_t)(REF ? 0 : v_level(amin_u8[bh0 + h], probs[(bh0 + h) * geo.row_stride + tt]));
+    }
+    // lane (j, ig): acc[cc][r] = out_j[CPP * (4 ig + r) + cc] over this wave's tokens; the 4 waves are added
+    // through LDS, four heads at a time
+    for (int pass = 0; pass * 4 < G; ++pass) {
+        if ((j >> 2) == pass) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int cc = 0; cc < CPP; ++cc) fold[wave][j & 3][CPP * (4 * (lane >> 4) + r) + cc] = acc[cc][r];
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < 4 * D; i += 256) {
+            const int hs = i / D, d = i - hs * D, hh = pass * 4 + hs;
+            if (hh < G)
+                partial[((bh0 + hh) * n_chunks + chunk) * D + d] = (fold[0][hs][d] + fold[1][hs][d]) + (fold[2][hs][d] + fold[3][hs][d]);
+        }
+        __syncthreads();
+    }
+}
+
+template <int D>
+VPlan mfma_v_plan(int B, int Hkv, int n_tokens) {
+    VPlan p;
+    p.tuned = true;
+    int k = 1;   // macro steps of 64 tokens per wave
+    while (k < 4 && (int64_t)B * Hkv * ((n_tokens + 512 * k - 1) / (512 * k)) >= 2048) k *= 2;
+    if (const char *e = getenv("AKV_TUNE_V_ITERS")) k = atoi(e) > 0 ? atoi(e) : k;
+    p.iters_per_wave = k;
+    p.tokens_per_wave = 64 * k;
+    p.chunk_tokens = 4 * p.tokens_per_wave;
+    p.n_chunks = n_tokens > 0 ? (n_tokens + p.chunk_tokens - 1) / p.chunk_tokens : 0;
+    return p;
+}
+
+template <int D>
+int launch_mfma_v_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const unsigned short *probs,
+                       const uint8_t *amin, float *partial, uint8_t *levels_out, int levels_stride, uint8_t *amin_out,
+                       const StepGeom &geo, int B, const VPlan &p, bool ref, hipStream_t st) {
+    const int64_t probs_bytes = (int64_t)B * geo.Hq * geo.row_stride * 2;
+    if (probs_bytes >= ((int64_t)1 << 31)) {
+        set_error("decode_step: probability rows of %lld bytes exceed the 2 GiB the grouped V pass addresses", (long long)probs_bytes);
+        return AKV_ERR_INVALID;
+    }
+    dim3 grid(p.n_chunks, geo.Hkv, B);
+    if (ref)
+        hipLaunchKernelGGL((mfma_v_pass_kernel<D, true>), grid, dim3(256), 0, st, f8, m4, l4, probs, amin, partial, levels_out,
+                           levels_stride, amin_out, geo, p.tokens_per_wave, p.n_chunks, (u32)probs_bytes);
+    else
+        hipLaunchKernelGGL((mfma_v_pass_kernel<D, false>), grid, dim3(256), 0, st, f8, m4, l4, probs, amin, partial, levels_out,
+                           levels_stride, amin_out, geo, p.tokens_per_wave, p.n_chunks, (u32)probs_bytes);
+    return check_launch("decode_step(mfma v_pass)");
+}
+
+#define AKV_INST_K(DD)                                                                                                \
     template int launch_mfma_k_pass<DD>(const uint8_t *, const uint8_t *, const uint8_t *, const uint8_t *,           \
                                         const unsigned short *, const unsigned short *, unsigned short *, uint8_t *, \
                                         u32 *, const StepGeom &, int, int, bool, float, hipStream_t, PassShape *);
-AKV_INST(64)
-AKV_INST(128)
-AKV_INST(256)
-#undef AKV_INST
+#define AKV_INST_V(DD)                                                                                                \
+    template VPlan mfma_v_plan<DD>(int, int, int);                                                                    \
+    template int launch_mfma_v_pass<DD>(const uint8_t *, const uint8_t *, const uint8_t *, const unsigned short *,    \
+                                        const uint8_t *, float *, uint8_t *, int, uint8_t *, const StepGeom &, int,    \
+                                        const VPlan &, bool, hipStream_t);
+AKV_INST_K(64)
+AKV_INST_K(128)
+AKV_INST_K(256)
+AKV_INST_V(64)
+AKV_INST_V(128)   // head_dim 256 keeps the vector-ALU V pass: its tiles and accumulators do not fit the register file
+#undef AKV_INST_K
+#undef AKV_INST_V
 
 }  // namespace akv

@@ -89,6 +89,12 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
                        const unsigned short *q, const unsigned short *k_new, unsigned short *scores,
                        uint8_t *levels_out, u32 *prep, const StepGeom &geo, int B, int n_blocks, bool ref, float scale,
                        hipStream_t st, PassShape *shape_only = nullptr);
+template <int D>
+VPlan mfma_v_plan(int B, int Hkv, int n_tokens);
+template <int D>
+int launch_mfma_v_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const unsigned short *probs,
+                       const uint8_t *amin, float *partial, uint8_t *levels_out, int levels_stride, uint8_t *amin_out,
+                       const StepGeom &geo, int B, const VPlan &p, bool ref, hipStream_t st);
 // words of set-up data per (batch, KV head) that launch_mfma_k_pass needs in `prep`
 inline size_t mfma_k_prep_words(int D) { return (size_t)64 * (2 * (D / 16) + 4); }
 
