@@ -832,10 +832,10 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     // grouped-query heads: one workgroup per plane chunk serves 2 or 4 query heads (AKV_TUNE_GROUP: see group_heads),
     // or up to 16 on the matrix cores (K pass)
     const bool grouped = group_heads(geo.G) > 1;
-    bool matrix = geo.G >= 2 && geo.G <= 16;
+    bool matrix = geo.G >= 2 && geo.G <= 16 && D <= 128;   // (the 32-bit level masks hold 128 channels)
     if (const char *e = getenv("AKV_TUNE_MFMA")) matrix = matrix && atoi(e) != 0;
     const int bpw = k_blocks_per_wave(B, Hq, n_blocks);
-    bool matrix_v = matrix && D <= 128;
+    bool matrix_v = matrix;
     if (const char *e = getenv("AKV_TUNE_MFMA_V")) matrix_v = matrix_v && atoi(e) != 0;
     VPlan p = v_plan(B, grouped ? Hq / group_heads(geo.G) : Hq, D, R);
     if constexpr (D <= 128) {
@@ -845,8 +845,9 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     PassShape ks = {0, 0, 0}, vs = {0, 0, 0};
     if (n_blocks > 0) {
         if (matrix) {
-            int rc = launch_mfma_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, nullptr, geo, B, n_blocks, ref, scale,
-                                           st, &ks);
+            int rc = AKV_OK;
+            if constexpr (D <= 128)
+                rc = launch_mfma_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, nullptr, geo, B, n_blocks, ref, scale, st, &ks);
             if (rc != AKV_OK) return rc;
         } else if (grouped) {
             int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo, B, n_blocks, ref, scale, st, &ks);
@@ -928,7 +929,9 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         return check_launch("decode_step(mono)");
     }
     if (n_blocks > 0 && matrix) {
-        int rc = launch_mfma_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, reinterpret_cast<u32 *>(ws + lay.prep),
+        int rc = AKV_OK;
+        if constexpr (D <= 128)
+            rc = launch_mfma_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, reinterpret_cast<u32 *>(ws + lay.prep),
                                        geo_k, B, n_blocks, ref, scale, st);
         if (rc != AKV_OK) return rc;
     } else if (n_blocks > 0 && grouped) {

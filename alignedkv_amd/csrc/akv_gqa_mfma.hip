@@ -157,6 +157,7 @@ __global__ __launch_bounds__(64) void mfma_k_prepare_kernel(const uint8_t *__res
                                                            const unsigned short *__restrict__ k_new, u32 *__restrict__ prep,
                                                            uint8_t *__restrict__ levels_out, StepGeom geo) {
     constexpr int KG = D / 16;
+    static_assert(4 * KG <= 32, "the level masks are 32 bits wide");
     const int lane = threadIdx.x;
     const int bh_kv = blockIdx.x, b = bh_kv / geo.Hkv, hkv = bh_kv - b * geo.Hkv;
     const int G = geo.G;
@@ -640,9 +641,8 @@ int launch_mfma_v_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
                                         const VPlan &, bool, hipStream_t);
 AKV_INST_K(64)
 AKV_INST_K(128)
-AKV_INST_K(256)
 AKV_INST_V(64)
-AKV_INST_V(128)   // head_dim 256 keeps the vector-ALU V pass: its tiles and accumulators do not fit the register file
+AKV_INST_V(128)   // head_dim 256 keeps the vector-ALU passes: 32-bit level masks, and the V tiles do not fit the registers
 #undef AKV_INST_K
 #undef AKV_INST_V
 

@@ -14,11 +14,14 @@ def dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-@pytest.mark.parametrize("B,Hq,Hkv,lens,steps", [(3, 8, 2, [130, 64, 7], 70), (2, 4, 4, [200, 255], 3),
-                                                 (4, 16, 2, [63, 127, 128, 1], 66), (2, 8, 1, [300, 190], 5)])
-def test_gqa_ragged_step_matches_per_sequence_oracle(B, Hq, Hkv, lens, steps):
+@pytest.mark.parametrize("B,Hq,Hkv,lens,steps,D", [(3, 8, 2, [130, 64, 7], 70, 128), (2, 4, 4, [200, 255], 3, 128),
+                                                   (4, 16, 2, [63, 127, 128, 1], 66, 128), (2, 8, 1, [300, 190], 5, 128),
+                                                   (2, 8, 2, [500, 321], 4, 64), (2, 12, 4, [260, 700], 3, 64),
+                                                   (2, 8, 2, [450, 130], 4, 256), (1, 6, 2, [1100], 2, 128),
+                                                   (2, 40, 2, [200, 330], 2, 128)])
+def test_gqa_ragged_step_matches_per_sequence_oracle(B, Hq, Hkv, lens, steps, D):
     from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
-    D, G = 128, Hq // Hkv
+    G = Hq // Hkv
     Lmax = max(lens) + steps + 5
     _, k, v = make_qkv(B, Lmax, Hkv, D, seed=sum(lens), n_outliers=4)
     rng = np.random.default_rng(Hq)
