@@ -605,9 +605,9 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
 }
 
 // grid (B*H), 256 threads: the middle stage on its own (no flushed block yet, or fusion switched off).
-template <int D>
-__global__ __launch_bounds__(256) void fused_middle_kernel(MiddleArgs a) {
-    middle_body<D, 256>(a, blockIdx.x);
+template <int D, int NT>
+__global__ __launch_bounds__(NT) void fused_middle_kernel(MiddleArgs a) {
+    middle_body<D, NT>(a, blockIdx.x);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -949,7 +949,14 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
     }
     mark(1, st);
-    hipLaunchKernelGGL((fused_middle_kernel<D>), dim3(B * Hq), dim3(256), 0, st, ma);
+    {
+        // threads per (batch, head) row: 512 and 1024 measure level with 256 at batch 8 x 32 heads x 4096 tokens
+        int nt = 256;
+        if (const char *e = getenv("AKV_TUNE_MIDDLE_NT")) nt = atoi(e);
+        if (nt == 1024) hipLaunchKernelGGL((fused_middle_kernel<D, 1024>), dim3(B * Hq), dim3(1024), 0, st, ma);
+        else if (nt == 512) hipLaunchKernelGGL((fused_middle_kernel<D, 512>), dim3(B * Hq), dim3(512), 0, st, ma);
+        else hipLaunchKernelGGL((fused_middle_kernel<D, 256>), dim3(B * Hq), dim3(256), 0, st, ma);
+    }
     int rc = check_launch("decode_step(middle)");
     if (rc != AKV_OK) return rc;
     if (literal_broadcast && !ref && R > 0) {
