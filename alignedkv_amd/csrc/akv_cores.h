@@ -146,6 +146,81 @@ __device__ __forceinline__ void pin_accumulators(float *a) {
                       "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15]));
 }
 
+// ------------------------------------------------------------------------------------------------
+// K with 256-token plane blocks (d_block == 256): scores of blocks [first_blk, end_blk) of one (batch, head).
+// A channel's row of a block is 256 B of high bytes and 128 B in each nibble plane, so a skipped nibble row is
+// a whole 128-byte line: HBM delivers exactly the bytes the levels ask for (with 64-token blocks a 32-byte row
+// shares its line with three other channels).
+//   Lane layout: lane -> channel 4 g + lane/16 of load group g (4 channels), slots (lane & 15) * 16 .. + 16.
+//   qf[g]: q of the lane's channel in group g; bit g of need_mid / need_last: fetch that plane row.
+//   valid_tokens: scores of tokens at and beyond it are not stored (the last block may be partly filled).
+// The 4 lanes of a slot range hold 16 partial sums each: two reduce-scatter steps (12 shuffles per 256 tokens,
+// against 15 per 64 tokens in the 64-token layout) leave 4 consecutive scores per lane.
+// ------------------------------------------------------------------------------------------------
+template <int D, int HG>
+__device__ __forceinline__ void k256_issue(KHalfTile<HG> &t, const __amdgpu_buffer_rsrc_t rH, const __amdgpu_buffer_rsrc_t rM,
+                                           const __amdgpu_buffer_rsrc_t rL, int blk, int g0, u32 need_mid, u32 need_last) {
+    const int lane = threadIdx.x & 63;
+    const int cs = lane >> 4, piece = lane & 15;
+#pragma unroll
+    for (int g = 0; g < HG; ++g) {
+        const int c = 4 * (g0 + g) + cs;
+        t.h[g] = __builtin_amdgcn_raw_buffer_load_b128(rH, blk * (D * 256) + c * 256 + piece * 16, 0, 0);
+    }
+#pragma unroll
+    for (int g = 0; g < HG; ++g) {
+        const int gg = g0 + g, c = 4 * gg + cs;
+        const int off = blk * (D * 128) + c * 128 + piece * 8;
+        t.m[g] = __builtin_amdgcn_raw_buffer_load_b64(rM, ((need_mid >> gg) & 1u) ? off : kSkip, 0, 0);
+        t.l[g] = __builtin_amdgcn_raw_buffer_load_b64(rL, ((need_last >> gg) & 1u) ? off : kSkip, 0, 0);
+    }
+}
+
+template <int D>
+__device__ __forceinline__ void k256_score_blocks(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_blocks,
+                                                  int first_blk, int end_blk, const float *qf, u32 need_mid, u32 need_last,
+                                                  unsigned short *s_row, int valid_tokens, float scale) {
+    constexpr int CB = 256;
+    constexpr int NG = D / 4;      // load groups of 4 channels
+    constexpr int HG = 4;          // groups per half tile: 8 KiB per wave in flight
+    static_assert(NG % (2 * HG) == 0 && NG <= 32, "head_dim 64 or 128");
+    const int lane = threadIdx.x & 63;
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_blocks * (D * CB));
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_blocks * (D * CB / 2));
+    const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_blocks * (D * CB / 2));
+    const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)valid_tokens * 2);
+    const int slot = (lane & 15) * 16 + ((lane & 32) ? 8 : 0) + ((lane & 16) ? 4 : 0);
+    KHalfTile<HG> ta, tb;
+    k256_issue<D, HG>(ta, rH, rM, rL, first_blk, 0, need_mid, need_last);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int blk = first_blk; blk < end_blk; ++blk) {
+        float acc[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int g0 = 0; g0 < NG; g0 += 2 * HG) {
+            k256_issue<D, HG>(tb, rH, rM, rL, blk, g0 + HG, need_mid, need_last);
+            __builtin_amdgcn_sched_barrier(0);
+            k_compute_half<HG>(acc, ta, g0, qf, need_mid, need_last);
+            pin_accumulators(acc);
+            __builtin_amdgcn_sched_barrier(0);
+            // past the last block the offsets fall outside the buffer resources: nothing is fetched
+            if (g0 + 2 * HG < NG) k256_issue<D, HG>(ta, rH, rM, rL, blk, g0 + 2 * HG, need_mid, need_last);
+            else k256_issue<D, HG>(ta, rH, rM, rL, blk + 1 < end_blk ? blk + 1 : n_blocks, 0, need_mid, need_last);
+            __builtin_amdgcn_sched_barrier(0);
+            k_compute_half<HG>(acc, tb, g0 + HG, qf, need_mid, need_last);
+            pin_accumulators(acc);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        reduce_scatter_step<16>(acc, 32);
+        reduce_scatter_step<8>(acc, 16);
+        const u32 w0 = (u32)float_to_half_bits(acc[0] * scale) | ((u32)float_to_half_bits(acc[1] * scale) << 16);
+        const u32 w1 = (u32)float_to_half_bits(acc[2] * scale) | ((u32)float_to_half_bits(acc[3] * scale) << 16);
+        // device scope: the workgroup that runs the softmax for this (batch, head) may sit on another XCD
+        __builtin_amdgcn_raw_buffer_store_b64((u32x2){w0, w1}, rS, (blk * CB + slot) * 2, 0, kDeviceScope);
+    }
+}
+
 template <int HV>
 struct VHalfTile {   // HV wave-wide loads: 64/(D/16) token rows each
     u32x4 h[HV];
@@ -386,6 +461,15 @@ inline VPlan v_plan(int B, int H, int D, int n_tokens) {
 
 inline int k_blocks_per_wave(int B, int H, int n_blocks) {
     // enough waves to fill 256 CUs several times over, a few blocks per wave to amortise set-up
+    int bpw = 1;
+    while (bpw < 4 && (int64_t)B * H * ((n_blocks + bpw * 2 - 1) / (bpw * 2)) >= 8192) bpw *= 2;
+    if (const char *e = getenv("AKV_TUNE_K_BPW")) bpw = atoi(e) > 0 ? atoi(e) : bpw;
+    return bpw;
+}
+
+
+inline int k256_blocks_per_wave(int B, int H, int n_blocks) {
+    // a wave streams 64 KiB per 256-token block: one block per wave unless that makes more than ~16 k waves
     int bpw = 1;
     while (bpw < 4 && (int64_t)B * H * ((n_blocks + bpw * 2 - 1) / (bpw * 2)) >= 8192) bpw *= 2;
     if (const char *e = getenv("AKV_TUNE_K_BPW")) bpw = atoi(e) > 0 ? atoi(e) : bpw;

@@ -26,14 +26,14 @@ namespace akv {
 __global__ __launch_bounds__(256) void k_save_blocks_kernel(
     uint8_t *__restrict__ first_8, uint8_t *__restrict__ mid_4, uint8_t *__restrict__ last_4,
     const unsigned short *__restrict__ k_new, int n_max_blocks, int H, int D, int cb, int tile_slots,
-    int tiles_per_block, int start_block, int seqlen) {
+    int start_pos, int n_tokens, int seqlen) {
     extern __shared__ unsigned short tile[];   // [tile_slots][D + 2]
     const int pitch = D + 2;
-    const int z = blockIdx.x / tiles_per_block, tile_id = blockIdx.x - z * tiles_per_block;
     const int h = blockIdx.y, b = blockIdx.z;
-    const int slot0 = tile_id * tile_slots;                       // first slot of this tile in the block
-    const int t0 = z * cb + slot0;                                // first source token
-    const int nv = min(min(tile_slots, cb - slot0), seqlen - t0); // valid tokens of this tile
+    const int t0 = blockIdx.x * tile_slots;                       // first source token of this tile
+    const int pos = start_pos + t0;                               // its position in the cache (a multiple of tile_slots)
+    const int z = pos / cb, slot0 = pos - z * cb;                 // destination block and first slot in it
+    const int nv = min(tile_slots, n_tokens - t0);                // valid tokens of this tile
     if (nv <= 0) return;
     const int halfD = D >> 1;
     const u32 *src32 = reinterpret_cast<const u32 *>(k_new);
@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256) void k_save_blocks_kernel(
         tile[j * pitch + 2 * dp + 1] = (unsigned short)(w >> 16);
     }
     __syncthreads();
-    const int64_t blk_base = (((int64_t)b * H + h) * n_max_blocks + (start_block + z)) * (int64_t)D * (cb >> 1);
+    const int64_t blk_base = (((int64_t)b * H + h) * n_max_blocks + z) * (int64_t)D * (cb >> 1);
     uint8_t *f8 = first_8 + blk_base * 2 + slot0;
     uint8_t *m4 = mid_4 + blk_base + (slot0 >> 1);
     uint8_t *l4 = last_4 + blk_base + (slot0 >> 1);
@@ -151,6 +151,43 @@ __global__ __launch_bounds__(256) void k_compute_cb64_kernel(
 }
 
 // ------------------------------------------------------------------------------------------------
+// k_cache_compute, tuned: d_block == 256 (see k256_score_blocks).
+// grid (ceil(n_blocks / (4*blocks_per_wave)), H, B), 256 threads (4 waves).
+// ------------------------------------------------------------------------------------------------
+template <int D, bool REF>
+__global__ __launch_bounds__(256) void k_compute_cb256_kernel(
+    const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
+    const uint8_t *__restrict__ sum_u8, const uint8_t *__restrict__ max_u8, const unsigned short *__restrict__ q,
+    unsigned short *__restrict__ s, uint8_t *__restrict__ levels_out, int n_blocks, int n_max_blocks, int H,
+    int blocks_per_wave, float scale) {
+    constexpr int CB = 256;
+    constexpr int NG = D / 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int bh = b * H + h;
+    const int first_blk = (blockIdx.x * 4 + wave) * blocks_per_wave;
+    if (first_blk >= n_blocks) return;
+    const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
+    const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
+    // per-lane channel data: channel of group g is 4 g + lane/16
+    float qf[NG];
+    u32 need_mid = 0, need_last = 0;
+    const unsigned char mx = REF ? 0 : max_u8[bh];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+        const int c = 4 * g + (lane >> 4);
+        qf[g] = half_bits_to_float(q[(int64_t)bh * D + c]);
+        const int lv = REF ? 0 : k_level(mx, sum_u8[(int64_t)bh * D + c]);
+        need_mid |= (lv < 2 ? 1u : 0u) << g;
+        need_last |= (lv == 0 ? 1u : 0u) << g;
+        if (levels_out != nullptr && blockIdx.x == 0 && wave == 0 && (lane & 15) == 0)
+            levels_out[(int64_t)bh * D + c] = (uint8_t)lv;
+    }
+    k256_score_blocks<D>(first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
+                         need_mid, need_last, s + (int64_t)bh * ((int64_t)(n_blocks + 1) * CB), n_blocks * CB, scale);
+}
+
+// ------------------------------------------------------------------------------------------------
 // k_cache_compute, any shape: one thread per slot pair, like the reference's launch
 // (extension/csrc/K_cache.cu:350-351) but with fp32 accumulation.
 // grid (n_blocks, H, B), d_block/2 threads.
@@ -193,6 +230,17 @@ static void launch_k_cb64(const uint8_t *f8, const uint8_t *m4, const uint8_t *l
                        n_blocks, n_max_blocks, H, bpw, scale);
 }
 
+template <int D, bool REF>
+static void launch_k_cb256(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *sum_u8,
+                           const uint8_t *max_u8, const uint8_t *q, uint8_t *s, uint8_t *levels, int B, int H,
+                           int n_blocks, int n_max_blocks, float scale, hipStream_t st) {
+    const int bpw = k256_blocks_per_wave(B, H, n_blocks);
+    dim3 grid((n_blocks + 4 * bpw - 1) / (4 * bpw), H, B);
+    hipLaunchKernelGGL((k_compute_cb256_kernel<D, REF>), grid, dim3(256), 0, st, f8, m4, l4, sum_u8, max_u8,
+                       reinterpret_cast<const unsigned short *>(q), reinterpret_cast<unsigned short *>(s), levels,
+                       n_blocks, n_max_blocks, H, bpw, scale);
+}
+
 }  // namespace akv
 
 using namespace akv;
@@ -209,20 +257,27 @@ int launch_k_save_blocks(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, cons
                 d_block, d_head);
     AKV_REQUIRE(start_pos >= 0 && seqlen >= 0 && n_blocks >= 0, "k_cache_save: negative start_pos/seqlen/n_blocks");
     AKV_REQUIRE(bsz <= 65535 && n_kv_heads <= 65535, "k_cache_save: bsz/heads exceed the grid limit 65535");
-    if (start_pos == 0 || seqlen % d_block == 0) {
+    const int tile_slots = d_block < 64 ? d_block : 64;
+    // Beyond the reference: a run of whole 64-token tiles appended inside a larger block (d_block a multiple of
+    // 64, start_pos and seqlen multiples of 64).  The reference launches nothing for this combination; the result
+    // here is that of seqlen calls of its single-token branch (extension/csrc/K_cache.cu:63-94,142-162).
+    const bool tile_append = start_pos != 0 && seqlen % d_block != 0 && seqlen > 1 && d_block % 64 == 0 &&
+                             start_pos % 64 == 0 && seqlen % 64 == 0;
+    if (start_pos == 0 || seqlen % d_block == 0 || tile_append) {
         if (n_blocks == 0) return AKV_OK;
-        const int start_block = start_pos / d_block;
-        AKV_REQUIRE((int64_t)(n_blocks - 1) * d_block < seqlen, "k_cache_save: n_blocks=%d needs more than seqlen=%d tokens",
+        AKV_REQUIRE(start_pos % tile_slots == 0, "k_cache_save: start_pos=%d is not a multiple of %d", start_pos, tile_slots);
+        // the reference's block branch stores the tokens of its first n_blocks blocks
+        const int n_tokens = tile_append ? seqlen : (int)min((int64_t)seqlen, (int64_t)n_blocks * d_block);
+        AKV_REQUIRE(tile_append || (int64_t)(n_blocks - 1) * d_block < seqlen, "k_cache_save: n_blocks=%d needs more than seqlen=%d tokens",
                     n_blocks, seqlen);
-        AKV_REQUIRE(start_block + n_blocks <= n_max_blocks, "k_cache_save: blocks %d..%d exceed n_max_blocks=%d",
-                    start_block, start_block + n_blocks, n_max_blocks);
-        const int tile_slots = d_block < 64 ? d_block : 64;
-        const int tiles_per_block = (d_block + tile_slots - 1) / tile_slots;
+        AKV_REQUIRE(((int64_t)start_pos + n_tokens + d_block - 1) / d_block <= n_max_blocks,
+                    "k_cache_save: tokens %d..%d exceed n_max_blocks=%d blocks of %d", start_pos, start_pos + n_tokens, n_max_blocks,
+                    d_block);
         size_t lds = (size_t)tile_slots * (d_head + 2) * sizeof(unsigned short);
         AKV_REQUIRE(lds <= 64 * 1024, "k_cache_save: d_head=%d too large for the staging tile (%zu bytes)", d_head, lds);
-        hipLaunchKernelGGL(k_save_blocks_kernel, dim3(n_blocks * tiles_per_block, n_kv_heads, bsz), dim3(256), lds, st,
-                           first_8, mid_4, last_4, reinterpret_cast<const unsigned short *>(k_new), n_max_blocks,
-                           n_kv_heads, d_head, d_block, tile_slots, tiles_per_block, start_block, seqlen);
+        hipLaunchKernelGGL(k_save_blocks_kernel, dim3((n_tokens + tile_slots - 1) / tile_slots, n_kv_heads, bsz), dim3(256), lds,
+                           st, first_8, mid_4, last_4, reinterpret_cast<const unsigned short *>(k_new), n_max_blocks,
+                           n_kv_heads, d_head, d_block, tile_slots, start_pos, n_tokens, seqlen);
         return check_launch("k_cache_save");
     }
     if (seqlen == 1) {
@@ -273,7 +328,15 @@ extern "C" int akv_k_cache_compute(const uint8_t *first_8, const uint8_t *mid_4,
     else                                                                                                         \
         launch_k_cb64<DD, false>(first_8, mid_4, last_4, sum_u8, max_u8, q, s_out, levels_out, bsz, n_kv_heads,  \
                                  n_blocks, n_max_blocks, scale, st);
-    if (d_block == 64 && d_head == 128) {
+    if (d_block == 256 && (d_head == 128 || d_head == 64)) {
+        if (d_head == 128) {
+            if (ref) launch_k_cb256<128, true>(first_8, mid_4, last_4, sum_u8, max_u8, q, s_out, levels_out, bsz, n_kv_heads, n_blocks, n_max_blocks, scale, st);
+            else launch_k_cb256<128, false>(first_8, mid_4, last_4, sum_u8, max_u8, q, s_out, levels_out, bsz, n_kv_heads, n_blocks, n_max_blocks, scale, st);
+        } else {
+            if (ref) launch_k_cb256<64, true>(first_8, mid_4, last_4, sum_u8, max_u8, q, s_out, levels_out, bsz, n_kv_heads, n_blocks, n_max_blocks, scale, st);
+            else launch_k_cb256<64, false>(first_8, mid_4, last_4, sum_u8, max_u8, q, s_out, levels_out, bsz, n_kv_heads, n_blocks, n_max_blocks, scale, st);
+        }
+    } else if (d_block == 64 && d_head == 128) {
         AKV_K_TUNED(128)
     } else if (d_block == 64 && d_head == 64) {
         AKV_K_TUNED(64)

@@ -109,7 +109,7 @@ def v_planes_alloc(bsz, n_heads, max_seq_len, head_dim):
             np.zeros((bsz, n_heads, max_seq_len, head_dim // 2), np.uint8))
 
 
-def k_cache_save(first_8, mid_4, last_4, k_new_bits, n_blocks, d_block, start_pos, seqlen):
+def k_cache_save(first_8, mid_4, last_4, k_new_bits, n_blocks, d_block, start_pos, seqlen, tile_append=False):
     """In-place plane write of K.  k_new_bits: uint16 [B, seqlen, H, D].
 
     Prefill branch (start_pos == 0 or seqlen % d_block == 0): blocks z < n_blocks, tokens
@@ -139,6 +139,11 @@ def k_cache_save(first_8, mid_4, last_4, k_new_bits, n_blocks, d_block, start_po
         first_8[:, :, blk, :, j] = hi[:, 0]
         mid_4[:, :, blk, :, j >> 1] += (mid[:, 0] << 4) >> ((j & 1) << 2)
         last_4[:, :, blk, :, j >> 1] += last[:, 0] << (4 - ((j & 1) << 2))
+    elif tile_append and d_block % 64 == 0 and start_pos % 64 == 0 and seqlen % 64 == 0:
+        # Not in the reference (it launches nothing here): whole 64-token tiles appended inside a larger block,
+        # defined as seqlen applications of the single-token branch above.
+        for i in range(seqlen):
+            k_cache_save(first_8, mid_4, last_4, k_new_bits[:, i:i + 1], 1, d_block, start_pos + i, 1)
 
 
 def v_cache_save(first_8, mid_4, last_4, v_new_bits, start_pos, seq_len):

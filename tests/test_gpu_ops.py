@@ -53,6 +53,23 @@ def test_k_cache_save_bit_exact(mod, B, H, D, cb, S, start_blk):
         assert np.array_equal(g.cpu().numpy(), w)
 
 
+def test_k_cache_save_tiles_inside_256_token_blocks(mod):
+    """Planes with d_block = 256 filled 64 tokens at a time: a prefill that ends inside a block, then appended tiles
+    (defined by the oracle as single-token saves of the reference's decoding branch)."""
+    B, H, D, cb = 2, 3, 128, 256
+    rng = np.random.default_rng(7)
+    kb = rng.integers(0, 65536, (B, 1024, H, D)).astype(np.uint16)
+    want = O.k_planes_alloc(B, H, 1024, D, cb)
+    got = k_planes_dev(B, H, 1024, D, cb)
+    O.k_cache_save(*want, kb[:, :576], 3, cb, 0, 576)                      # 2 blocks + one 64-token tile
+    mod.k_cache_save(*got, u8(kb[:, :576]), B, H, 3, 4, D, cb, 0, 576)
+    for start, n in ((576, 64), (640, 128), (768, 64)):
+        O.k_cache_save(*want, kb[:, start:start + n], 1, cb, start, n, tile_append=True)
+        mod.k_cache_save(*got, u8(kb[:, start:start + n]), B, H, 1, 4, D, cb, start, n)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.cpu().numpy(), w)
+
+
 def test_k_cache_save_single_token_branch(mod):
     rng = np.random.default_rng(1)
     B, H, D, cb = 2, 4, 128, 64
@@ -92,7 +109,8 @@ def _k_case(B, H, D, L, cb, seed, k_kind="outlier"):
 @pytest.mark.parametrize("reference", [False, True])
 @pytest.mark.parametrize("B,H,D,L,cb", [(2, 4, 128, 512, 64), (1, 8, 128, 1024, 64), (3, 2, 128, 320, 64),
                                         (2, 4, 64, 256, 64), (1, 2, 256, 192, 64), (2, 3, 16, 64, 16),
-                                        (1, 2, 128, 512, 128)])
+                                        (1, 2, 128, 512, 128), (2, 4, 128, 1024, 256), (1, 3, 64, 768, 256),
+                                        (3, 2, 128, 256, 256)])
 def test_k_cache_compute_parity(mod, B, H, D, L, cb, reference):
     q, planes, ksum, kmax = _k_case(B, H, D, L, cb, L + D)
     nb = L // cb
