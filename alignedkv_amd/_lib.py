@@ -25,7 +25,7 @@ SIGNATURES = {
     "akv_v_cache_test_compute": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
     "akv_v_cache_compute_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "akv_v_cache_compute": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, _I, _I, _I, _I, _I, _I, _I, _P]),
-    "akv_decode_step_gqa": (c_int, [_P] * 14 + [_I] + [_P] * 3 + [_I, _P, c_size_t] + [_P] * 3 + [_I] * 9 + [_P] + [_I] * 2 + [_P]),
+    "akv_decode_step_gqa": (c_int, [_P] * 14 + [_I] + [_P] * 3 + [_I, _P, c_size_t] + [_P] * 3 + [_I] * 10 + [_P] + [_I] * 2 + [_P]),
     "akv_dense_decode_step_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "akv_dense_decode_step": (c_int, [_P] * 8 + [_I, _P, c_size_t] + [_I] * 5 + [_P]),
     "akv_profile_enable": (c_int, [_I]),

@@ -152,7 +152,7 @@ __device__ __forceinline__ void pin_accumulators(float *a) {
 // a whole 128-byte line: HBM delivers exactly the bytes the levels ask for (with 64-token blocks a 32-byte row
 // shares its line with three other channels).
 //   Lane layout: lane -> channel 4 g + lane/16 of load group g (4 channels), slots (lane & 15) * 16 .. + 16.
-//   qf[g]: q of the lane's channel in group g; bit g of need_mid / need_last: fetch that plane row.
+//   bit g of need_mid / need_last: fetch that plane row of the lane's channel in group g.
 //   valid_tokens: scores of tokens at and beyond it are not stored (the last block may be partly filled).
 // The 4 lanes of a slot range hold 16 partial sums each: two reduce-scatter steps (12 shuffles per 256 tokens,
 // against 15 per 64 tokens in the 64-token layout) leave 4 consecutive scores per lane.
@@ -178,8 +178,9 @@ __device__ __forceinline__ void k256_issue(KHalfTile<HG> &t, const __amdgpu_buff
 
 template <int D>
 __device__ __forceinline__ void k256_score_blocks(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_blocks,
-                                                  int first_blk, int end_blk, const float *qf, u32 need_mid, u32 need_last,
+                                                  int first_blk, int end_blk, u32 *qh, u32 need_mid, u32 need_last,
                                                   unsigned short *s_row, int valid_tokens, float scale) {
+    // qh[g / 2]: q of the lane's channels of groups g (low half) and g + 1 (high half), fp16
     constexpr int CB = 256;
     constexpr int NG = D / 4;      // load groups of 4 channels
     constexpr int HG = 4;          // groups per half tile: 8 KiB per wave in flight
@@ -197,8 +198,20 @@ __device__ __forceinline__ void k256_score_blocks(const uint8_t *f8, const uint8
         float acc[16];
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+        // the substitution bytes derived from these masks are cheap to rebuild; kept across the loop they would
+        // take 64 registers: hide their loop invariance from the compiler
+        asm volatile("" : "+v"(need_mid), "+v"(need_last));
 #pragma unroll
         for (int g0 = 0; g0 < NG; g0 += 2 * HG) {
+            // q stays packed in registers (16 instead of 32): unpack the 8 values of this pair of half tiles
+            float qf[NG];
+#pragma unroll
+            for (int g = g0; g < g0 + 2 * HG; g += 2) {
+                u32 w = qh[g >> 1];
+                asm volatile("" : "+v"(w));
+                qf[g] = lo_half_to_float(w);
+                qf[g + 1] = hi_half_to_float(w);
+            }
             k256_issue<D, HG>(tb, rH, rM, rL, blk, g0 + HG, need_mid, need_last);
             __builtin_amdgcn_sched_barrier(0);
             k_compute_half<HG>(acc, ta, g0, qf, need_mid, need_last);

@@ -174,12 +174,14 @@ __global__ __launch_bounds__(256) void fused_pre_kernel(uint8_t *__restrict__ kf
         tile[j][2 * dp + 1] = (unsigned short)(w >> 16);
     }
     __syncthreads();
-    const int64_t base = ((int64_t)bh * geo.n_max_blocks + blk) * (int64_t)D * (CB / 2);
+    // the 64 tokens go to slots s0 .. s0 + 63 of K plane block kblk (blocks of geo.kb tokens)
+    const int KB = geo.kb, kblk = (blk * CB) / KB, s0 = blk * CB - kblk * KB;
+    const int64_t base = ((int64_t)bh * geo.n_max_blocks + kblk) * (int64_t)D * (KB / 2);
     for (int idx = threadIdx.x; idx < D * (CB / 4); idx += 256) {
         const int d = idx / (CB / 4), j = (idx - d * (CB / 4)) * 4;
         const u32 w = (u32)(tile[j][d] >> 8) | ((u32)(tile[j + 1][d] >> 8) << 8) | ((u32)(tile[j + 2][d] >> 8) << 16) |
                       ((u32)(tile[j + 3][d] >> 8) << 24);
-        *reinterpret_cast<u32 *>(kf8 + base * 2 + (int64_t)d * CB + j) = w;
+        *reinterpret_cast<u32 *>(kf8 + base * 2 + (int64_t)d * KB + s0 + j) = w;
     }
     for (int idx = threadIdx.x; idx < D * (CB / 8); idx += 256) {
         const int d = idx / (CB / 8), j = (idx - d * (CB / 8)) * 8;
@@ -190,8 +192,8 @@ __global__ __launch_bounds__(256) void fused_pre_kernel(uint8_t *__restrict__ kf
             mw |= ((le & 0xf0u) | (lo >> 4)) << (8 * i);
             lw |= (((le & 0x0fu) << 4) | (lo & 0x0fu)) << (8 * i);
         }
-        *reinterpret_cast<u32 *>(km4 + base + (int64_t)d * (CB / 2) + (j >> 1)) = mw;
-        *reinterpret_cast<u32 *>(kl4 + base + (int64_t)d * (CB / 2) + (j >> 1)) = lw;
+        *reinterpret_cast<u32 *>(km4 + base + (int64_t)d * (KB / 2) + ((s0 + j) >> 1)) = mw;
+        *reinterpret_cast<u32 *>(kl4 + base + (int64_t)d * (KB / 2) + ((s0 + j) >> 1)) = lw;
     }
 }
 
@@ -260,6 +262,56 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     }
     k_score_blocks<D>(ta, first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
                       need_mid, need_last, scores + (int64_t)bh * geo.row_stride, scale);
+}
+
+// K pass over planes with 256-token blocks (multi-head; see k256_score_blocks).
+// grid (ceil(n_kblocks / (4*blocks_per_wave)), H, B), 256 threads.
+template <int D, bool REF>
+__global__ __launch_bounds__(256) void fused_k_pass256_kernel(
+    const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
+    const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
+    unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, StepGeom geo, int blocks_per_wave,
+    float scale) {
+    constexpr int KB = 256;
+    constexpr int NG = D / 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int chunk, h, b;
+    if (!step_block(geo, chunk, h, b)) return;
+    const int bh = b * geo.Hq + h;
+    int R, nrest;
+    seq_state(geo, b, R, nrest);
+    const int n_blocks = (R + KB - 1) / KB;     // the last one may be partly filled
+    const int first_blk = (chunk * 4 + wave) * blocks_per_wave;
+    if (first_blk >= n_blocks && !(levels_out != nullptr && chunk == 0 && wave == 0)) return;
+    const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
+    const int64_t plane_off = (int64_t)bh * geo.n_max_blocks * (D * (KB / 2));
+    u32 qh[NG / 2];
+    u32 esum[NG];
+    u32 mx = 0;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+        const int c = 4 * g + (lane >> 4);
+        const u32 qb = q[(int64_t)bh * D + c];
+        if (g & 1) qh[g >> 1] |= qb << 16; else qh[g >> 1] = qb;
+        // column max including the token appended by this step
+        const u32 cm = max((u32)kcm[(int64_t)bh * D + c], exp_field(k_new[(int64_t)bh * D + c]));
+        esum[g] = (exp_field(qb) + cm) & 0xffu;
+        mx = max(mx, esum[g]);
+    }
+    mx = max(mx, (u32)__shfl_xor((int)mx, 16, 64));
+    mx = max(mx, (u32)__shfl_xor((int)mx, 32, 64));
+    u32 need_mid = 0, need_last = 0;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+        const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)esum[g]);
+        need_mid |= (lv < 2 ? 1u : 0u) << g;
+        need_last |= (lv == 0 ? 1u : 0u) << g;
+        if (levels_out != nullptr && chunk == 0 && wave == 0 && (lane & 15) == 0)
+            levels_out[(int64_t)bh * D + 4 * g + (lane >> 4)] = (uint8_t)lv;
+    }
+    if (first_blk >= n_blocks) return;
+    k256_score_blocks<D>(first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qh,
+                         need_mid, need_last, scores + (int64_t)bh * geo.row_stride, R, scale);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -803,7 +855,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
                     uint8_t *vcm, uint8_t *restk, uint8_t *restv, const uint8_t *q, const uint8_t *k_new,
                     const uint8_t *v_new, const uint8_t *mask, int mask_stride, uint8_t *out, uint8_t *scores,
                     uint8_t *probs, int row_stride, uint8_t *ws, uint8_t *k_levels_out, uint8_t *v_levels_out,
-                    uint8_t *amin_out, int B, int Hq, int Hkv, int n_max_blocks, int max_seq_len, int cb, int top_k,
+                    uint8_t *amin_out, int B, int Hq, int Hkv, int n_max_blocks, int max_seq_len, int cb, int kb, int top_k,
                     int cur_len, int *seq_lens, bool ref, int literal_broadcast, hipStream_t st) {
     const StepLayout lay = step_layout(B, Hq, D, max_seq_len);
     uint8_t *toe = ws + lay.toe;
@@ -821,6 +873,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     StepGeom geo;
     geo.Hq = Hq; geo.Hkv = Hkv; geo.G = Hq / Hkv;
     geo.cb = cb; geo.max_seq_len = max_seq_len; geo.n_max_blocks = n_max_blocks; geo.row_stride = row_stride;
+    geo.kb = kb;
     geo.cur_len = cur_len; geo.seq_lens = seq_lens;
     geo.task_map = nullptr;
 
@@ -834,7 +887,8 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     const bool grouped = group_heads(geo.G) > 1;
     bool matrix = geo.G >= 2 && geo.G <= 16 && D <= 128;   // (the 32-bit level masks hold 128 channels)
     if (const char *e = getenv("AKV_TUNE_MFMA")) matrix = matrix && atoi(e) != 0;
-    const int bpw = k_blocks_per_wave(B, Hq, n_blocks);
+    const int n_kblocks = (R + kb - 1) / kb;    // K plane blocks that hold tokens (the last one may be partly filled)
+    const int bpw = kb == 256 ? k256_blocks_per_wave(B, Hq, n_kblocks) : k_blocks_per_wave(B, Hq, n_blocks);
     bool matrix_v = matrix;
     if (const char *e = getenv("AKV_TUNE_MFMA_V")) matrix_v = matrix_v && atoi(e) != 0;
     VPlan p = v_plan(B, grouped ? Hq / group_heads(geo.G) : Hq, D, R);
@@ -853,7 +907,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
             int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo, B, n_blocks, ref, scale, st, &ks);
             if (rc != AKV_OK) return rc;
         } else {
-            ks = PassShape{group_grid_x((n_blocks + 4 * bpw - 1) / (4 * bpw), geo.G), Hkv, 4 * bpw * cb};
+            ks = PassShape{group_grid_x((n_kblocks + 4 * bpw - 1) / (4 * bpw), geo.G), Hkv, 4 * bpw * kb};
         }
         if (matrix_v) vs = PassShape{p.n_chunks, Hkv, p.chunk_tokens};
         else vs = PassShape{grouped ? p.n_chunks : group_grid_x(p.n_chunks, geo.G), grouped ? Hkv * (geo.G / group_heads(geo.G)) : Hkv,
@@ -892,7 +946,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
                            vcm, Hkv, D, cb, cur_len % cb);
         int rc = check_launch("decode_step(persist)");
         if (rc != AKV_OK) return rc;
-        rc = launch_k_save_blocks(kf8, km4, kl4, restk, B, Hkv, 1, n_max_blocks, D, cb, rest_start, cb, st);
+        rc = launch_k_save_blocks(kf8, km4, kl4, restk, B, Hkv, 1, n_max_blocks, D, kb, rest_start, cb, st);
         if (rc != AKV_OK) return rc;
         rc = launch_v_save(vf8, vm4, vl4, restv, B, Hkv, max_seq_len, D, rest_start, cb, cb, st);
         if (rc != AKV_OK) return rc;
@@ -910,7 +964,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     // measures level with the four launches at batch 8 x 32 heads x 4096 tokens on MI355X.
     bool mono = false;
     if (const char *e = getenv("AKV_TUNE_MONO")) mono = atoi(e) != 0;
-    mono = mono && n_blocks >= 1 && geo.G == 1 && !ragged && !(literal_broadcast && !ref);
+    mono = mono && n_blocks >= 1 && geo.G == 1 && !ragged && kb == 64 && !(literal_broadcast && !ref);
     if (mono) {
         if (ref)
             hipLaunchKernelGGL((mono_step_kernel<D, true>), dim3(B * Hq), dim3(1024), 0, st, kf8, km4, kl4, vf8, vm4, vl4,
@@ -936,6 +990,18 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
     } else if (n_blocks > 0 && grouped) {
         int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo_k, B, n_blocks, ref, scale, st);
+        if (rc != AKV_OK) return rc;
+    } else if (n_blocks > 0 && kb == 256) {
+        dim3 grid(ks.grid_x, ks.grid_y, B);
+        if constexpr (D <= 128) {
+            if (ref)
+                hipLaunchKernelGGL((fused_k_pass256_kernel<D, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
+                                   k_levels_out, geo_k, bpw, scale);
+            else
+                hipLaunchKernelGGL((fused_k_pass256_kernel<D, false>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
+                                   k_levels_out, geo_k, bpw, scale);
+        }
+        int rc = check_launch("decode_step(k_pass256)");
         if (rc != AKV_OK) return rc;
     } else if (n_blocks > 0) {
         dim3 grid(ks.grid_x, ks.grid_y, B);
@@ -1053,7 +1119,7 @@ extern "C" int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t
                                    uint8_t *out, uint8_t *scores, uint8_t *probs, int row_stride, void *workspace,
                                    size_t workspace_bytes, uint8_t *k_levels_out, uint8_t *v_levels_out,
                                    uint8_t *amin_out, int bsz, int n_q_heads, int n_kv_heads, int n_max_blocks,
-                                   int max_seq_len, int head_dim, int d_block, int top_max_k, int cur_len,
+                                   int max_seq_len, int head_dim, int d_block, int k_block, int top_max_k, int cur_len,
                                    int *seq_lens, int reference, int literal_broadcast, akv_stream_t stream) {
     AKV_REQUIRE(k_first_8 && k_mid_4 && k_last_4 && v_first_8 && v_mid_4 && v_last_4 && k_exp_column_max &&
                     v_exp_column_max && restk && restv && q && k_new && v_new && out && scores && probs && workspace,
@@ -1065,6 +1131,8 @@ extern "C" int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t
     AKV_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256,
                 "decode_step: head_dim %d not supported by the fused step (64, 128, 256); use the five ops", head_dim);
     AKV_REQUIRE(d_block == 64, "decode_step: d_block %d not supported by the fused step (64); use the five ops", d_block);
+    AKV_REQUIRE(k_block == 64 || (k_block == 256 && n_q_heads == n_kv_heads && head_dim <= 128),
+                "decode_step: k_block %d: K plane blocks are 64 tokens, or 256 for multi-head caches with head_dim 64 or 128", k_block);
     AKV_REQUIRE(top_max_k == 32, "decode_step: top_max_k %d not supported by the fused step (32)", top_max_k);
     AKV_REQUIRE(bsz <= 65535 && n_kv_heads <= 65535, "decode_step: bsz/heads exceed the grid limit 65535");
     AKV_REQUIRE(cur_len >= 0 && cur_len + 1 <= max_seq_len, "decode_step: cache full (%d of %d tokens)", cur_len, max_seq_len);
@@ -1073,13 +1141,13 @@ extern "C" int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t
     const int flushed = (cur_len + 1) / d_block * d_block;
     AKV_REQUIRE(flushed + d_block <= 65536 * 32, "decode_step: at most %d flushed tokens (16-bit group index of the probe)",
                 65536 * 32);
-    AKV_REQUIRE((int64_t)n_max_blocks * d_block >= flushed, "decode_step: K planes hold %d blocks, %d tokens flushed",
-                n_max_blocks, flushed);
+    AKV_REQUIRE((int64_t)n_max_blocks * k_block >= flushed, "decode_step: K planes hold %d blocks of %d, %d tokens flushed",
+                n_max_blocks, k_block, flushed);
     AKV_REQUIRE(row_stride % 8 == 0 && row_stride >= flushed + d_block,
                 "decode_step: row_stride %d must be a multiple of 8 and >= %d", row_stride, flushed + d_block);
     AKV_REQUIRE(mask == nullptr || mask_stride == 0 || mask_stride >= cur_len + 1,
                 "decode_step: mask row stride %d shorter than %d (0 = one row for all sequences)", mask_stride, cur_len + 1);
-    AKV_REQUIRE((int64_t)max_seq_len * head_dim < (int64_t)1 << 31 && (int64_t)n_max_blocks * head_dim * d_block < (int64_t)1 << 31,
+    AKV_REQUIRE((int64_t)max_seq_len * head_dim < (int64_t)1 << 31 && (int64_t)n_max_blocks * head_dim * k_block < (int64_t)1 << 31,
                 "decode_step: one (batch, head) slice of a high-byte plane must stay below 2 GiB");
     const size_t need = akv_decode_step_workspace_bytes(bsz, n_q_heads, head_dim, max_seq_len);
     AKV_REQUIRE(workspace_bytes >= need, "decode_step: workspace of %zu bytes, %zu needed", workspace_bytes, need);
@@ -1091,7 +1159,7 @@ extern "C" int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t
     return run_step<DD>(k_first_8, k_mid_4, k_last_4, v_first_8, v_mid_4, v_last_4, k_exp_column_max, v_exp_column_max, \
                         restk, restv, q, k_new, v_new, mask, mask_stride, out, scores, probs, row_stride, ws,          \
                         k_levels_out, v_levels_out, amin_out, bsz, n_q_heads, n_kv_heads, n_max_blocks, max_seq_len,   \
-                        d_block, top_max_k, cur_len, seq_lens, reference != 0, literal_broadcast, st);
+                        d_block, k_block, top_max_k, cur_len, seq_lens, reference != 0, literal_broadcast, st);
     if (head_dim == 64) { AKV_STEP(64) }
     if (head_dim == 128) { AKV_STEP(128) }
     AKV_STEP(256)
@@ -1113,6 +1181,6 @@ extern "C" int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_
     return akv_decode_step_gqa(k_first_8, k_mid_4, k_last_4, v_first_8, v_mid_4, v_last_4, k_exp_column_max,
                                v_exp_column_max, restk, restv, q, k_new, v_new, mask, mask_stride, out, scores, probs,
                                row_stride, workspace, workspace_bytes, k_levels_out, v_levels_out, amin_out, bsz,
-                               n_kv_heads, n_kv_heads, n_max_blocks, max_seq_len, head_dim, d_block, top_max_k, cur_len,
-                               nullptr, reference, literal_broadcast, stream);
+                               n_kv_heads, n_kv_heads, n_max_blocks, max_seq_len, head_dim, d_block, d_block, top_max_k,
+                               cur_len, nullptr, reference, literal_broadcast, stream);
 }

@@ -170,20 +170,21 @@ __global__ __launch_bounds__(256) void k_compute_cb256_kernel(
     const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
     const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
     // per-lane channel data: channel of group g is 4 g + lane/16
-    float qf[NG];
+    u32 qh[NG / 2];
     u32 need_mid = 0, need_last = 0;
     const unsigned char mx = REF ? 0 : max_u8[bh];
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
         const int c = 4 * g + (lane >> 4);
-        qf[g] = half_bits_to_float(q[(int64_t)bh * D + c]);
+        const u32 qb = q[(int64_t)bh * D + c];
+        if (g & 1) qh[g >> 1] |= qb << 16; else qh[g >> 1] = qb;
         const int lv = REF ? 0 : k_level(mx, sum_u8[(int64_t)bh * D + c]);
         need_mid |= (lv < 2 ? 1u : 0u) << g;
         need_last |= (lv == 0 ? 1u : 0u) << g;
         if (levels_out != nullptr && blockIdx.x == 0 && wave == 0 && (lane & 15) == 0)
             levels_out[(int64_t)bh * D + c] = (uint8_t)lv;
     }
-    k256_score_blocks<D>(first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
+    k256_score_blocks<D>(first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qh,
                          need_mid, need_last, s + (int64_t)bh * ((int64_t)(n_blocks + 1) * CB), n_blocks * CB, scale);
 }
 

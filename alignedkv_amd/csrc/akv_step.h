@@ -12,7 +12,8 @@ __device__ __forceinline__ u32 exp_field(u32 half_bits) { return (half_bits >> 1
 // cached before this step per sequence; without it every sequence has cur_len tokens.
 struct StepGeom {
     int Hq, Hkv, G;
-    int cb, max_seq_len, n_max_blocks, row_stride;
+    int cb, max_seq_len, n_max_blocks, row_stride;   // cb: tokens per flush; n_max_blocks: K plane blocks of kb tokens
+    int kb;                                          // tokens per K plane block (64 or 256)
     int cur_len;
     const int *seq_lens;
     const u32 *task_map;   // per-sequence lengths: workgroup -> (chunk, head index, batch) of this launch, or null

@@ -209,12 +209,13 @@ class _AlignedKVModule:
     def decode_step_gqa(self, k_planes, v_planes, k_exp_column_max, v_exp_column_max, restk, restv, q, k_new, v_new,
                         mask, out, scores, probs, bsz, n_q_heads, n_kv_heads, n_max_blocks, max_seq_len, head_dim,
                         d_block, top_max_k, cur_len, seq_lens, reference, k_levels_out=None, v_levels_out=None,
-                        amin_out=None):
+                        amin_out=None, k_block=None, literal_broadcast=False):
         """Fused step with grouped-query heads and optional per-sequence lengths (seq_lens: int32 device tensor
         [bsz], incremented by the step; cur_len then bounds them).  See akv_decode_step_gqa in include/alignedkv.h."""
         lib = load_library()
         dev = q.device
-        kplane = bsz * n_kv_heads * n_max_blocks * head_dim * d_block
+        k_block = d_block if k_block is None else k_block     # tokens per K plane block (n_max_blocks counts these)
+        kplane = bsz * n_kv_heads * n_max_blocks * head_dim * k_block
         vplane = bsz * n_kv_heads * max_seq_len * head_dim
         tok_q, tok_kv = bsz * n_q_heads * head_dim * 2, bsz * n_kv_heads * head_dim * 2
         for name, t, n in (("k_first_8", k_planes[0], kplane), ("k_mid_4", k_planes[1], kplane // 2),
@@ -254,8 +255,8 @@ class _AlignedKVModule:
                                           _ptr(v_new), _ptr(mask), mask_stride, _ptr(out), _ptr(scores), _ptr(probs),
                                           row_stride, _ptr(ws), ws.numel(), _ptr(k_levels_out), _ptr(v_levels_out),
                                           _ptr(amin_out), bsz, n_q_heads, n_kv_heads, n_max_blocks, max_seq_len,
-                                          head_dim, d_block, top_max_k, cur_len, _ptr(seq_lens),
-                                          int(bool(reference)), 0, _stream_ptr(dev)), lib)
+                                          head_dim, d_block, k_block, top_max_k, cur_len, _ptr(seq_lens),
+                                          int(bool(reference)), int(bool(literal_broadcast)), _stream_ptr(dev)), lib)
 
 
 cuda_module = _AlignedKVModule()

@@ -41,7 +41,7 @@ class QuantizedCache_AlignedKV(_HFCache):
     num_attention_heads, num_key_value_heads, hidden_size (or head_dim), max_position_embeddings."""
 
     def __init__(self, config, max_batch_size: int, max_cache_len: Optional[int], device, dtype=None,
-                 literal_colmax: bool = True, literal_broadcast: bool = False) -> None:
+                 literal_colmax: bool = True, literal_broadcast: bool = False, k_block: int = 64) -> None:
         try:
             super().__init__()
         except Exception:
@@ -58,7 +58,7 @@ class QuantizedCache_AlignedKV(_HFCache):
         self.value_cache: List[V_Cache_Class] = []
         for idx in range(config.num_hidden_layers):
             self.key_cache.append(K_Cache_Class(max_batch_size, self.max_cache_len, self.num_key_value_heads,
-                                                self.head_dim, idx, device, register, literal_colmax))
+                                                self.head_dim, idx, device, register, literal_colmax, k_block))
             self.value_cache.append(V_Cache_Class(max_batch_size, self.max_cache_len, self.num_key_value_heads,
                                                   self.head_dim, idx, device, register, 32, literal_colmax,
                                                   literal_broadcast))
@@ -141,14 +141,25 @@ class QuantizedCache_AlignedKV(_HFCache):
             klv = torch.empty((B, H, D), dtype=torch.uint8, device=q.device)
             vlv = torch.empty((B, H, flushed), dtype=torch.uint8, device=q.device) if flushed else None
             amin = torch.empty((B, H), dtype=torch.uint8, device=q.device)
-        cuda_module.decode_step(
-            (kc.k_cache_first_8, kc.k_cache_mid_4, kc.k_cache_last_4),
-            (vc.v_cache_first_8, vc.v_cache_mid_4, vc.v_cache_last_4),
-            kc._colmax, vc._colmax, kc._rest.view(torch.uint8), vc._rest.view(torch.uint8),
-            q.view(torch.uint8), k.view(torch.uint8), v.view(torch.uint8), mask2d, out.view(torch.uint8),
-            self._scores.view(torch.uint8), self._probs.view(torch.uint8), B, H, kc.n_max_blocks, self.max_cache_len,
-            D, column_block, vc.top_max_k, start_pos, kc.reststartpos, kc._restlen, self.reference,
-            self.literal_broadcast, klv, vlv, amin)
+        if kc.k_block == column_block:
+            cuda_module.decode_step(
+                (kc.k_cache_first_8, kc.k_cache_mid_4, kc.k_cache_last_4),
+                (vc.v_cache_first_8, vc.v_cache_mid_4, vc.v_cache_last_4),
+                kc._colmax, vc._colmax, kc._rest.view(torch.uint8), vc._rest.view(torch.uint8),
+                q.view(torch.uint8), k.view(torch.uint8), v.view(torch.uint8), mask2d, out.view(torch.uint8),
+                self._scores.view(torch.uint8), self._probs.view(torch.uint8), B, H, kc.n_max_blocks, self.max_cache_len,
+                D, column_block, vc.top_max_k, start_pos, kc.reststartpos, kc._restlen, self.reference,
+                self.literal_broadcast, klv, vlv, amin)
+        else:
+            assert kc.reststartpos + kc._restlen == start_pos
+            cuda_module.decode_step_gqa(
+                (kc.k_cache_first_8, kc.k_cache_mid_4, kc.k_cache_last_4),
+                (vc.v_cache_first_8, vc.v_cache_mid_4, vc.v_cache_last_4),
+                kc._colmax, vc._colmax, kc._rest.view(torch.uint8), vc._rest.view(torch.uint8),
+                q.view(torch.uint8), k.view(torch.uint8), v.view(torch.uint8), mask2d, out.view(torch.uint8),
+                self._scores.view(torch.uint8), self._probs.view(torch.uint8), B, H, H, kc.k_n_max_blocks,
+                self.max_cache_len, D, column_block, vc.top_max_k, start_pos, None, self.reference, klv, vlv, amin,
+                k_block=kc.k_block, literal_broadcast=self.literal_broadcast)
         kc._advance_after_fused_step()
         vc._advance_after_fused_step()
         kc.last_levels, vc.last_levels, vc.last_alignment_min = klv, vlv, amin

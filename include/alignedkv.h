@@ -164,6 +164,10 @@ AKV_API int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_las
  * n_kv_heads).  seq_lens != NULL: device int32 [bsz], tokens cached per sequence before the step; cur_len is
  * then an upper bound of them (it sizes the launches), a sequence flushes its rest buffer on the step that
  * fills it, and the step increments every entry of seq_lens on the device.
+ * k_block: tokens per block of the K planes, [bsz, n_kv_heads, n_max_blocks, head_dim, k_block] (the d_block of
+ * akv_k_cache_save / akv_k_cache_compute).  64 is the reference's layout.  256 (multi-head, head_dim 64 or 128)
+ * makes a channel's nibble row a whole 128-byte line, so a skipped row saves exactly its bytes in HBM traffic;
+ * tokens still enter the planes 64 at a time (d_block, the length of the rest buffers), as whole tiles inside a block.
  */
 AKV_API int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,
                                 uint8_t *v_mid_4, uint8_t *v_last_4, uint8_t *k_exp_column_max,
@@ -172,7 +176,7 @@ AKV_API int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k
                                 uint8_t *out, uint8_t *scores, uint8_t *probs, int row_stride, void *workspace,
                                 size_t workspace_bytes, uint8_t *k_levels_out, uint8_t *v_levels_out, uint8_t *amin_out,
                                 int bsz, int n_q_heads, int n_kv_heads, int n_max_blocks, int max_seq_len, int head_dim,
-                                int d_block, int top_max_k, int cur_len, int *seq_lens, int reference,
+                                int d_block, int k_block, int top_max_k, int cur_len, int *seq_lens, int reference,
                                 int literal_broadcast, akv_stream_t stream);
 
 /*

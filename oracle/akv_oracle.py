@@ -409,6 +409,7 @@ class OracleCache:
     n_heads: int
     head_dim: int
     d_block: int = COLUMN_BLOCK
+    k_block: int = COLUMN_BLOCK      # tokens per block of the K planes (a multiple of d_block, the flush unit)
     top_max_k: int = TOP_MAX_K
     literal_colmax: bool = True
     literal_broadcast: bool = False
@@ -425,7 +426,7 @@ class OracleCache:
     last: dict = field(default_factory=dict, repr=False)   # intermediates of the last decode step
 
     def __post_init__(self):
-        self.k_planes = k_planes_alloc(self.bsz, self.n_heads, self.max_seq_len, self.head_dim, self.d_block)
+        self.k_planes = k_planes_alloc(self.bsz, self.n_heads, self.max_seq_len, self.head_dim, self.k_block)
         self.v_planes = v_planes_alloc(self.bsz, self.n_heads, self.max_seq_len, self.head_dim)
         shp = (self.bsz, 1, self.n_heads, self.head_dim)
         self.k_colmax = np.zeros(shp, np.uint8)
@@ -444,7 +445,11 @@ class OracleCache:
         if start_pos == 0:
             self.k_colmax = colmax_prefill(k, self.literal_colmax)
             self.v_colmax = colmax_prefill(v, self.literal_colmax)
-            k_cache_save(*self.k_planes, as_bits(k), seqlen // cb, cb, 0, seqlen)
+            if self.k_block == cb:
+                k_cache_save(*self.k_planes, as_bits(k), seqlen // cb, cb, 0, seqlen)
+            elif seqlen - seqlen % cb:
+                n = seqlen - seqlen % cb      # whole 64-token tiles; the last block may stay partly filled
+                k_cache_save(*self.k_planes, as_bits(k[:, :n]), cdiv(n, self.k_block), self.k_block, 0, n)
             v_cache_save(*self.v_planes, as_bits(v), 0, seqlen - seqlen % cb)
             r = seqlen % cb
             self.restk = np.zeros((self.bsz, cb, self.n_heads, self.head_dim), np.float16)
@@ -460,7 +465,10 @@ class OracleCache:
             self.restv[:, self.rest_len:self.rest_len + 1] = v
             self.rest_len += 1
             if self.rest_len == cb:
-                k_cache_save(*self.k_planes, as_bits(self.restk), 1, cb, self.rest_start, cb)
+                if self.k_block == cb or self.rest_start == 0:
+                    k_cache_save(*self.k_planes, as_bits(self.restk), 1, self.k_block, self.rest_start, cb)
+                else:
+                    k_cache_save(*self.k_planes, as_bits(self.restk), 1, self.k_block, self.rest_start, cb, tile_append=True)
                 v_cache_save(*self.v_planes, as_bits(self.restv), self.rest_start, cb)
                 self.rest_len = 0
                 self.rest_start += cb
@@ -478,10 +486,10 @@ class OracleCache:
         self.save(k_half, v_half, start_pos, 1)
         L = start_pos + 1
         R = self.rest_start
-        nb = R // cb
+        nb = cdiv(R, self.k_block)
         # K side: extension/k_cache_file.py:132-159
         ksum, kmax = k_sum_and_max(q, self.k_colmax)
-        s, klv = k_cache_compute(*self.k_planes, ksum, kmax, as_bits(q), nb, cb,
+        s, klv = k_cache_compute(*self.k_planes, ksum, kmax, as_bits(q), nb, self.k_block,
                                  1.0 / math.sqrt(D), self.reference, return_levels=True)
         assert self.rest_len + R == L
         if self.rest_len:

@@ -33,17 +33,18 @@ def planes_equal(cache, oc, layer=0):
 
 
 @pytest.mark.parametrize("fused", [True, False])
-@pytest.mark.parametrize("prefill,steps,literal_broadcast", [(200, 70, False), (64, 3, False), (1, 66, False),
-                                                             (130, 5, True)])
-def test_cache_matches_oracle_step_by_step(prefill, steps, literal_broadcast, fused):
+@pytest.mark.parametrize("prefill,steps,literal_broadcast,k_block", [(200, 70, False, 64), (64, 3, False, 64), (1, 66, False, 64),
+                                                                     (130, 5, True, 64), (200, 70, False, 256), (1, 66, False, 256),
+                                                                     (700, 72, False, 256), (512, 3, True, 256)])
+def test_cache_matches_oracle_step_by_step(prefill, steps, literal_broadcast, k_block, fused):
     from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
     B, H, D = 2, 4, 128
     Lmax = prefill + steps + 10
     q_all, k, v = make_qkv(B, prefill + steps, H, D, seed=prefill)
     rng = np.random.default_rng(prefill)
-    cache = QuantizedCache_AlignedKV(cfg(H, D), B, Lmax, "cuda", torch.half, literal_broadcast=literal_broadcast)
+    cache = QuantizedCache_AlignedKV(cfg(H, D), B, Lmax, "cuda", torch.half, literal_broadcast=literal_broadcast, k_block=k_block)
     cache.fused = fused
-    oc = O.OracleCache(B, Lmax, H, D, literal_broadcast=literal_broadcast)
+    oc = O.OracleCache(B, Lmax, H, D, literal_broadcast=literal_broadcast, k_block=k_block)
     kc, vc = cache.key_cache[0], cache.value_cache[0]
     kc.record_levels = vc.record_levels = True
     # prefill: dense attention + plane writes

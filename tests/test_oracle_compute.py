@@ -156,13 +156,14 @@ def test_colmax_literal_vs_abs():
     assert upd.reshape(-1).tolist() == [19, 14]
 
 
-@pytest.mark.parametrize("prefill,steps", [(1, 70), (63, 3), (64, 2), (130, 66), (200, 1)])
-def test_cache_state_machine_and_reference_mode_matches_dense(prefill, steps):
+@pytest.mark.parametrize("prefill,steps,k_block", [(1, 70, 64), (63, 3, 64), (64, 2, 64), (130, 66, 64), (200, 1, 64),
+                                                   (1, 70, 256), (200, 130, 256), (320, 2, 256)])
+def test_cache_state_machine_and_reference_mode_matches_dense(prefill, steps, k_block):
     B, H, D = 2, 4, 32
     L = prefill + steps
     q, k, v = make_qkv(B, L, H, D, prefill, n_outliers=0)
     rng = np.random.default_rng(9)
-    c = O.OracleCache(B, L + 3, H, D, reference=True)
+    c = O.OracleCache(B, L + 3, H, D, reference=True, k_block=k_block)
     c.save(k[:, :prefill], v[:, :prefill], 0, prefill)
     for t in range(prefill, L):
         qt = rng.standard_normal((B, 1, H, D)).astype(np.float16)
@@ -172,9 +173,9 @@ def test_cache_state_machine_and_reference_mode_matches_dense(prefill, steps):
         assert np.max(np.abs(o.astype(np.float32) - want)) <= 5e-3   # half-rounded scale + fp16 scores
     # planes hold exactly the first rest_start tokens, whatever mix of prefill and flushes wrote them
     R = c.rest_start
-    one = O.OracleCache(B, L + 3, H, D)
+    one = O.OracleCache(B, L + 3, H, D, k_block=k_block)
     if R:
-        O.k_cache_save(*one.k_planes, O.as_bits(k[:, :R]), R // 64, 64, 0, R)
+        O.k_cache_save(*one.k_planes, O.as_bits(k[:, :R]), O.cdiv(R, k_block), k_block, 0, R)
         O.v_cache_save(*one.v_planes, O.as_bits(v[:, :R]), 0, R)
     for a, b in zip(c.k_planes + c.v_planes, one.k_planes + one.v_planes):
         assert np.array_equal(a, b)
