@@ -158,8 +158,7 @@ __device__ __forceinline__ void pin_accumulators(float *a) {
 // against 15 per 64 tokens in the 64-token layout) leave 4 consecutive scores per lane.
 // ------------------------------------------------------------------------------------------------
 template <int D, int HG>
-__device__ __forceinline__ void k256_issue(KHalfTile<HG> &t, const __amdgpu_buffer_rsrc_t rH, const __amdgpu_buffer_rsrc_t rM,
-                                           const __amdgpu_buffer_rsrc_t rL, int blk, int g0, u32 need_mid, u32 need_last) {
+__device__ __forceinline__ void k256_issue_h(KHalfTile<HG> &t, const __amdgpu_buffer_rsrc_t rH, int blk, int g0) {
     const int lane = threadIdx.x & 63;
     const int cs = lane >> 4, piece = lane & 15;
 #pragma unroll
@@ -167,6 +166,13 @@ __device__ __forceinline__ void k256_issue(KHalfTile<HG> &t, const __amdgpu_buff
         const int c = 4 * (g0 + g) + cs;
         t.h[g] = __builtin_amdgcn_raw_buffer_load_b128(rH, blk * (D * 256) + c * 256 + piece * 16, 0, 0);
     }
+}
+
+template <int D, int HG>
+__device__ __forceinline__ void k256_issue_ml(KHalfTile<HG> &t, const __amdgpu_buffer_rsrc_t rM, const __amdgpu_buffer_rsrc_t rL,
+                                              int blk, int g0, u32 need_mid, u32 need_last) {
+    const int lane = threadIdx.x & 63;
+    const int cs = lane >> 4, piece = lane & 15;
 #pragma unroll
     for (int g = 0; g < HG; ++g) {
         const int gg = g0 + g, c = 4 * gg + cs;
@@ -176,8 +182,23 @@ __device__ __forceinline__ void k256_issue(KHalfTile<HG> &t, const __amdgpu_buff
     }
 }
 
+template <int D, int HG>
+__device__ __forceinline__ void k256_issue(KHalfTile<HG> &t, const __amdgpu_buffer_rsrc_t rH, const __amdgpu_buffer_rsrc_t rM,
+                                           const __amdgpu_buffer_rsrc_t rL, int blk, int g0, u32 need_mid, u32 need_last) {
+    k256_issue_h<D, HG>(t, rH, blk, g0);
+    k256_issue_ml<D, HG>(t, rM, rL, blk, g0, need_mid, need_last);
+}
+
+// The high-byte rows of the wave's first half tile do not depend on the fetch levels: a kernel calls this first,
+// works out q and the levels while the loads are in flight, then calls k256_score_blocks.
 template <int D>
-__device__ __forceinline__ void k256_score_blocks(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_blocks,
+__device__ __forceinline__ void k256_prefetch_first(KHalfTile<4> &ta, const uint8_t *f8, int n_blocks, int first_blk) {
+    k256_issue_h<D, 4>(ta, make_rsrc(f8, (u32)n_blocks * (D * 256)), first_blk, 0);
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <int D>
+__device__ __forceinline__ void k256_score_blocks(KHalfTile<4> &ta, const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_blocks,
                                                   int first_blk, int end_blk, u32 *qh, u32 need_mid, u32 need_last,
                                                   unsigned short *s_row, int valid_tokens, float scale) {
     // qh[g / 2]: q of the lane's channels of groups g (low half) and g + 1 (high half), fp16
@@ -191,8 +212,8 @@ __device__ __forceinline__ void k256_score_blocks(const uint8_t *f8, const uint8
     const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_blocks * (D * CB / 2));
     const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)valid_tokens * 2);
     const int slot = (lane & 15) * 16 + ((lane & 32) ? 8 : 0) + ((lane & 16) ? 4 : 0);
-    KHalfTile<HG> ta, tb;
-    k256_issue<D, HG>(ta, rH, rM, rL, first_blk, 0, need_mid, need_last);
+    KHalfTile<HG> tb;
+    k256_issue_ml<D, HG>(ta, rM, rL, first_blk, 0, need_mid, need_last);   // its high bytes: k256_prefetch_first
     __builtin_amdgcn_sched_barrier(0);
     for (int blk = first_blk; blk < end_blk; ++blk) {
         float acc[16];

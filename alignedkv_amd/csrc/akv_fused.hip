@@ -236,17 +236,24 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     const int64_t plane_off = (int64_t)bh_kv * geo.n_max_blocks * (D * (CB / 2));
     KHalfTile<D / 32> ta;
     k_prefetch_first<D>(ta, first_8 + plane_off * 2, n_blocks, first_blk);
+    // q and the exponent sums of all channels, staged once per workgroup (three scattered global loads per
+    // channel and wave otherwise: half as many load instructions again as the planes themselves need)
+    __shared__ u32 staged[D];      // [channel]: q bits | exponent sum << 16
+    for (int c = threadIdx.x; c < D; c += 256) {
+        const u32 qb = q[(int64_t)bh * D + c];
+        // column max including the token appended by this step
+        const u32 cm = max((u32)kcm[(int64_t)bh_kv * D + c], exp_field(k_new[(int64_t)bh_kv * D + c]));
+        staged[c] = qb | (((exp_field(qb) + cm) & 0xffu) << 16);
+    }
+    __syncthreads();
     float qf[NG];
     u32 esum[NG];
     u32 mx = 0;
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
-        const int c = g * 16 + (lane >> 2);
-        const u32 qb = q[(int64_t)bh * D + c];
-        qf[g] = half_bits_to_float(qb);
-        // column max including the token appended by this step
-        const u32 cm = max((u32)kcm[(int64_t)bh_kv * D + c], exp_field(k_new[(int64_t)bh_kv * D + c]));
-        esum[g] = (exp_field(qb) + cm) & 0xffu;
+        const u32 w = staged[g * 16 + (lane >> 2)];
+        qf[g] = lo_half_to_float(w);
+        esum[g] = w >> 16;
         mx = max(mx, esum[g]);
     }
 #pragma unroll
@@ -281,21 +288,30 @@ __global__ __launch_bounds__(256) void fused_k_pass256_kernel(
     int R, nrest;
     seq_state(geo, b, R, nrest);
     const int n_blocks = (R + KB - 1) / KB;     // the last one may be partly filled
-    const int first_blk = (chunk * 4 + wave) * blocks_per_wave;
-    if (first_blk >= n_blocks && !(levels_out != nullptr && chunk == 0 && wave == 0)) return;
+    const int first_blk = (chunk * 4 + wave) * blocks_per_wave;    // may lie past the end: the wave then only helps staging
     const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
     const int64_t plane_off = (int64_t)bh * geo.n_max_blocks * (D * (KB / 2));
+    KHalfTile<4> ta;
+    k256_prefetch_first<D>(ta, first_8 + plane_off * 2, n_blocks, first_blk);
+    // q and the exponent sums of all channels, staged once per workgroup: every lane needs 32 of them (channels
+    // 4 g + lane/16), and 96 scattered global loads per wave would double the pass's load instructions
+    __shared__ u32 staged[D];      // [channel]: q bits | exponent sum << 16
+    for (int c = threadIdx.x; c < D; c += 256) {
+        const u32 qb = q[(int64_t)bh * D + c];
+        // column max including the token appended by this step
+        const u32 cm = max((u32)kcm[(int64_t)bh * D + c], exp_field(k_new[(int64_t)bh * D + c]));
+        staged[c] = qb | (((exp_field(qb) + cm) & 0xffu) << 16);
+    }
+    __syncthreads();
     u32 qh[NG / 2];
     u32 esum[NG];
     u32 mx = 0;
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
-        const int c = 4 * g + (lane >> 4);
-        const u32 qb = q[(int64_t)bh * D + c];
+        const u32 w = staged[4 * g + (lane >> 4)];
+        const u32 qb = w & 0xffffu;
         if (g & 1) qh[g >> 1] |= qb << 16; else qh[g >> 1] = qb;
-        // column max including the token appended by this step
-        const u32 cm = max((u32)kcm[(int64_t)bh * D + c], exp_field(k_new[(int64_t)bh * D + c]));
-        esum[g] = (exp_field(qb) + cm) & 0xffu;
+        esum[g] = w >> 16;
         mx = max(mx, esum[g]);
     }
     mx = max(mx, (u32)__shfl_xor((int)mx, 16, 64));
@@ -310,7 +326,7 @@ __global__ __launch_bounds__(256) void fused_k_pass256_kernel(
             levels_out[(int64_t)bh * D + 4 * g + (lane >> 4)] = (uint8_t)lv;
     }
     if (first_blk >= n_blocks) return;
-    k256_score_blocks<D>(first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qh,
+    k256_score_blocks<D>(ta, first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qh,
                          need_mid, need_last, scores + (int64_t)bh * geo.row_stride, R, scale);
 }
 

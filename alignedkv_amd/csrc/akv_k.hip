@@ -169,6 +169,8 @@ __global__ __launch_bounds__(256) void k_compute_cb256_kernel(
     if (first_blk >= n_blocks) return;
     const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
     const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
+    KHalfTile<4> ta;
+    k256_prefetch_first<D>(ta, first_8 + plane_off * 2, n_blocks, first_blk);
     // per-lane channel data: channel of group g is 4 g + lane/16
     u32 qh[NG / 2];
     u32 need_mid = 0, need_last = 0;
@@ -184,7 +186,7 @@ __global__ __launch_bounds__(256) void k_compute_cb256_kernel(
         if (levels_out != nullptr && blockIdx.x == 0 && wave == 0 && (lane & 15) == 0)
             levels_out[(int64_t)bh * D + c] = (uint8_t)lv;
     }
-    k256_score_blocks<D>(first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qh,
+    k256_score_blocks<D>(ta, first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qh,
                          need_mid, need_last, s + (int64_t)bh * ((int64_t)(n_blocks + 1) * CB), n_blocks * CB, scale);
 }
 

@@ -29,7 +29,8 @@ HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the K pass at the default workload, from the rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs summarised in profiles/decode_step_c2_hbm_traffic.txt (FETCH_SIZE scaled x2.0 by the
 # known-size copy kernel, WRITE_SIZE x1.0): 222.4 MiB read + 2.0 MiB written.
-MEASURED_K_PASS_TRAFFIC = {(8, 32, 128, 4096, "outlier"): int((222.4 + 2.0) * (1 << 20))}
+MEASURED_K_PASS_TRAFFIC = {(8, 32, 128, 4096, "outlier", 64): int((222.4 + 2.0) * (1 << 20)),
+                           (8, 32, 128, 4096, "outlier", 256): int((198.5 + 2.0) * (1 << 20))}
 
 
 def parse():
@@ -43,6 +44,8 @@ def parse():
     ap.add_argument("--cache-len", type=int, default=4096)
     ap.add_argument("--layers", type=int, default=4, help="caches the steps rotate over")
     ap.add_argument("--k-kind", default="outlier", choices=["outlier", "lognormal"])
+    ap.add_argument("--k-block", type=int, default=64, choices=[64, 256],
+                    help="tokens per block of the K planes: 64 = the reference's layout, 256 = whole 128-byte lines per nibble row")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=10)
     ap.add_argument("--seed", type=int, default=0)
@@ -70,7 +73,8 @@ def make_layer_inputs(torch, B, L, H, D, seed, k_kind):
 
 
 class StepRunner:
-    """Pre-marshalled akv_decode_step call for one layer at a fixed state (cur_len = cache_len)."""
+    """Pre-marshalled akv_decode_step_gqa call (multi-head, uniform length) for one layer at a fixed state
+    (cur_len = cache_len)."""
 
     def __init__(self, torch, lib, cache, layer, q, k_new, v_new, out, reference, record):
         from alignedkv_amd.extension._plane_cache import column_block
@@ -91,12 +95,12 @@ class StepRunner:
         self.args = [p(kc.k_cache_first_8), p(kc.k_cache_mid_4), p(kc.k_cache_last_4), p(vc.v_cache_first_8),
                      p(vc.v_cache_mid_4), p(vc.v_cache_last_4), p(kc._colmax), p(vc._colmax), p(kc._rest), p(vc._rest),
                      p(q), p(k_new), p(v_new), None, 0, p(out), p(self.scores), p(self.probs), width, p(self.ws),
-                     self.ws.numel(), p(self.k_levels), p(self.v_levels), p(self.amin), B, H, kc.n_max_blocks,
-                     cache.max_cache_len, D, column_block, vc.top_max_k, kc.current_cache_len, kc.reststartpos,
-                     kc._restlen, int(reference), 0, torch.cuda.current_stream().cuda_stream]
+                     self.ws.numel(), p(self.k_levels), p(self.v_levels), p(self.amin), B, H, H, kc.k_n_max_blocks,
+                     cache.max_cache_len, D, column_block, kc.k_block, vc.top_max_k, kc.current_cache_len, None,
+                     int(reference), 0, torch.cuda.current_stream().cuda_stream]
 
     def __call__(self):
-        rc = self.lib.akv_decode_step(*self.args)
+        rc = self.lib.akv_decode_step_gqa(*self.args)
         if rc != 0:
             raise RuntimeError(self.lib.akv_last_error().decode())
 
@@ -159,8 +163,8 @@ def cpu_baseline(torch, cache, q, k_new, v_new, n_steps):
     from oracle import akv_oracle_c as OC
     kc, vc = cache.key_cache[0], cache.value_cache[0]
     B, H, D = cache.max_batch_size, cache.num_key_value_heads, cache.head_dim
-    R, cb = kc.reststartpos, 64
-    nb = R // cb
+    R, cb, kb = kc.reststartpos, 64, kc.k_block
+    nb = (R + kb - 1) // kb
     kp = [t.cpu().numpy() for t in (kc.k_cache_first_8, kc.k_cache_mid_4, kc.k_cache_last_4)]
     vp = [t.cpu().numpy() for t in (vc.v_cache_first_8, vc.v_cache_mid_4, vc.v_cache_last_4)]
     kcm, vcm = kc._colmax.cpu().numpy(), vc._colmax.cpu().numpy()
@@ -173,7 +177,7 @@ def cpu_baseline(torch, cache, q, k_new, v_new, n_steps):
         kcm2 = O.colmax_update(kcm, kn)
         vcm2 = O.colmax_update(vcm, vn)
         ksum, kmax = O.k_sum_and_max(qn, kcm2)
-        s, klv = OC.k_cache_compute(*kp, ksum, kmax, O.as_bits(qn), nb, cb, 1.0 / math.sqrt(D), False)
+        s, klv = OC.k_cache_compute(*kp, ksum, kmax, O.as_bits(qn), nb, kb, 1.0 / math.sqrt(D), False)
         s = s.copy()
         restk = np.zeros((B, cb, H, D), np.float16)
         restv = np.zeros((B, cb, H, D), np.float16)
@@ -301,7 +305,7 @@ def main():
     assert L % 64 == 0, "the cache length of the benchmark must be a multiple of the 64-token flush block"
     cfg = SimpleNamespace(num_hidden_layers=a.layers, num_attention_heads=H, num_key_value_heads=H, hidden_size=H * D,
                           max_position_embeddings=L + 64)
-    cache = QuantizedCache_AlignedKV(cfg, B, L + 64, "cuda", torch.half)
+    cache = QuantizedCache_AlignedKV(cfg, B, L + 64, "cuda", torch.half, k_block=a.k_block)
     for layer in range(a.layers):
         k, v = make_layer_inputs(torch, B, L, H, D, a.seed + layer, a.k_kind)
         cache.key_cache[layer].save(k, 0, L)
@@ -356,8 +360,8 @@ def main():
         "value": round(us, 2), "unit": "us/step", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(us / 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "C2: batch %d, %d heads x %d, cache %d + 1 appended token, K %s, %d layers rotated"
-                               % (B, H, D, L, a.k_kind, a.layers)},
+        "config": {"workload": "C2: batch %d, %d heads x %d, cache %d + 1 appended token, K %s, %d layers rotated, K plane blocks of %d tokens"
+                               % (B, H, D, L, a.k_kind, a.layers, a.k_block)},
         "effective_hbm_gbps": round(eff_gbps, 1), "pct_hbm_peak": round(100 * eff_gbps / HBM_PEAK_GBPS, 1),
         "algorithmic_bytes": int(by["total"]), "dense_fp16_bytes": int(by["dense"]),
         "bytes_vs_dense": round(by["total"] / by["dense"], 4),
@@ -368,9 +372,9 @@ def main():
         "v_pass_gbps": round(v_pass_bytes / (ph[2] * 1e-6) / 1e9, 1),
         "dense_in_planes_us": round(sec_ref * 1e6, 2),
         "speedup_vs_dense_in_planes": round(sec_ref / sec, 3),
-        "roofline": {"kernel": "fused_k_pass_kernel<128,false>", "bound": "hbm", "achieved": round(achieved, 1),
+        "roofline": {"kernel": "fused_k_pass_kernel<128,false>" if a.k_block == 64 else "fused_k_pass256_kernel<128,false>", "bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_K_PASS_TRAFFIC.get((B, H, D, L, a.k_kind)), "algorithmic_bytes_per_launch": int(k_pass_bytes),
+                     "traffic": MEASURED_K_PASS_TRAFFIC.get((B, H, D, L, a.k_kind, a.k_block)), "algorithmic_bytes_per_launch": int(k_pass_bytes),
                      "avg_launch_us": round(ph[0], 2), "event_pair_overhead_us": round(event_pair_us, 2)},
     }
     if copy_gbps is not None:
