@@ -27,10 +27,10 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
 
 # HBM bytes per launch of the K pass at the default workload, from the rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs summarised in profiles/decode_step_c2_hbm_traffic.txt (FETCH_SIZE scaled x2.0 by the
+# WRITE_SIZE runs summarised in profiles/decode_step_c2_hbm_traffic.txt (256-token K blocks) and decode_step_c2_k_block64_hbm_traffic.txt (FETCH_SIZE scaled x2.0 by the
 # known-size copy kernel, WRITE_SIZE x1.0): 222.4 MiB read + 2.0 MiB written.
 MEASURED_K_PASS_TRAFFIC = {(8, 32, 128, 4096, "outlier", 64): int((222.4 + 2.0) * (1 << 20)),
-                           (8, 32, 128, 4096, "outlier", 256): int((198.5 + 2.0) * (1 << 20))}
+                           (8, 32, 128, 4096, "outlier", 256): int((197.9 + 2.0) * (1 << 20))}
 
 
 def parse():
@@ -44,8 +44,9 @@ def parse():
     ap.add_argument("--cache-len", type=int, default=4096)
     ap.add_argument("--layers", type=int, default=4, help="caches the steps rotate over")
     ap.add_argument("--k-kind", default="outlier", choices=["outlier", "lognormal"])
-    ap.add_argument("--k-block", type=int, default=64, choices=[64, 256],
-                    help="tokens per block of the K planes: 64 = the reference's layout, 256 = whole 128-byte lines per nibble row")
+    ap.add_argument("--k-block", type=int, default=256, choices=[64, 256],
+                    help="tokens per block of the K planes (the ops' d_block): 256 = a nibble row is a whole 128-byte line, "
+                         "64 = the block length the reference's Python classes use")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=10)
     ap.add_argument("--seed", type=int, default=0)
@@ -283,7 +284,9 @@ def bench_c3(a):
            "effective_hbm_gbps": round(kv_bytes / sec / 1e9, 1), "pct_hbm_peak": round(100 * kv_bytes / sec / 1e9 / HBM_PEAK_GBPS, 1),
            "kernel_us": {"k_pass": round(acc[0], 2), "middle": round(acc[1], 2), "v_pass": round(acc[2], 2),
                          "combine": round(acc[3], 2)},
-           "dense_in_planes_us": round(sec_ref * 1e6, 2), "speedup_vs_dense_in_planes": round(sec_ref / sec, 3)}
+           "k_block": a.k_block, "other_k_block_us": {"k_block": other_kb, "us_per_step": round(sec_other * 1e6, 2),
+                                                   "max_abs_diff_of_outputs": layout_diff},
+        "dense_in_planes_us": round(sec_ref * 1e6, 2), "speedup_vs_dense_in_planes": round(sec_ref / sec, 3)}
     print(json.dumps(res))
 
 
@@ -355,6 +358,20 @@ def main():
     ref_runners = [StepRunner(torch, lib, cache, i, q, k_new, v_new, out, True, False) for i in range(a.layers)]
     sec_ref = time_steps(torch, ref_runners, max(a.steps // 2, 20), 10)
 
+    # the same step with the other K plane block length (same inputs)
+    other_kb = 64 if a.k_block == 256 else 256
+    cache2 = QuantizedCache_AlignedKV(cfg, B, L + 64, "cuda", torch.half, k_block=other_kb)
+    for layer in range(a.layers):
+        k, v = make_layer_inputs(torch, B, L, H, D, a.seed + layer, a.k_kind)
+        cache2.key_cache[layer].save(k, 0, L)
+        cache2.value_cache[layer].save(v, 0, L)
+        del k, v
+    out2 = torch.empty_like(q)
+    runners2 = [StepRunner(torch, lib, cache2, i, q, k_new, v_new, out2, False, False) for i in range(a.layers)]
+    sec_other = time_steps(torch, runners2, max(a.steps // 2, 20), 10)
+    layout_diff = float((out2.float() - out_aligned.float()).abs().max())   # summation order differs, levels do not
+    del cache2, runners2
+
     res = {
         "metric": "decode-attn us/step (+ effective HBM GB/s, %% of peak), B=%d L=%d %dx%d" % (B, L, H, D),
         "value": round(us, 2), "unit": "us/step", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -370,6 +387,8 @@ def main():
         "kernel_us": {"k_pass": round(ph[0], 2), "middle": round(ph[1], 2), "v_pass": round(ph[2], 2),
                       "combine": round(ph[3], 2)},
         "v_pass_gbps": round(v_pass_bytes / (ph[2] * 1e-6) / 1e9, 1),
+        "k_block": a.k_block, "other_k_block_us": {"k_block": other_kb, "us_per_step": round(sec_other * 1e6, 2),
+                                                   "max_abs_diff_of_outputs": layout_diff},
         "dense_in_planes_us": round(sec_ref * 1e6, 2),
         "speedup_vs_dense_in_planes": round(sec_ref / sec, 3),
         "roofline": {"kernel": "fused_k_pass_kernel<128,false>" if a.k_block == 64 else "fused_k_pass256_kernel<128,false>", "bound": "hbm", "achieved": round(achieved, 1),
