@@ -57,6 +57,9 @@ AKV_API const char *akv_last_error(void);
  * 0 .. min(n_blocks*d_block, seqlen) of k_new.  Otherwise, seqlen == 1: inserts one token at slot
  * start_pos % d_block of block start_pos / d_block.  Nibble bytes are written, not accumulated
  * (identical to the reference's `+=` on zero-initialised planes).  Needs d_block % 8 == 0, d_head % 2 == 0.
+ * Beyond the reference (which launches nothing for it): start_pos != 0, seqlen % d_block != 0, with d_block,
+ * start_pos and seqlen multiples of 64 -- whole 64-token tiles appended inside a block, the result of seqlen
+ * single-token inserts.  Used by caches whose K planes have 256-token blocks and a 64-token rest buffer.
  */
 AKV_API int akv_k_cache_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8_t *k_new,
                      int bsz, int n_kv_heads, int n_blocks, int n_max_blocks, int d_head, int d_block,
