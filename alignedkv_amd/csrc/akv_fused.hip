@@ -1032,8 +1032,9 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     }
     mark(1, st);
     {
-        // threads per (batch, head) row: 512 and 1024 measure level with 256 at batch 8 x 32 heads x 4096 tokens
-        int nt = 256;
+        // threads per (batch, head) row: a thread keeps 32 scores in registers between the softmax passes, so
+        // rows above 8192 / 16384 tokens get 512 / 1024 threads (512 and 1024 measure level with 256 at 4096 tokens)
+        int nt = R <= 8192 ? 256 : (R <= 16384 ? 512 : 1024);
         if (const char *e = getenv("AKV_TUNE_MIDDLE_NT")) nt = atoi(e);
         if (nt == 1024) hipLaunchKernelGGL((fused_middle_kernel<D, 1024>), dim3(B * Hq), dim3(1024), 0, st, ma);
         else if (nt == 512) hipLaunchKernelGGL((fused_middle_kernel<D, 512>), dim3(B * Hq), dim3(512), 0, st, ma);
