@@ -100,6 +100,12 @@ class StepRunner:
                      cache.max_cache_len, D, column_block, kc.k_block, vc.top_max_k, kc.current_cache_len, None,
                      int(reference), 0, torch.cuda.current_stream().cuda_stream]
 
+        self.cur_len_index = len(self.args) - 5
+
+    def at_length(self, cur_len):
+        self.args[self.cur_len_index] = cur_len
+        return self
+
     def __call__(self):
         rc = self.lib.akv_decode_step_gqa(*self.args)
         if rc != 0:
@@ -411,6 +417,17 @@ def main():
                                          % a.cpu_steps}
         res["parity"] = {"max_abs_err_vs_oracle": err, "k_levels_equal": bool(np.array_equal(cklv, k_levels)),
                          "v_level_mismatches": int((cvlv != v_levels).sum()), "v_levels_total": int(v_levels.size)}
+    # 64 consecutive decode steps per layer (the cache grows from L to L + 64: the rest buffer fills up and is
+    # flushed once), averaged: what a generation loop sees, against `value` which repeats the first of them
+    if L % 64 == 0:
+        grow = [StepRunner(torch, lib, cache, i, q, k_new, v_new, out, False, False) for i in range(a.layers)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for sidx in range(64):
+            for r in grow:
+                r.at_length(L + sidx)()
+        torch.cuda.synchronize()
+        res["avg_us_over_64_growing_steps"] = round((time.perf_counter() - t0) / (64 * a.layers) * 1e6, 2)
     print(json.dumps(res))
 
 
