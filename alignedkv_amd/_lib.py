@@ -28,6 +28,7 @@ SIGNATURES = {
     "akv_decode_step_gqa": (c_int, [_P] * 14 + [_I] + [_P] * 3 + [_I, _P, c_size_t] + [_P] * 3 + [_I] * 10 + [_P] + [_I] * 2 + [_P]),
     "akv_dense_decode_step_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "akv_dense_decode_step": (c_int, [_P] * 8 + [_I, _P, c_size_t] + [_I] * 5 + [_P]),
+    "akv_reload_tuning": (c_int, []),
     "akv_profile_enable": (c_int, [_I]),
     "akv_copy_probe": (c_int, [_P, _P, c_size_t, _P]),
     "akv_profile_read": (c_int, [_P]),

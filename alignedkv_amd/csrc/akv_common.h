@@ -5,6 +5,7 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 
 #include "../../include/alignedkv.h"
 
@@ -17,6 +18,28 @@ namespace akv {
 // ---- host-side error reporting -------------------------------------------------------------
 void set_error(const char *fmt, ...);
 int check_launch(const char *what);
+
+// Tuning switches from the environment (AKV_TUNE_*), read once per call site and again after
+// akv_reload_tuning(): a getenv per switch and step costs a few microseconds of host time per decode step,
+// which is what a batch-1 step is bound by.
+extern int g_tune_epoch;
+struct TuneVar {
+    const char *name;
+    int epoch;
+    bool present;
+    int value;
+    bool get(int &out) {
+        if (epoch != g_tune_epoch) {
+            const char *e = getenv(name);
+            present = e != nullptr;
+            value = e != nullptr ? atoi(e) : 0;
+            epoch = g_tune_epoch;
+        }
+        out = value;
+        return present;
+    }
+};
+#define AKV_TUNE(NAME, VAR) static akv::TuneVar tune_##VAR = {NAME, -1, false, 0}; int VAR = 0; const bool has_##VAR = tune_##VAR.get(VAR)
 
 #define AKV_REQUIRE(cond, ...)            \
     do {                                   \

@@ -902,11 +902,11 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     // or up to 16 on the matrix cores (K pass)
     const bool grouped = group_heads(geo.G) > 1;
     bool matrix = geo.G >= 2 && geo.G <= 16 && D <= 128;   // (the 32-bit level masks hold 128 channels)
-    if (const char *e = getenv("AKV_TUNE_MFMA")) matrix = matrix && atoi(e) != 0;
+    { AKV_TUNE("AKV_TUNE_MFMA", v); if (has_v) matrix = matrix && v != 0; }
     const int n_kblocks = (R + kb - 1) / kb;    // K plane blocks that hold tokens (the last one may be partly filled)
     const int bpw = kb == 256 ? k256_blocks_per_wave(B, Hq, n_kblocks) : k_blocks_per_wave(B, Hq, n_blocks);
     bool matrix_v = matrix;
-    if (const char *e = getenv("AKV_TUNE_MFMA_V")) matrix_v = matrix_v && atoi(e) != 0;
+    { AKV_TUNE("AKV_TUNE_MFMA_V", v); if (has_v) matrix_v = matrix_v && v != 0; }
     VPlan p = v_plan(B, grouped ? Hq / group_heads(geo.G) : Hq, D, R);
     if constexpr (D <= 128) {
         if (matrix_v) p = mfma_v_plan<D>(B, Hkv, R);
@@ -979,7 +979,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     // One launch for the whole step: opt-in (AKV_TUNE_MONO=1), multi-head uniform-length caches only.  It
     // measures level with the four launches at batch 8 x 32 heads x 4096 tokens on MI355X.
     bool mono = false;
-    if (const char *e = getenv("AKV_TUNE_MONO")) mono = atoi(e) != 0;
+    { AKV_TUNE("AKV_TUNE_MONO", v); if (has_v) mono = v != 0; }
     mono = mono && n_blocks >= 1 && geo.G == 1 && !ragged && kb == 64 && !(literal_broadcast && !ref);
     if (mono) {
         if (ref)
@@ -1035,7 +1035,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         // threads per (batch, head) row: a thread keeps 32 scores in registers between the softmax passes, so
         // rows above 8192 / 16384 tokens get 512 / 1024 threads (512 and 1024 measure level with 256 at 4096 tokens)
         int nt = R <= 8192 ? 256 : (R <= 16384 ? 512 : 1024);
-        if (const char *e = getenv("AKV_TUNE_MIDDLE_NT")) nt = atoi(e);
+        { AKV_TUNE("AKV_TUNE_MIDDLE_NT", v); if (has_v) nt = v; }
         if (nt == 1024) hipLaunchKernelGGL((fused_middle_kernel<D, 1024>), dim3(B * Hq), dim3(1024), 0, st, ma);
         else if (nt == 512) hipLaunchKernelGGL((fused_middle_kernel<D, 512>), dim3(B * Hq), dim3(512), 0, st, ma);
         else hipLaunchKernelGGL((fused_middle_kernel<D, 256>), dim3(B * Hq), dim3(256), 0, st, ma);

@@ -350,12 +350,12 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
                        uint8_t *levels_out, u32 *prep, const StepGeom &geo, int B, int n_blocks, bool ref, float scale,
                        hipStream_t st, PassShape *shape_only) {
     int sl = 8;
-    if (const char *e = getenv("AKV_TUNE_K_SL")) sl = atoi(e) == 16 ? 16 : (atoi(e) == 4 ? 4 : 8);
+    { AKV_TUNE("AKV_TUNE_K_SL", v); if (has_v) sl = v == 16 ? 16 : (v == 4 ? 4 : 8); }
     const int nbt = sl / 4;
     const int n_tasks = (n_blocks + nbt - 1) / nbt;
     int tpw = 1;
     while (tpw < 8 && (int64_t)B * geo.Hkv * ((n_tasks + 8 * tpw - 1) / (8 * tpw)) * 4 >= 8192) tpw *= 2;
-    if (const char *e = getenv("AKV_TUNE_K_TPW")) tpw = atoi(e) > 0 ? atoi(e) : tpw;
+    { AKV_TUNE("AKV_TUNE_K_TPW", v); if (has_v && v > 0) tpw = v; }
     if (shape_only != nullptr) {
         *shape_only = PassShape{(n_tasks + 4 * tpw - 1) / (4 * tpw), geo.Hkv, 4 * tpw * nbt * 64};
         return AKV_OK;
@@ -376,7 +376,7 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
     hipLaunchKernelGGL((mfma_k_pass_kernel<D, RF, SLL, AH>), grid, dim3(256), 0, st, f8, m4, l4, prep, scores, geo, tpw, \
                        scale, (u32)scores_bytes)
     int ahead = 3;
-    if (const char *e = getenv("AKV_TUNE_K_AHEAD")) ahead = atoi(e);
+    { AKV_TUNE("AKV_TUNE_K_AHEAD", v); if (has_v) ahead = v; }
     constexpr int DEEP = (D / 16) % 8 == 0 ? 7 : 3;
     if (sl == 16) { if (ref) AKV_MK(true, 16, 1); else AKV_MK(false, 16, 1); }
     else if (sl == 8 && ahead == 7) { if (ref) AKV_MK(true, 8, DEEP); else AKV_MK(false, 8, DEEP); }
@@ -603,7 +603,7 @@ VPlan mfma_v_plan(int B, int Hkv, int n_tokens) {
     p.tuned = true;
     int k = 1;   // macro steps of 64 tokens per wave
     while (k < 4 && (int64_t)B * Hkv * ((n_tokens + 512 * k - 1) / (512 * k)) >= 2048) k *= 2;
-    if (const char *e = getenv("AKV_TUNE_V_ITERS")) k = atoi(e) > 0 ? atoi(e) : k;
+    { AKV_TUNE("AKV_TUNE_V_ITERS", v); if (has_v && v > 0) k = v; }
     p.iters_per_wave = k;
     p.tokens_per_wave = 64 * k;
     p.chunk_tokens = 4 * p.tokens_per_wave;

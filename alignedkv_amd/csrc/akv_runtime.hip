@@ -23,7 +23,14 @@ int check_launch(const char *what) {
     return AKV_OK;
 }
 
+int g_tune_epoch = 0;
+
 }  // namespace akv
+
+extern "C" int akv_reload_tuning(void) {
+    ++akv::g_tune_epoch;
+    return AKV_OK;
+}
 
 // Plain streaming copy, 16 bytes per thread and iteration: the known-size kernel that hardware byte
 // counters of the other kernels are scaled against.

@@ -199,6 +199,8 @@ AKV_API int akv_dense_decode_step(uint8_t *k_cache, uint8_t *v_cache, const uint
  * events on its stream around its four phases; akv_profile_read waits for the last recorded step and
  * returns the elapsed milliseconds of {K pass, middle, V pass, combine}.  Process-wide, not thread safe.
  */
+/* The AKV_TUNE_* environment switches are read when first used; call this after changing one in a running process. */
+AKV_API int akv_reload_tuning(void);
 AKV_API int akv_profile_enable(int enable);
 /* Plain device copy of `bytes` bytes (multiple of 16): the known-size kernel hardware byte counters are scaled against. */
 AKV_API int akv_copy_probe(void *dst, const void *src, size_t bytes, akv_stream_t stream);

@@ -217,11 +217,15 @@ def test_one_launch_step_matches_the_four_launch_step(monkeypatch, reference):
         c.value_cache[0].save(dev(v[:, :prefill]), 0, prefill)
         c.key_cache[0].record_levels = c.value_cache[0].record_levels = True
         caches.append(c)
+    from alignedkv_amd import load_library
+    lib = load_library()
     for t in range(prefill, prefill + steps):
         qt = dev(rng.standard_normal((B, 1, H, D)).astype(np.float16))
         monkeypatch.setenv("AKV_TUNE_MONO", "0")
+        lib.akv_reload_tuning()      # the switches are read once and again after this call
         o4 = caches[0].auto_compute(qt, dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None)
         monkeypatch.setenv("AKV_TUNE_MONO", "1")
+        lib.akv_reload_tuning()
         o1 = caches[1].auto_compute(qt, dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None)
         assert (o4.float() - o1.float()).abs().max().item() <= 1e-3
         for name in ("last_levels",):
@@ -232,3 +236,5 @@ def test_one_launch_step_matches_the_four_launch_step(monkeypatch, reference):
     k0, k1 = caches[0].key_cache[0], caches[1].key_cache[0]
     assert torch.equal(k0.k_cache_first_8, k1.k_cache_first_8) and torch.equal(k0.k_cache_last_4, k1.k_cache_last_4)
     assert k0.reststartpos == k1.reststartpos == (prefill + steps) // 64 * 64
+    monkeypatch.delenv("AKV_TUNE_MONO")
+    lib.akv_reload_tuning()
