@@ -398,13 +398,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     const unsigned short *mrow = a.mask ? a.mask + (int64_t)b * a.mask_stride : nullptr;
     const int nvec = R >> 3;
     const bool in_regs = nvec <= NT * VPT;
-#ifdef AKV_DEBUG_TS
-    unsigned long long *mts = reinterpret_cast<unsigned long long *>(a.toe) + 2 * 1024 * 1024 / 8 + (int64_t)bh * 16;
-#define AKV_MTS(i) if (threadIdx.x == 0) mts[i] = wall_clock64();
-#else
-#define AKV_MTS(i)
-#endif
-    AKV_MTS(0)
     // scores of the flushed part are read at device scope: other workgroups of the same launch wrote them
     const __amdgpu_buffer_rsrc_t rScores = make_rsrc(srow, (u32)R * 2);
 
@@ -470,7 +463,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
         }
     }
     lds_barrier();
-    AKV_MTS(1)
 
     // (c) softmax over [0, R + nrest): scores + mask in fp16, softmax in fp32, probabilities in fp16
     //     (model/KVCache_AlignedKV.py:119-121), and the running arg-max of the residue classes mod 32:
@@ -499,9 +491,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
                 for (int j = 0; j < 8; ++j) m = fmaxf(m, x[v][j]);
             }
         }
-        AKV_MTS(2)
         m = block_reduce<NW>(m, true, red);
-        AKV_MTS(3)
 #pragma unroll
         for (int v = 0; v < VPT; ++v)
             if (tid + NT * v < nvec) {
@@ -513,7 +503,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
             }
         const float et = tid < nrest ? expf(xt - m) : 0.f;
         sum = block_reduce<NW>(sum + et, false, red);
-        AKV_MTS(4)
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
             const int i = tid + NT * v;
@@ -573,7 +562,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
         }
     }
 
-    AKV_MTS(5)
     // (d)+(e) probe over the flushed part (extension/v_cache_file.py:119-143) and the alignment threshold
     //     of this (batch, head) (extension/v_cache_file.py:156-160)
     if (R > 0) {
@@ -586,13 +574,11 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
             best[j] = max(best[j], (u32)__shfl_xor((int)best[j], 16, 64));
             best[j] = max(best[j], (u32)__shfl_xor((int)best[j], 32, 64));
         }
-        AKV_MTS(8)
         if (lane < 4) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) cand_key[wave][8 * lane + j] = best[j];
         }
         lds_barrier();
-        AKV_MTS(9)
         if (tid < 32) {
             u32 key = 0u;
 #pragma unroll
@@ -601,7 +587,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
             probe_t[tid] = (int)(0xffffu - (key & 0xffffu)) * 32 + tid;
         }
         lds_barrier();
-        AKV_MTS(6)
         u32 align = 0xffu;
         for (int d = tid; d < D; d += NT) {
             // the 32 gathered bytes first, then the sum: 32 independent loads in flight instead of a chain
@@ -630,7 +615,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     } else {
         lds_barrier();
     }
-    AKV_MTS(7)
     // (f) the tail's share of the output, an fp16 matmul result (extension/v_cache_file.py:189): a thread takes 8
     //     channels of every NRG-th tail token, lanes of a wave that share the channels fold by shuffles, waves by LDS
     {
@@ -697,10 +681,6 @@ __global__ __launch_bounds__(1024) void mono_step_kernel(
     __shared__ float wave_part[NW][D];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int bh = blockIdx.x;
-#ifdef AKV_DEBUG_TS
-    unsigned long long *ts = reinterpret_cast<unsigned long long *>(ma.toe) + 1024 * 1024 / 8 + (int64_t)bh * 8;
-    if (threadIdx.x == 0) ts[0] = wall_clock64();
-#endif
     // ---- K pass: wave w scores blocks [w*bpw, (w+1)*bpw)
     {
         // wave w takes blocks w, w + 16, ...: at any time the 16 waves stream 16 neighbouring blocks
@@ -737,16 +717,10 @@ __global__ __launch_bounds__(1024) void mono_step_kernel(
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
-#ifdef AKV_DEBUG_TS
-    if (threadIdx.x == 0) ts[1] = wall_clock64();
-#endif
     // ---- middle: append, tail scores, softmax, probe, threshold, tail output
     middle_body<D, NT>(ma, bh);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
-#ifdef AKV_DEBUG_TS
-    if (threadIdx.x == 0) ts[2] = wall_clock64();
-#endif
     // ---- V pass: wave w accumulates tokens [w*tpw, (w+1)*tpw)
     int R, nrest_unused;
     seq_state(ma.g, bh / ma.g.Hq, R, nrest_unused);
@@ -765,9 +739,6 @@ __global__ __launch_bounds__(1024) void mono_step_kernel(
     }
     v_fold_lanes<D, NW>(acc, wave_part);
     __syncthreads();
-#ifdef AKV_DEBUG_TS
-    if (threadIdx.x == 0) { ts[3] = wall_clock64(); ts[4] = __smid(); }
-#endif
     for (int d = threadIdx.x; d < D; d += NT) {
         float sum = 0.f;
 #pragma unroll
