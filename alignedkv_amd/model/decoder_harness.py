@@ -146,12 +146,12 @@ class RandomLlamaDecoder(torch.nn.Module):
         return torch.stack(toks, dim=1), torch.stack(all_logits, dim=0)
 
 
-def make_cache(kind: str, cfg: DecoderConfig, bsz: int, max_len: int, device="cuda"):
+def make_cache(kind: str, cfg: DecoderConfig, bsz: int, max_len: int, device="cuda", k_block: int = 64):
     """kind: 'alignedkv' (fused step), 'alignedkv_ops' (the reference's op sequence), 'alignedkv_reference'
     (every plane read), 'dense_torch'."""
     if kind == "dense_torch":
         return DenseTorchCache(cfg.num_hidden_layers)
-    c = QuantizedCache_AlignedKV(cfg, bsz, max_len, device, torch.half)
+    c = QuantizedCache_AlignedKV(cfg, bsz, max_len, device, torch.half, k_block=k_block)
     c.reference = kind == "alignedkv_reference"
     if kind == "alignedkv_ops":
         c.fused = False
@@ -169,13 +169,14 @@ def main():
     ap.add_argument("--prefill", type=int, default=128)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--kinds", default="dense_torch,alignedkv_reference,alignedkv")
+    ap.add_argument("--k-block", type=int, default=64, help="tokens per block of the K planes (64 or 256)")
     a = ap.parse_args()
     cfg = DecoderConfig(a.layers, a.hidden, a.heads, a.heads, a.ffn, a.vocab, max_position_embeddings=a.prefill + a.steps + 64)
     model = RandomLlamaDecoder(cfg)
     prompt = torch.randint(0, a.vocab, (a.batch, a.prefill), device="cuda", generator=torch.Generator(device="cuda").manual_seed(1))
     base_tokens = base_logits = None
     for kind in a.kinds.split(","):
-        cache = make_cache(kind, cfg, a.batch, a.prefill + a.steps + 64)
+        cache = make_cache(kind, cfg, a.batch, a.prefill + a.steps + 64, k_block=a.k_block)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         toks, logits = model.generate(prompt, a.steps, cache, forced_tokens=base_tokens)
