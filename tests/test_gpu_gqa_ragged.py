@@ -168,3 +168,34 @@ def test_config3_full_size_against_c_oracle():
     assert worst <= 1e-3, f"max abs err {worst}"
     assert flips <= 1e-3 * total
     print(f"C3: max err {worst:.2e}, V level flips {flips}/{total}, plane bytes per query group {moved / dense:.3f} of dense")
+
+
+def test_unsupported_combinations_are_refused_before_launch():
+    from alignedkv_amd.extension.KV_cache_cpp_extention import cuda_module as m
+    from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
+    B, Hq, Hkv, D = 2, 8, 2, 128
+    c = RaggedGQACache(1, B, 256, Hq, Hkv, D)
+    q = torch.zeros((B, 1, Hq, D), dtype=torch.half, device="cuda")
+    kv = torch.zeros((B, 1, Hkv, D), dtype=torch.half, device="cuda")
+    out = torch.empty_like(q)
+
+    def step(**kw):
+        args = dict(k_block=None, seq_lens=c.seq_lens[0], cur_len=0)
+        args.update(kw)
+        m.decode_step_gqa(c.k_planes[0], c.v_planes[0], c.k_colmax[0], c.v_colmax[0], c.restk[0].view(torch.uint8),
+                          c.restv[0].view(torch.uint8), q.view(torch.uint8), kv.view(torch.uint8), kv.view(torch.uint8), None,
+                          out.view(torch.uint8), c.scores.view(torch.uint8), c.probs.view(torch.uint8), B, Hq, Hkv,
+                          c.n_max_blocks, c.max_seq_len, D, 64, 32, args["cur_len"], args["seq_lens"], False,
+                          k_block=args["k_block"])
+
+    with pytest.raises(RuntimeError, match="seq_lens"):
+        step(seq_lens=c.seq_lens[0].long())
+    with pytest.raises(RuntimeError, match="cache full"):
+        step(cur_len=256)
+    # 256-token K blocks are for multi-head caches; the plane size check of the wrapper comes first for other sizes
+    with pytest.raises(RuntimeError):
+        step(k_block=256)
+    with pytest.raises(RuntimeError):
+        step(k_block=128)
+    step()   # and the supported call goes through
+    assert c.seq_lens[0].cpu().tolist() == [1, 1]
