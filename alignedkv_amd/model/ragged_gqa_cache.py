@@ -65,12 +65,14 @@ class RaggedGQACache:
         self.seq_lens[layer][b] = S
         self.len_bound[layer] = max(self.len_bound[layer], S)
 
-    def decode(self, layer: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask2d=None) -> torch.Tensor:
+    def decode(self, layer: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask2d=None, bound=None) -> torch.Tensor:
         """One decode step for every sequence: q fp16 [bsz,1,n_q_heads,head_dim], k/v [bsz,1,n_kv_heads,head_dim].
-        Returns fp16 [bsz,1,n_q_heads,head_dim] and advances the lengths."""
+        Returns fp16 [bsz,1,n_q_heads,head_dim] and advances the lengths.  bound: upper bound of the lengths that
+        sizes the launches (default: the largest length this object has seen)."""
         B, Hq, Hkv, D = self.bsz, self.n_q_heads, self.n_kv_heads, self.head_dim
         assert tuple(q.shape) == (B, 1, Hq, D) and tuple(k.shape) == (B, 1, Hkv, D) and k.shape == v.shape
-        bound = self.len_bound[layer]
+        fixed_bound = bound is not None
+        bound = self.len_bound[layer] if bound is None else bound
         assert bound + 1 <= self.max_seq_len, "cache full"
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         out = torch.empty_like(q)
@@ -86,6 +88,24 @@ class RaggedGQACache:
                                     out.view(torch.uint8), self.scores.view(torch.uint8), self.probs.view(torch.uint8),
                                     B, Hq, Hkv, self.n_max_blocks, self.max_seq_len, D, column_block, 32, bound,
                                     self.seq_lens[layer], self.reference, klv, vlv if flushed else None, amin)
-        self.len_bound[layer] = bound + 1
+        if not fixed_bound:
+            self.len_bound[layer] = bound + 1
         self.last_k_levels, self.last_v_levels, self.last_alignment_min = klv, vlv, amin
         return out
+
+    def capture_decode(self, layer: int):
+        """One decode step of `layer` as a HIP graph.  With the capacity as the length bound every argument of
+        akv_decode_step_gqa is constant from step to step (the lengths live on the device and the step advances
+        them itself), so the five launches of a step are captured once and replayed: the host then pays one graph
+        launch per step instead of five kernel launches, which is what bounds small batches.
+        Returns (graph, q, k, v, out): write the step's inputs into q, k, v, call graph.replay(), read out.
+        The caller keeps the lengths below the capacity (the step does not check them on the device)."""
+        assert not self.record_levels, "level recording sizes its buffers per step"
+        dev = self.seq_lens[layer].device
+        q = torch.zeros((self.bsz, 1, self.n_q_heads, self.head_dim), dtype=torch.half, device=dev)
+        k = torch.zeros((self.bsz, 1, self.n_kv_heads, self.head_dim), dtype=torch.half, device=dev)
+        v = torch.zeros_like(k)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = self.decode(layer, q, k, v, bound=self.max_seq_len - 1)
+        return graph, q, k, v, out

@@ -199,3 +199,33 @@ def test_unsupported_combinations_are_refused_before_launch():
         step(k_block=128)
     step()   # and the supported call goes through
     assert c.seq_lens[0].cpu().tolist() == [1, 1]
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(8, 8), (8, 2)])
+def test_captured_step_replays_like_the_eager_step(Hq, Hkv):
+    """The step with per-sequence lengths has constant arguments: captured once in a HIP graph and replayed with
+    eager work and synchronisations in between, every replay must equal the eager step on a twin cache."""
+    from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
+    B, D, lens, steps = 3, 128, [190, 62, 700], 8
+    Lmax = 1024
+    _, k, v = make_qkv(B, Lmax, Hkv, D, seed=3)
+    rng = np.random.default_rng(2)
+    eager, graphed = RaggedGQACache(1, B, Lmax, Hq, Hkv, D), RaggedGQACache(1, B, Lmax, Hq, Hkv, D)
+    for c in (eager, graphed):
+        for b in range(B):
+            c.prefill(0, b, dev(k[b:b + 1, :lens[b]]), dev(v[b:b + 1, :lens[b]]))
+    graph, gq, gk, gv, gout = graphed.capture_decode(0)
+    for s in range(steps):
+        q = dev(rng.standard_normal((B, 1, Hq, D)).astype(np.float16))
+        kn = dev(np.stack([k[b, lens[b] + s] for b in range(B)])[:, None])
+        vn = dev(np.stack([v[b, lens[b] + s] for b in range(B)])[:, None])
+        want = eager.decode(0, q, kn, vn)
+        torch.cuda.synchronize()
+        gq.copy_(q); gk.copy_(kn); gv.copy_(vn)
+        graph.replay()
+        torch.cuda.synchronize()
+        # the eager step sizes its launches by the longest sequence, the graph by the capacity: same results
+        assert (gout.float() - want.float()).abs().max().item() <= 1e-3, f"replay {s}"
+        assert torch.equal(graphed.seq_lens[0], eager.seq_lens[0])
+    for i in range(3):
+        assert torch.equal(graphed.k_planes[0][i], eager.k_planes[0][i]) and torch.equal(graphed.v_planes[0][i], eager.v_planes[0][i])
