@@ -1,0 +1,60 @@
+"""Writes tests/golden/akv_small_cases.npz: small seeded decode cases with everything the NumPy oracle derives
+from them (planes, fetch levels, threshold, probabilities, outputs).
+
+The reference ships no tests, golden vectors or fixtures, and its kernels are CUDA (nothing of it can run in this
+image), so these vectors come from this repository's own oracle (oracle/akv_oracle.py), whose functions are pinned
+by tests/test_oracle_*.py.  They freeze that behaviour: the C restatement, the NumPy oracle of any later state of
+the repository and the HIP path are all compared with the same committed numbers.
+
+    python tests/golden/make_fixtures.py
+"""
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+from oracle import akv_oracle as O          # noqa: E402
+from tests.common import make_qkv           # noqa: E402
+
+CASES = {   # name: (B, H, D, prefill, steps, k_block, literal_broadcast)
+    "mha_d64": (1, 1, 64, 130, 2, 64, False),
+    "mha_d128_flush": (1, 1, 128, 62, 3, 64, False),      # the second step fills the rest buffer
+    "mha_kblock256": (1, 1, 64, 200, 2, 256, False),
+    "mha_literal_broadcast": (2, 2, 64, 64, 1, 64, True),
+}
+
+
+def main():
+    out = {}
+    for name, (B, H, D, prefill, steps, kb, lit) in CASES.items():
+        _, k, v = make_qkv(B, prefill + steps, H, D, seed=len(name) + prefill)
+        rng = np.random.default_rng(prefill)
+        q = rng.standard_normal((steps, B, 1, H, D)).astype(np.float16)
+        c = O.OracleCache(B, prefill + steps + 64, H, D, k_block=kb, literal_broadcast=lit)
+        c.save(k[:, :prefill], v[:, :prefill], 0, prefill)
+        outs = []
+        for s in range(steps):
+            outs.append(c.decode(q[s], k[:, prefill + s:prefill + s + 1], v[:, prefill + s:prefill + s + 1]))
+        out[name + "/shape"] = np.array([B, H, D, prefill, steps, kb, int(lit)], np.int32)
+        out[name + "/k"], out[name + "/v"], out[name + "/q"] = O.as_bits(k), O.as_bits(v), O.as_bits(q)
+        out[name + "/out"] = O.as_bits(np.stack(outs))
+        nkb = O.cdiv(c.rest_start, kb)
+        for i, p in enumerate(c.k_planes):
+            assert not p[:, :, nkb:].any()
+            out[name + f"/k_plane{i}"] = p[:, :, :nkb]           # the blocks that hold tokens; the rest is zero
+        for i, p in enumerate(c.v_planes):
+            assert not p[:, :, c.rest_start:].any()
+            out[name + f"/v_plane{i}"] = p[:, :, :c.rest_start]
+        out[name + "/k_colmax"], out[name + "/v_colmax"] = c.k_colmax, c.v_colmax
+        out[name + "/k_levels"], out[name + "/v_levels"] = c.last["k_levels"], c.last["v_levels"]
+        out[name + "/amin"] = c.last["amin"]
+        out[name + "/probs"] = O.as_bits(c.last["probs"])
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "akv_small_cases.npz")
+    np.savez_compressed(path, **out)
+    print(path, os.path.getsize(path), "bytes")
+
+
+if __name__ == "__main__":
+    main()
