@@ -65,7 +65,8 @@ __global__ void fused_persist_kernel(const unsigned short *__restrict__ k_new, c
 // Task maps of a step with per-sequence lengths (see step_block): for each of the two streaming passes the
 // workgroups that have tokens to read, ordered by (batch, head index, chunk) with the chunk fastest, then kNoTask
 // up to the size of the grid; v_chunks[b] = V-pass chunks of sequence b, for the combine kernel (the lengths
-// themselves advance while it runs).  One workgroup of 256 threads; scratch: 2 * 257 ints of LDS.
+// themselves advance while it runs).  One workgroup of 256 threads per sequence and map: it sums the entry counts
+// of the sequences before its own, writes its sequence's entries and its share of the kNoTask tail.
 struct TaskMaps {
     u32 *map_k, *map_v;      // null: no map for that pass
     int *v_chunks;
@@ -73,50 +74,58 @@ struct TaskMaps {
 };
 
 __device__ __forceinline__ void build_task_map(const StepGeom &geo, u32 *map, const PassShape &sh, int B, int *v_chunks,
-                                               int *part) {
+                                               int *red, int b_mine) {
     const int tid = threadIdx.x;
-    const int per = (B + 255) / 256, b0 = tid * per, b1 = min(b0 + per, B);
-    int mine = 0;
-    for (int b = b0; b < b1; ++b) {
+    auto chunks_of = [&](int b) {
         int R, nrest;
         seq_state(geo, b, R, nrest);
-        const int n = (R + sh.tokens_per_wg - 1) / sh.tokens_per_wg;
-        if (v_chunks != nullptr) v_chunks[b] = n;
-        mine += n * sh.grid_y;
+        // (never more than the grid holds, whatever the length says: the map has grid_x entries per head)
+        return min((R + sh.tokens_per_wg - 1) / sh.tokens_per_wg, sh.grid_x);
+    };
+    int before = 0, all = 0;
+    for (int b = tid; b < B; b += 256) {
+        const int c = chunks_of(b) * sh.grid_y;
+        all += c;
+        if (b < b_mine) before += c;
     }
-    part[tid] = mine;
-    __syncthreads();
-    if (tid == 0) {
-        int run = 0;
-        for (int i = 0; i < 256; ++i) {
-            const int v = part[i];
-            part[i] = run;
-            run += v;
-        }
-        part[256] = run;
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        before += __shfl_xor(before, m, 64);
+        all += __shfl_xor(all, m, 64);
+    }
+    if ((tid & 63) == 0) {
+        red[2 * (tid >> 6)] = before;
+        red[2 * (tid >> 6) + 1] = all;
     }
     __syncthreads();
-    int at = part[tid];
-    for (int b = b0; b < b1; ++b) {
-        int R, nrest;
-        seq_state(geo, b, R, nrest);
-        const int n = (R + sh.tokens_per_wg - 1) / sh.tokens_per_wg;
-        for (int y = 0; y < sh.grid_y; ++y)
-            for (int x = 0; x < n; ++x) map[at++] = pack_task(x, y, b);
+    const int at = red[0] + red[2] + red[4] + red[6], total = red[1] + red[3] + red[5] + red[7];
+    const int n = chunks_of(b_mine), cnt = n * sh.grid_y;
+    if (v_chunks != nullptr && tid == 0) v_chunks[b_mine] = n;
+    for (int i = tid; i < cnt; i += 256) {
+        const int y = i / n, x = i - y * n;
+        map[at + i] = pack_task(x, y, b_mine);
     }
-    const int total = part[256], grid = sh.grid_x * sh.grid_y * B;
-    for (int i = total + tid; i < grid; i += 256) map[i] = kNoTask;
-    __syncthreads();
+    // the entries past the last task: an equal share per workgroup
+    const int grid = sh.grid_x * sh.grid_y * B, tail = grid - total, share = (tail + B - 1) / B;
+    for (int i = b_mine * share + tid; i < min((b_mine + 1) * share, tail); i += 256) map[total + i] = kNoTask;
 }
 
-__device__ __forceinline__ void build_task_maps(const StepGeom &geo, const TaskMaps &m, int B, int *part) {
-    if (m.map_k != nullptr) build_task_map(geo, m.map_k, m.k, B, nullptr, part);
-    if (m.map_v != nullptr) build_task_map(geo, m.map_v, m.v, B, m.v_chunks, part);
+// extra = index among the 2 * B map workgroups: the first B build the K pass's map, the others the V pass's
+__device__ __forceinline__ void build_task_maps(const StepGeom &geo, const TaskMaps &m, int B, int *red, int extra) {
+    if (extra < B) {
+        if (m.map_k != nullptr) build_task_map(geo, m.map_k, m.k, B, nullptr, red, extra);
+    } else {
+        if (m.map_v != nullptr) build_task_map(geo, m.map_v, m.v, B, m.v_chunks, red, extra - B);
+    }
 }
 
 // Ragged mode, first kernel of every step: append the token of every sequence to its rest buffer, update the
 // column maxima and, for the sequences whose rest buffer is full with it, write the 64-token block into the
-// planes (same bytes as k_save_blocks_kernel / v_save_vec8_kernel).  grid (B*Hkv), 256 threads.
+// planes (same bytes as k_save_blocks_kernel / v_save_vec8_kernel).  kPreSplit workgroups per (batch, KV head):
+// the first appends, and a flush is shared between them (16 tokens of V and a quarter of the channels of K each;
+// the token of this step is taken from the step's inputs, so no workgroup waits for the append).
+// grid (B*Hkv*kPreSplit [+ 2*B for the task maps]), 256 threads.
+constexpr int kPreSplit = 4;
 template <int D>
 __global__ __launch_bounds__(256) void fused_pre_kernel(uint8_t *__restrict__ kf8, uint8_t *__restrict__ km4,
                                                         uint8_t *__restrict__ kl4, uint8_t *__restrict__ vf8,
@@ -126,30 +135,37 @@ __global__ __launch_bounds__(256) void fused_pre_kernel(uint8_t *__restrict__ kf
                                                         unsigned short *__restrict__ restk, unsigned short *__restrict__ restv,
                                                         uint8_t *__restrict__ kcm, uint8_t *__restrict__ vcm, StepGeom geo,
                                                         TaskMaps maps, int B) {
-    constexpr int CB = 64;
-    __shared__ unsigned short tile[CB][D + 2];
-    if ((int)blockIdx.x == B * geo.Hkv) {   // the extra workgroup: task maps of the K and the V pass
-        build_task_maps(geo, maps, B, reinterpret_cast<int *>(&tile[0][0]));
+    constexpr int CB = 64, S = kPreSplit, DS = D / S, TS = CB / S;
+    static_assert(DS % 8 == 0, "a workgroup's share of the channels is a whole number of 16-byte vectors");
+    __shared__ unsigned short tile[CB][DS + 2];
+    __shared__ int map_scratch[8];
+    const int n_bh = B * geo.Hkv;
+    if ((int)blockIdx.x >= n_bh * S) {   // the extra workgroups: task maps of the K pass and of the V pass
+        build_task_maps(geo, maps, B, map_scratch, (int)blockIdx.x - n_bh * S);
         return;
     }
-    const int bh = blockIdx.x, b = bh / geo.Hkv, h = bh - b * geo.Hkv;
+    const int bh = blockIdx.x / S, sub = blockIdx.x - bh * S, b = bh / geo.Hkv, h = bh - b * geo.Hkv;
     const int cur = geo.seq_lens[b];
     const int slot = cur % CB;
-    for (int d = threadIdx.x; d < D; d += 256) {
-        const u32 kb = k_new[(int64_t)bh * D + d], vb = v_new[(int64_t)bh * D + d];
-        const int64_t at = (((int64_t)b * CB + slot) * geo.Hkv + h) * D + d;
-        restk[at] = (unsigned short)kb;
-        restv[at] = (unsigned short)vb;
-        kcm[(int64_t)bh * D + d] = (uint8_t)max((u32)kcm[(int64_t)bh * D + d], exp_field(kb));
-        vcm[(int64_t)bh * D + d] = (uint8_t)max((u32)vcm[(int64_t)bh * D + d], exp_field(vb));
+    if (sub == 0) {
+        for (int d = threadIdx.x; d < D; d += 256) {
+            const u32 kb = k_new[(int64_t)bh * D + d], vb = v_new[(int64_t)bh * D + d];
+            const int64_t at = (((int64_t)b * CB + slot) * geo.Hkv + h) * D + d;
+            restk[at] = (unsigned short)kb;
+            restv[at] = (unsigned short)vb;
+            kcm[(int64_t)bh * D + d] = (uint8_t)max((u32)kcm[(int64_t)bh * D + d], exp_field(kb));
+            vcm[(int64_t)bh * D + d] = (uint8_t)max((u32)vcm[(int64_t)bh * D + d], exp_field(vb));
+        }
     }
     if (slot != CB - 1) return;
-    __syncthreads();                          // the token written above is part of the block
     const int blk = cur / CB;
-    // V rows: 8 channels per thread and token
-    for (int idx = threadIdx.x; idx < CB * (D / 8); idx += 256) {
-        const int j = idx / (D / 8), d8 = idx - j * (D / 8);
-        const u32x4 w = *reinterpret_cast<const u32x4 *>(restv + (((int64_t)b * CB + j) * geo.Hkv + h) * D + d8 * 8);
+    // row j of the block: the rest buffer, or this step's token for the last one
+    auto k_row = [&](int j) { return j == CB - 1 ? k_new + (int64_t)bh * D : restk + (((int64_t)b * CB + j) * geo.Hkv + h) * D; };
+    auto v_row = [&](int j) { return j == CB - 1 ? v_new + (int64_t)bh * D : restv + (((int64_t)b * CB + j) * geo.Hkv + h) * D; };
+    // V rows sub*TS .. sub*TS + TS - 1: 8 channels per thread and token
+    for (int idx = threadIdx.x; idx < TS * (D / 8); idx += 256) {
+        const int j = sub * TS + idx / (D / 8), d8 = idx % (D / 8);
+        const u32x4 w = *reinterpret_cast<const u32x4 *>(v_row(j) + d8 * 8);
         const u32 ww[4] = {w.x, w.y, w.z, w.w};
         u32 hi0 = 0, hi1 = 0, mid = 0, last = 0;
 #pragma unroll
@@ -166,29 +182,34 @@ __global__ __launch_bounds__(256) void fused_pre_kernel(uint8_t *__restrict__ kf
         *reinterpret_cast<u32 *>(vm4 + row * (D / 2) + d8 * 4) = mid;
         *reinterpret_cast<u32 *>(vl4 + row * (D / 2) + d8 * 4) = last;
     }
-    // K block: transpose through LDS
-    for (int idx = threadIdx.x; idx < CB * (D / 2); idx += 256) {
-        const int j = idx / (D / 2), dp = idx - j * (D / 2);
-        const u32 w = *reinterpret_cast<const u32 *>(restk + (((int64_t)b * CB + j) * geo.Hkv + h) * D + dp * 2);
-        tile[j][2 * dp] = (unsigned short)(w & 0xffffu);
-        tile[j][2 * dp + 1] = (unsigned short)(w >> 16);
+    // K block, channels sub*DS .. sub*DS + DS - 1: transpose through LDS
+    const int d0 = sub * DS;
+    for (int idx = threadIdx.x; idx < CB * (DS / 8); idx += 256) {
+        const int j = idx / (DS / 8), d8 = idx % (DS / 8);
+        const u32x4 w = *reinterpret_cast<const u32x4 *>(k_row(j) + d0 + d8 * 8);
+        const u32 ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            tile[j][d8 * 8 + 2 * i] = (unsigned short)(ww[i] & 0xffffu);
+            tile[j][d8 * 8 + 2 * i + 1] = (unsigned short)(ww[i] >> 16);
+        }
     }
     __syncthreads();
     // the 64 tokens go to slots s0 .. s0 + 63 of K plane block kblk (blocks of geo.kb tokens)
     const int KB = geo.kb, kblk = (blk * CB) / KB, s0 = blk * CB - kblk * KB;
     const int64_t base = ((int64_t)bh * geo.n_max_blocks + kblk) * (int64_t)D * (KB / 2);
-    for (int idx = threadIdx.x; idx < D * (CB / 4); idx += 256) {
-        const int d = idx / (CB / 4), j = (idx - d * (CB / 4)) * 4;
-        const u32 w = (u32)(tile[j][d] >> 8) | ((u32)(tile[j + 1][d] >> 8) << 8) | ((u32)(tile[j + 2][d] >> 8) << 16) |
-                      ((u32)(tile[j + 3][d] >> 8) << 24);
+    for (int idx = threadIdx.x; idx < DS * (CB / 4); idx += 256) {
+        const int dl = idx / (CB / 4), d = d0 + dl, j = (idx % (CB / 4)) * 4;
+        const u32 w = (u32)(tile[j][dl] >> 8) | ((u32)(tile[j + 1][dl] >> 8) << 8) | ((u32)(tile[j + 2][dl] >> 8) << 16) |
+                      ((u32)(tile[j + 3][dl] >> 8) << 24);
         *reinterpret_cast<u32 *>(kf8 + base * 2 + (int64_t)d * KB + s0 + j) = w;
     }
-    for (int idx = threadIdx.x; idx < D * (CB / 8); idx += 256) {
-        const int d = idx / (CB / 8), j = (idx - d * (CB / 8)) * 8;
+    for (int idx = threadIdx.x; idx < DS * (CB / 8); idx += 256) {
+        const int dl = idx / (CB / 8), d = d0 + dl, j = (idx % (CB / 8)) * 8;
         u32 mw = 0, lw = 0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const u32 le = tile[j + 2 * i][d] & 0xffu, lo = tile[j + 2 * i + 1][d] & 0xffu;
+            const u32 le = tile[j + 2 * i][dl] & 0xffu, lo = tile[j + 2 * i + 1][dl] & 0xffu;
             mw |= ((le & 0xf0u) | (lo >> 4)) << (8 * i);
             lw |= (((le & 0x0fu) << 4) | (lo & 0x0fu)) << (8 * i);
         }
@@ -914,14 +935,14 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     int persist = 1;
     if (ragged) {
         // per-sequence lengths live on the device: one small kernel appends every token and flushes the rest
-        // buffers that fill up with it; its last workgroup writes the task maps
+        // buffers that fill up with it; its last 2*B workgroups write the task maps
         TaskMaps maps;
         maps.map_k = mapped ? reinterpret_cast<u32 *>(ws + lay.map_k) : nullptr;
         maps.map_v = v_mapped ? reinterpret_cast<u32 *>(ws + lay.map_v) : nullptr;
         maps.v_chunks = v_chunks;
         maps.k = ks;
         maps.v = vs;
-        hipLaunchKernelGGL((fused_pre_kernel<D>), dim3(B * Hkv + (mapped ? 1 : 0)), dim3(256), 0, st, kf8, km4, kl4, vf8, vm4,
+        hipLaunchKernelGGL((fused_pre_kernel<D>), dim3(B * Hkv * kPreSplit + (mapped ? 2 * B : 0)), dim3(256), 0, st, kf8, km4, kl4, vf8, vm4,
                            vl4, k16, v16, rk16, rv16, kcm, vcm, geo, maps, B);
         int rc = check_launch("decode_step(pre)");
         if (rc != AKV_OK) return rc;

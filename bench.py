@@ -202,6 +202,26 @@ def cpu_baseline(torch, cache, q, k_new, v_new, n_steps):
     return min(times), out.reshape(B, 1, H, D), klv, vlv, OC.num_threads()
 
 
+def cpu_dense_torch(torch, B, H, D, L, n_steps=10, warm=3):
+    """Dense attention as the reference's model file computes it (model/Llama_AlignedKV.py:119-140: fp16
+    tensors, fp32 softmax) with torch on the host cores, one step over L tokens.  Returns (seconds, threads)."""
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn((B, 1, H, D), generator=g).half()
+    k = torch.randn((B, L, H, D), generator=g).half()
+    v = torch.randn((B, L, H, D), generator=g).half()
+    kt, vt = k.permute(0, 2, 3, 1), v.transpose(1, 2)
+    times = []
+    for i in range(warm + n_steps):
+        t0 = time.perf_counter()
+        s = torch.matmul(q.transpose(1, 2), kt) / math.sqrt(D)
+        pr = torch.softmax(s.float(), dim=-1).type_as(q)
+        torch.matmul(pr, vt).transpose(1, 2).contiguous()
+        if i >= warm:
+            times.append(time.perf_counter() - t0)
+    times.sort()
+    return times[len(times) // 2], torch.get_num_threads()
+
+
 def bench_c3(a):
     """Grouped-query, ragged-length decode step (akv_decode_step_gqa) at batch 32, 32 query heads over 8 KV
     heads x 128, lengths uniform in [2048, 8192].  The lengths are reset before every step so that each step
@@ -415,6 +435,9 @@ def main():
         res["cpu_baseline"] = {"value": round(cpu_sec * 1e6, 1), "unit": "us/step", "cores": threads, "kind": "port",
                                "sample": "%d full-size steps of layer 0 (min), C restatement with OpenMP + NumPy host logic"
                                          % a.cpu_steps}
+        dsec, dthreads = cpu_dense_torch(torch, B, H, D, L + 1)
+        res["cpu_dense_torch"] = {"value": round(dsec * 1e6, 1), "unit": "us/step", "cores": dthreads,
+                                  "sample": "median of 10 dense fp16 attention steps (fp32 softmax) with torch on the host"}
         res["parity"] = {"max_abs_err_vs_oracle": err, "k_levels_equal": bool(np.array_equal(cklv, k_levels)),
                          "v_level_mismatches": int((cvlv != v_levels).sum()), "v_levels_total": int(v_levels.size)}
     # 64 consecutive decode steps per layer (the cache grows from L to L + 64: the rest buffer fills up and is
