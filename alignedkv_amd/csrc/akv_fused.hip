@@ -432,6 +432,22 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
             sv[v] = load_b128_device(rScores, i < nvec ? i * 16 : kSkip);
         }
     }
+    // the tail's key rows and q: LPT lanes per tail token, 8 channels per 16-byte load, all rows in flight at once
+    // (a real decode step has 32 tail tokens on average)
+    constexpr int LPT = NT / 64;              // lanes per token (the rest buffer holds at most 64 tokens)
+    constexpr int NKV = (D / 8 + LPT - 1) / LPT;
+    const int tr = tid / LPT, tj = tid % LPT;
+    u32x4 tkw[NKV], tqw[NKV];
+    {
+        const unsigned short *krow = (tr == newest && a.persist) ? knew : a.restk + (((int64_t)b * cb + tr) * Hkv + h) * D;
+#pragma unroll
+        for (int i = 0; i < NKV; ++i) {
+            const int v8 = tj + i * LPT;
+            const bool on = tr < nrest && v8 < D / 8;
+            tkw[i] = on ? *reinterpret_cast<const u32x4 *>(krow + v8 * 8) : (u32x4){0u, 0u, 0u, 0u};
+            tqw[i] = on ? *reinterpret_cast<const u32x4 *>(qrow + v8 * 8) : (u32x4){0u, 0u, 0u, 0u};
+        }
+    }
     // (a) append the token: rest buffers and column maxima (extension/k_cache_file.py:98-101).
     //     vcm_mine: this thread's channel of the V column maxima after the update (threads < D).
     u32 vcm_mine = 0;
@@ -454,33 +470,26 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
         vcm_mine = vc;
     }
     // (b) scores of the tail: fp16(fp16(q.k) / sqrt(D)), the two roundings of an fp16 matmul followed by
-    //     an fp16 division (extension/k_cache_file.py:156).  LPT lanes per tail token, 8 channels per 16-byte load:
-    //     all rows are in flight at once (a real decode step has 32 tail tokens on average).
+    //     an fp16 division (extension/k_cache_file.py:156)
     const float sqrt_d = sqrtf((float)D);
     {
-        constexpr int LPT = NT / 64;          // lanes per token (the rest buffer holds at most 64 tokens)
-        const int r = tid / LPT, j = tid % LPT;
         float part = 0.f;
-        if (r < nrest) {
-            const unsigned short *krow = (r == newest && a.persist) ? knew : a.restk + (((int64_t)b * cb + r) * Hkv + h) * D;
-            for (int v8 = j; v8 < D / 8; v8 += LPT) {
-                const u32x4 kw = *reinterpret_cast<const u32x4 *>(krow + v8 * 8);
-                const u32x4 qw = *reinterpret_cast<const u32x4 *>(qrow + v8 * 8);
-                const u32 kk[4] = {kw.x, kw.y, kw.z, kw.w}, qq[4] = {qw.x, qw.y, qw.z, qw.w};
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    part = fmaf(lo_half_to_float(kk[i]), lo_half_to_float(qq[i]), part);
-                    part = fmaf(hi_half_to_float(kk[i]), hi_half_to_float(qq[i]), part);
-                }
+        for (int i = 0; i < NKV; ++i) {
+            const u32 kk[4] = {tkw[i].x, tkw[i].y, tkw[i].z, tkw[i].w}, qq[4] = {tqw[i].x, tqw[i].y, tqw[i].z, tqw[i].w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                part = fmaf(lo_half_to_float(kk[c]), lo_half_to_float(qq[c]), part);
+                part = fmaf(hi_half_to_float(kk[c]), hi_half_to_float(qq[c]), part);
             }
         }
 #pragma unroll
         for (int mk = 1; mk < LPT; mk <<= 1) part += __shfl_xor(part, mk, 64);
-        if (r < nrest && j == 0) {
+        if (tr < nrest && tj == 0) {
             const float dot16 = half_bits_to_float(float_to_half_bits(part));
             const unsigned short sc = float_to_half_bits(dot16 / sqrt_d);
-            tail_s[r] = sc;
-            srow[R + r] = sc;
+            tail_s[tr] = sc;
+            srow[R + tr] = sc;
         }
     }
     lds_barrier();
@@ -583,6 +592,20 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
         }
     }
 
+    // value rows of the tail, used by (f): requested here so that they travel while the probe runs
+    constexpr int VPR = D / 8;                // 16-byte vectors per row
+    constexpr int NRG = NT / VPR;             // row groups
+    constexpr int MAXR = (64 + NRG - 1) / NRG;
+    static_assert(VPR <= 32, "head_dim above 256 needs another tail mapping");
+    const int c8 = tid % VPR, rg = tid / VPR;
+    u32x4 tvw[MAXR];
+#pragma unroll
+    for (int k = 0; k < MAXR; ++k) {
+        const int r = rg + k * NRG;
+        const unsigned short *vrow = (r == newest && a.persist) ? vnew : a.restv + (((int64_t)b * cb + r) * Hkv + h) * D;
+        tvw[k] = r < nrest ? *reinterpret_cast<const u32x4 *>(vrow + c8 * 8) : (u32x4){0u, 0u, 0u, 0u};
+    }
+
     // (d)+(e) probe over the flushed part (extension/v_cache_file.py:119-143) and the alignment threshold
     //     of this (batch, head) (extension/v_cache_file.py:156-160)
     if (R > 0) {
@@ -637,21 +660,17 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
         lds_barrier();
     }
     // (f) the tail's share of the output, an fp16 matmul result (extension/v_cache_file.py:189): a thread takes 8
-    //     channels of every NRG-th tail token, lanes of a wave that share the channels fold by shuffles, waves by LDS
+    //     channels of every NRG-th tail token (requested before the probe), lanes of a wave that share the channels
+    //     fold by shuffles, waves by LDS
     {
-        constexpr int VPR = D / 8;            // 16-byte vectors per row
-        constexpr int NRG = NT / VPR;         // row groups
-        constexpr int RGW = 64 / VPR;         // row groups inside a wave
-        static_assert(VPR <= 32, "head_dim above 256 needs another tail mapping");
-        const int c8 = tid % VPR, rg = tid / VPR;
         float acc[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[i] = 0.f;
-        for (int r = rg; r < nrest; r += NRG) {
-            const unsigned short *vrow = (r == newest && a.persist) ? vnew : a.restv + (((int64_t)b * cb + r) * Hkv + h) * D;
-            const u32x4 vw = *reinterpret_cast<const u32x4 *>(vrow + c8 * 8);
-            const u32 vv[4] = {vw.x, vw.y, vw.z, vw.w};
-            const float pr = tail_p[r];
+#pragma unroll
+        for (int k = 0; k < MAXR; ++k) {
+            const int r = rg + k * NRG;
+            const u32 vv[4] = {tvw[k].x, tvw[k].y, tvw[k].z, tvw[k].w};
+            const float pr = r < nrest ? tail_p[r] : 0.f;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 acc[2 * i] = fmaf(lo_half_to_float(vv[i]), pr, acc[2 * i]);
@@ -662,7 +681,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
         for (int mk = VPR; mk < 64; mk <<= 1)
 #pragma unroll
             for (int i = 0; i < 8; ++i) acc[i] += __shfl_xor(acc[i], mk, 64);
-        (void)RGW;
         if (lane < VPR) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) tail_o[wave][c8 * 8 + i] = acc[i];
