@@ -445,41 +445,40 @@ __device__ __forceinline__ void v_macro_ops(VMacroOps &o, const u32x2 *p, unsign
     if (REF) {
         mid = last = head ? 0xffffu : 0u;
         o.lv2 = 0;
-    } else {
-        // most tokens are at level 2 for every head: first the smallest 16-bit difference of the lane's 16 tokens
-        // (the differences wrap like the reference's `short` arithmetic, extension/csrc/V_cache.cu:195-197,211)
+    } else if (head) {
+        // 16-bit differences of two tokens at a time (they wrap like the reference's `short` arithmetic,
+        // extension/csrc/V_cache.cu:195-197,211); level < 2 <=> diff < 0x0800, level 0 <=> diff < 0x0400, read off the
+        // sign of a saturating subtraction.  Word w = 2 s + (0: tokens 0,1 | 1: tokens 2,3 of step s) leaves the flag
+        // of its first token in bit 2 w and of its second in bit 16 + 2 w.
         const unsigned short a16 = (unsigned short)((unsigned)amin << 10);
         const u16x2 a2 = {a16, a16};
-        i16x2 mn = {32767, 32767};
+        const i16x2 c8 = {0x0800, 0x0800}, c4 = {0x0400, 0x0400};
+        u32 acc8 = 0, acc4 = 0;
 #pragma unroll
-        for (int sidx = 0; sidx < 4; ++sidx) {
-            const i16x2 d0 = wrap_diff16(a2, p[sidx].x), d1 = wrap_diff16(a2, p[sidx].y);
-            mn = __builtin_elementwise_min(mn, __builtin_elementwise_min(d0, d1));
+        for (int w = 0; w < 8; ++w) {
+            const i16x2 d = wrap_diff16(a2, (w & 1) ? p[w >> 1].y : p[w >> 1].x);
+            union { i16x2 v; u32 u; } t8, t4;
+            t8.v = __builtin_elementwise_sub_sat(d, c8);
+            t4.v = __builtin_elementwise_sub_sat(d, c4);
+            acc8 |= ((t8.u >> 15) & 0x00010001u) << (2 * w);
+            acc4 |= ((t4.u >> 15) & 0x00010001u) << (2 * w);
         }
-        if (head && min(mn.x, mn.y) < 0x0800) {   // some token of this lane is at level 0 or 1: classify all
-            o.lv2 = 0;
-#pragma unroll
-            for (int sidx = 0; sidx < 4; ++sidx)
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const u32 bits = ((u < 2 ? p[sidx].x : p[sidx].y) >> (16 * (u & 1))) & 0xffffu;
-                    const int lv = v_level(amin, (unsigned short)bits);
-                    mid |= (lv < 2 ? 1u : 0u) << (4 * sidx + u);
-                    last |= (lv == 0 ? 1u : 0u) << (4 * sidx + u);
-                    o.lv1 |= (lv == 1 ? 1u : 0u) << (4 * sidx + u);
-                    o.lv2 |= (lv == 2 ? 1u : 0u) << (4 * sidx + u);
-                }
-        }
+        mid = (acc8 & 0xffffu) | ((acc8 >> 16) << 1);
+        last = (acc4 & 0xffffu) | ((acc4 >> 16) << 1);
+        o.lv1 = mid & ~last;
+        o.lv2 = ~mid & 0xffffu;
     }
-    // union over the heads: OR over the 16 lanes of the lane group
+    // union over the heads: OR over the 16 lanes of the lane group (one DPP row)
     u32 both = mid | (last << 16);
-#pragma unroll
-    for (int m = 1; m < 16; m <<= 1) both |= (u32)__shfl_xor((int)both, m, 64);
+    both |= (u32)__builtin_amdgcn_update_dpp(0, (int)both, 0x128, 0xf, 0xf, false);   // row_ror:8
+    both |= (u32)__builtin_amdgcn_update_dpp(0, (int)both, 0x124, 0xf, 0xf, false);   // row_ror:4
+    both |= (u32)__builtin_amdgcn_update_dpp(0, (int)both, 0x122, 0xf, 0xf, false);   // row_ror:2
+    both |= (u32)__builtin_amdgcn_update_dpp(0, (int)both, 0x121, 0xf, 0xf, false);   // row_ror:1
     o.need = both;
 }
 
 template <int D, bool REF>
-__global__ __launch_bounds__(256) void mfma_v_pass_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void mfma_v_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const unsigned short *__restrict__ probs, const uint8_t *__restrict__ amin_u8, float *__restrict__ partial,
     uint8_t *__restrict__ levels_out, int levels_stride, uint8_t *__restrict__ amin_out, StepGeom geo,
