@@ -245,7 +245,7 @@ __device__ __forceinline__ void kt_compute_coarse(f32x4 *acc, const KTaskTile<SL
 }
 
 template <int D, bool REF, int SL, int AHEAD>
-__global__ __launch_bounds__(256) void mfma_k_pass_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && AHEAD == 3 ? 3 : 1))) void mfma_k_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const u32 *__restrict__ prep, unsigned short *__restrict__ scores, StepGeom geo, int tasks_per_wave, float scale,
     u32 scores_bytes) {
@@ -354,7 +354,7 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
     const int nbt = sl / 4;
     const int n_tasks = (n_blocks + nbt - 1) / nbt;
     int tpw = 1;
-    while (tpw < 8 && (int64_t)B * geo.Hkv * ((n_tasks + 8 * tpw - 1) / (8 * tpw)) * 4 >= 8192) tpw *= 2;
+    while (tpw < 8 && (int64_t)B * geo.Hkv * ((n_tasks + 8 * tpw - 1) / (8 * tpw)) * 4 >= 32768) tpw *= 2;
     { AKV_TUNE("AKV_TUNE_K_TPW", v); if (has_v && v > 0) tpw = v; }
     if (shape_only != nullptr) {
         *shape_only = PassShape{(n_tasks + 4 * tpw - 1) / (4 * tpw), geo.Hkv, 4 * tpw * nbt * 64};
