@@ -845,8 +845,18 @@ __global__ void fused_combine_kernel(const float *__restrict__ partial, const un
     // last kernel of the step: the sequence lengths kept on the device advance here
     if (seq_lens_rw != nullptr && threadIdx.x == 0 && bh % Hq == 0) seq_lens_rw[bh / Hq] += 1;
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        // fixed order (the bits do not depend on which workgroup finished first), eight loads in flight at a time
+        const float *src = partial + (int64_t)bh * n_chunks * D + d;
         float acc = 0.f;
-        for (int c = 0; c < n_sum; ++c) acc += partial[((int64_t)bh * n_chunks + c) * D + d];
+        int c = 0;
+        for (; c + 8 <= n_sum; c += 8) {
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = src[(int64_t)(c + i) * D];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc += v[i];
+        }
+        for (; c < n_sum; ++c) acc += src[(int64_t)c * D];
         const float o16 = half_bits_to_float(float_to_half_bits(acc));
         out[(int64_t)bh * D + d] = float_to_half_bits(o16 + half_bits_to_float(otail[(int64_t)bh * D + d]));
     }
