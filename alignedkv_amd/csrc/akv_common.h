@@ -18,6 +18,7 @@ namespace akv {
 // ---- host-side error reporting -------------------------------------------------------------
 void set_error(const char *fmt, ...);
 int check_launch(const char *what);
+int compute_units();   // of the current device (0: unknown)
 
 // Tuning switches from the environment (AKV_TUNE_*), read once per call site and again after
 // akv_reload_tuning(): a getenv per switch and step costs a few microseconds of host time per decode step,

@@ -256,16 +256,21 @@ __device__ __forceinline__ void k256_score_blocks(KHalfTile<4> &ta, const uint8_
 }
 
 template <int HV>
-struct VHalfTile {   // HV wave-wide loads: 64/(D/16) token rows each
+struct VHighPart {   // HV wave-wide loads: 64/(D/16) token rows each, high bytes
     u32x4 h[HV];
+};
+template <int HV>
+struct VLowPart {    // the nibble rows of the same tokens
     u32x2 m[HV], l[HV];
     u32 cm[HV], cl[HV];   // substitution bytes of skipped planes
 };
+template <int HV>
+struct VHalfTile : VHighPart<HV>, VLowPart<HV> {};
 
 // Requests the rows of the tokens base + u*TPL + tl (u < HV).  The high-byte rows do not depend on the
 // fetch level and are requested before the probabilities (sb) are looked at.
 template <int D, int HV>
-__device__ __forceinline__ void v_issue_half_h(VHalfTile<HV> &t, const __amdgpu_buffer_rsrc_t rH, int base, int t_end) {
+__device__ __forceinline__ void v_issue_half_h(VHighPart<HV> &t, const __amdgpu_buffer_rsrc_t rH, int base, int t_end) {
     constexpr int LPR = D / 16, TPL = 64 / LPR;
     const int lane = threadIdx.x & 63;
     const int tl = lane / LPR, cl = lane % LPR;
@@ -277,7 +282,7 @@ __device__ __forceinline__ void v_issue_half_h(VHalfTile<HV> &t, const __amdgpu_
 }
 
 template <int D, bool REF, int HV>
-__device__ __forceinline__ void v_issue_half_ml(VHalfTile<HV> &t, const __amdgpu_buffer_rsrc_t rM,
+__device__ __forceinline__ void v_issue_half_ml(VLowPart<HV> &t, const __amdgpu_buffer_rsrc_t rM,
                                                 const __amdgpu_buffer_rsrc_t rL, int base, int t_end, const u32 *sb,
                                                 unsigned char amin) {
     constexpr int LPR = D / 16, TPL = 64 / LPR;
@@ -317,20 +322,24 @@ __device__ __forceinline__ void v_prefetch_first(VFirstTile<D> &ft, const uint8_
 }
 
 template <int HV>
-__device__ __forceinline__ void v_compute_half(float *acc, const VHalfTile<HV> &t, const u32 *sb) {
+__device__ __forceinline__ void v_compute_half(float *acc, const VHighPart<HV> &th, const VLowPart<HV> &t, const u32 *sb) {
 #pragma unroll
     for (int u = 0; u < HV; ++u) {
         const float sf = half_bits_to_float(sb[u]);
-        fma8(acc, t.h[u].x, t.h[u].y, t.m[u].x | t.cm[u], t.l[u].x | t.cl[u], sf);
-        fma8(acc + 8, t.h[u].z, t.h[u].w, t.m[u].y | t.cm[u], t.l[u].y | t.cl[u], sf);
+        fma8(acc, th.h[u].x, th.h[u].y, t.m[u].x | t.cm[u], t.l[u].x | t.cl[u], sf);
+        fma8(acc + 8, th.h[u].z, th.h[u].w, t.m[u].y | t.cm[u], t.l[u].y | t.cl[u], sf);
     }
+}
+template <int HV>
+__device__ __forceinline__ void v_compute_half(float *acc, const VHalfTile<HV> &t, const u32 *sb) {
+    v_compute_half<HV>(acc, t, t, sb);
 }
 
 // A half tile whose tokens are all at level 2 (wave-uniform): only the high bytes are requested and multiplied,
 // the low byte is the constant 0x80.  With ~1 % of the tokens below level 2 that is most half tiles, and it
 // saves two thirds of their load instructions (skipped nibble rows still cost an issue slot each).
 template <int HV>
-__device__ __forceinline__ void v_compute_half_coarse(float *acc, const VHalfTile<HV> &t, const u32 *sb) {
+__device__ __forceinline__ void v_compute_half_coarse(float *acc, const VHighPart<HV> &t, const u32 *sb) {
 #pragma unroll
     for (int u = 0; u < HV; ++u) {
         const float sf = half_bits_to_float(sb[u]);
@@ -425,6 +434,105 @@ __device__ __forceinline__ void v_accumulate_range(const uint8_t *f8, const uint
         VFirstTile<D> ft;
         v_prefetch_first<D>(ft, f8, n_tokens, g, t_end);
         v_accumulate<D, REF, 2>(ft, f8, m4, l4, n_tokens, s_row, amin, g, min(g + GT, t_end), acc, levels_row);
+    }
+}
+
+// One wave streams the half tiles first_half, first_half + half_stride, ... of a row of V planes (a half tile = HT
+// tokens): a ring of NR half tiles of high bytes, each requested together with its probabilities NR - 1 half tiles
+// before it is multiplied (neither depends on a fetch level); the nibble rows of a half tile with a token below
+// level 2 are requested one half tile ahead, before the newest high bytes, so that waiting for them does not wait
+// for those.  For callers that give a wave a long range: v_accumulate keeps one half tile in flight and leaves the
+// overlap to the number of waves.
+template <int D>
+struct VStream {
+    static constexpr int LPR = D / 16, TPL = 64 / LPR, U = LPR < 8 ? LPR : 8, HV = U / 2, HT = HV * TPL;
+};
+
+template <int D, int NR>
+struct VRing {
+    VHighPart<VStream<D>::HV> hi[NR];
+    u32 sb[NR][VStream<D>::HV];
+};
+
+// The wave's i-th half tile: interleaved over the n_waves waves of the workgroup (at any time the waves read
+// neighbouring rows).  Past the wave's share: n_halves (nothing is fetched).
+struct VSeq {
+    int wave, n_waves, n_per_wave, n_halves;
+    __device__ __forceinline__ int half(int i) const { return i < n_per_wave ? i * n_waves + wave : n_halves; }
+};
+
+// requests half tile `half` (tokens half * HT ...) into ring slot k
+template <int D, int NR>
+__device__ __forceinline__ void v_stream_issue(VRing<D, NR> &ring, int k, const __amdgpu_buffer_rsrc_t rH,
+                                               const __amdgpu_buffer_rsrc_t rS, int half, int n_tokens) {
+    using S = VStream<D>;
+    const int lane = threadIdx.x & 63, tl = lane / S::LPR;
+    const int base = half * S::HT;
+    // the probabilities first: loads return in order, and the fetch levels of a half tile are looked at one half
+    // tile before its high bytes are needed
+#pragma unroll
+    for (int u = 0; u < S::HV; ++u) {
+        const int t = base + u * S::TPL + tl;
+        ring.sb[k][u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < n_tokens ? t * 2 : kSkip, 0, 0);
+    }
+    v_issue_half_h<D, S::HV>(ring.hi[k], rH, base, n_tokens);
+}
+
+// the first PF half tiles of the wave: before anything the caller has to do first (they depend on nothing but
+// the probabilities, which the caller may still be writing: those are requested by v_stream_run, together with
+// the high bytes of the half tiles PF .. NR - 2)
+template <int D, int NR, int PF>
+__device__ __forceinline__ void v_stream_prefetch(VRing<D, NR> &ring, const uint8_t *f8, int n_tokens, const VSeq &seq) {
+    using S = VStream<D>;
+    static_assert(PF <= NR - 1, "the ring keeps one slot for the half tile being multiplied");
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
+#pragma unroll
+    for (int k = 0; k < PF; ++k) v_issue_half_h<D, S::HV>(ring.hi[k], rH, seq.half(k) * S::HT, n_tokens);
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+template <int D, bool REF, int NR, int PF>
+__device__ __forceinline__ void v_stream_run(VRing<D, NR> &ring, const uint8_t *f8, const uint8_t *m4, const uint8_t *l4,
+                                             int n_tokens, const unsigned short *s_row, unsigned char amin, const VSeq &seq,
+                                             float *acc) {
+    using S = VStream<D>;
+    static_assert(NR % 2 == 0, "the two nibble buffers alternate with the ring slots");
+    constexpr int HV = S::HV;
+    const int lane = threadIdx.x & 63, tl = lane / S::LPR;
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_tokens * (D / 2));
+    const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_tokens * (D / 2));
+    const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)n_tokens * 2);
+#pragma unroll
+    for (int k = PF; k < NR - 1; ++k) v_issue_half_h<D, HV>(ring.hi[k], rH, seq.half(k) * S::HT, n_tokens);
+    // probabilities of the half tiles requested so far
+#pragma unroll
+    for (int k = 0; k < NR - 1; ++k)
+#pragma unroll
+        for (int u = 0; u < HV; ++u) {
+            const int t = seq.half(k) * S::HT + u * S::TPL + tl;
+            ring.sb[k][u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < n_tokens ? t * 2 : kSkip, 0, 0);
+        }
+    VLowPart<HV> nib[2];
+    bool fine_now = v_half_is_fine<REF, HV>(ring.sb[0], amin);
+    if (fine_now) v_issue_half_ml<D, REF, HV>(nib[0], rM, rL, seq.half(0) * S::HT, n_tokens, ring.sb[0], amin);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int i0 = 0; i0 < seq.n_per_wave; i0 += NR) {
+#pragma unroll
+        for (int k = 0; k < NR; ++k) {
+            // nibble rows of the next half tile first, then the newest probabilities and high bytes
+            const int kn = (k + 1) % NR;
+            const bool fine_next = v_half_is_fine<REF, HV>(ring.sb[kn], amin);
+            if (fine_next)
+                v_issue_half_ml<D, REF, HV>(nib[(k + 1) & 1], rM, rL, seq.half(i0 + k + 1) * S::HT, n_tokens, ring.sb[kn], amin);
+            v_stream_issue<D, NR>(ring, (k + NR - 1) % NR, rH, rS, seq.half(i0 + k + NR - 1), n_tokens);
+            __builtin_amdgcn_sched_barrier(0);
+            if (fine_now) v_compute_half<HV>(acc, ring.hi[k], nib[k & 1], ring.sb[k]);
+            else v_compute_half_coarse<HV>(acc, ring.hi[k], ring.sb[k]);
+            pin_accumulators(acc);
+            __builtin_amdgcn_sched_barrier(0);
+            fine_now = fine_next;
+        }
     }
 }
 

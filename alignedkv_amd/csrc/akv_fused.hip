@@ -229,8 +229,13 @@ struct MiddleArgs {
     int persist;  // this kernel appends the token (it is not in the rest buffers / planes yet)
 };
 
-template <int D, int NT>
-__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh);
+struct NoHook {
+    __device__ __forceinline__ void operator()() const {}
+};
+// hook: called once the loads that depend on nothing have been requested (a caller that goes on in the same
+// workgroup requests its own data there: loads return in order, so these come back first)
+template <int D, int NT, typename Hook = NoHook>
+__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u32 *amin_lds = nullptr, Hook hook = Hook());
 
 // ------------------------------------------------------------------------------------------------
 // K pass.  grid (ceil(n_blocks / (4*blocks_per_wave)), H, B), 256 threads.
@@ -390,8 +395,8 @@ __device__ __forceinline__ void decode_scores8(const u32x4 w, const unsigned sho
 }
 
 // NT threads (a multiple of 256) of one workgroup run the stage for one (batch, head).
-template <int D, int NT>
-__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
+template <int D, int NT, typename Hook>
+__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u32 *amin_lds, Hook hook) {
     constexpr int VPT = 4;                    // 16-byte score vectors a thread keeps in registers
     constexpr int NW = NT / 64;               // waves
     __shared__ float red[NW];
@@ -450,16 +455,22 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
     }
     // (a) append the token: rest buffers and column maxima (extension/k_cache_file.py:98-101).
     //     vcm_mine: this thread's channel of the V column maxima after the update (threads < D).
+    static_assert(D <= NT, "one channel per thread");
     u32 vcm_mine = 0;
-    for (int d = tid; d < D; d += NT) {
+    {
+        const bool on = tid < D;
+        const int d = on ? tid : 0;
         u32 kc = a.kcm[(int64_t)bh_kv * D + d], vc = a.vcm[(int64_t)bh_kv * D + d];
+        const u32 kb = knew[d], vb = vnew[d];
+        __builtin_amdgcn_sched_barrier(0);
+        hook();
+        __builtin_amdgcn_sched_barrier(0);
         if (a.persist) {
             // every query head of the group derives the updated maxima itself (max is idempotent, so it does
             // not matter whether it reads them before or after the owner's store); only the owner stores
-            const u32 kb = knew[d], vb = vnew[d];
             kc = max(kc, exp_field(kb));
             vc = max(vc, exp_field(vb));
-            if (owner) {
+            if (owner && on) {
                 const int64_t at = (((int64_t)b * cb + newest) * Hkv + h) * D + d;
                 a.restk[at] = (unsigned short)kb;
                 a.restv[at] = (unsigned short)vb;
@@ -655,6 +666,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh) {
 #pragma unroll
             for (int w = 1; w < NW; ++w) mn = min(mn, red_min[w]);
             a.amin[bh] = (uint8_t)mn;
+            if (amin_lds != nullptr) *amin_lds = mn;   // for a caller that goes on in the same workgroup
         }
     } else {
         lds_barrier();
@@ -700,6 +712,47 @@ template <int D, int NT>
 __global__ __launch_bounds__(NT) void fused_middle_kernel(MiddleArgs a) {
     middle_body<D, NT>(a, blockIdx.x);
 }
+
+// Middle stage, V pass and final sum of one (batch, head) by one workgroup of 16 waves.
+template <int D, bool REF>
+__device__ __forceinline__ void row_tail(const uint8_t *__restrict__ v_first_8, const uint8_t *__restrict__ v_mid_4,
+                                         const uint8_t *__restrict__ v_last_4, const MiddleArgs &ma,
+                                         unsigned short *__restrict__ out, uint8_t *__restrict__ v_levels_out,
+                                         uint8_t *__restrict__ amin_out, float (*wave_part)[D]) {
+    constexpr int NT = 1024, NW = NT / 64;
+    const int wave = threadIdx.x >> 6;
+    const int bh = blockIdx.x;
+    // ---- middle: append, tail scores, softmax, probe, threshold, tail output
+    middle_body<D, NT>(ma, bh);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    // ---- V pass: wave w accumulates tokens [w*tpw, (w+1)*tpw)
+    int R, nrest_unused;
+    seq_state(ma.g, bh / ma.g.Hq, R, nrest_unused);
+    const unsigned char amin = REF ? 0 : ma.amin[bh];
+    if (!REF && amin_out != nullptr && threadIdx.x == 0) amin_out[bh] = amin;
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    {
+        // wave w takes the token groups w, w + 16, ... (128 tokens each): neighbouring waves, neighbouring rows
+        constexpr int GT = 2 * (D == 256 ? 32 : 64);
+        const int64_t row0 = (int64_t)bh * ma.g.max_seq_len;
+        v_accumulate_range<D, REF>(v_first_8 + row0 * D, v_mid_4 + row0 * (D / 2), v_last_4 + row0 * (D / 2), R,
+                                   ma.probs + (int64_t)bh * ma.g.row_stride, amin, wave * GT, R, acc,
+                                   v_levels_out != nullptr ? v_levels_out + (int64_t)bh * R : nullptr, NW);
+    }
+    v_fold_lanes<D, NW>(acc, wave_part);
+    __syncthreads();
+    for (int d = threadIdx.x; d < D; d += NT) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += wave_part[w][d];
+        const float o16 = half_bits_to_float(float_to_half_bits(sum));
+        out[(int64_t)bh * D + d] = float_to_half_bits(o16 + half_bits_to_float(ma.otail[(int64_t)bh * D + d]));
+    }
+}
+
 
 // ------------------------------------------------------------------------------------------------
 // Whole step in one launch: one workgroup of 16 waves per (batch, head) runs the K pass, the middle
@@ -756,26 +809,48 @@ __global__ __launch_bounds__(1024) void mono_step_kernel(
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
-    // ---- middle: append, tail scores, softmax, probe, threshold, tail output
-    middle_body<D, NT>(ma, bh);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
-    // ---- V pass: wave w accumulates tokens [w*tpw, (w+1)*tpw)
+    row_tail<D, REF>(v_first_8, v_mid_4, v_last_4, ma, out, v_levels_out, amin_out, wave_part);
+}
+
+// Second half of a step in one launch: the middle stage, the V pass and the final sum for one (batch, head) per
+// workgroup of 8 waves, after a K pass that ran as a launch of its own.  With about as many (batch, head) pairs as
+// compute units (or a multiple of them) every unit streams one row of V planes from start to end: no partial sums,
+// no combine launch, and the first high-byte tiles of every wave travel while the middle stage runs.
+// grid (B*H), 512 threads.
+template <int D, bool REF, int NR, int PF>
+__global__ __launch_bounds__(512) void tail_step_kernel(const uint8_t *__restrict__ v_first_8,
+                                                        const uint8_t *__restrict__ v_mid_4,
+                                                        const uint8_t *__restrict__ v_last_4, MiddleArgs ma,
+                                                        unsigned short *__restrict__ out,
+                                                        uint8_t *__restrict__ v_levels_out,
+                                                        uint8_t *__restrict__ amin_out) {
+    constexpr int NT = 512, NW = NT / 64;
+    __shared__ float wave_part[NW][D];
+    __shared__ u32 row_amin;
+    const int wave = threadIdx.x >> 6;
+    const int bh = blockIdx.x;
     int R, nrest_unused;
     seq_state(ma.g, bh / ma.g.Hq, R, nrest_unused);
-    const unsigned char amin = REF ? 0 : ma.amin[bh];
+    const int64_t row0 = (int64_t)bh * ma.g.max_seq_len;
+    const uint8_t *f8 = v_first_8 + row0 * D, *m4 = v_mid_4 + row0 * (D / 2), *l4 = v_last_4 + row0 * (D / 2);
+    // wave w takes the half tiles w, w + 8, ...
+    VSeq seq;
+    seq.wave = wave; seq.n_waves = NW;
+    seq.n_halves = (R + VStream<D>::HT - 1) / VStream<D>::HT;
+    seq.n_per_wave = (seq.n_halves + NW - 1) / NW;
+    VRing<D, NR> ring;
+    middle_body<D, NT>(ma, bh, &row_amin, [&]() { v_stream_prefetch<D, NR, PF>(ring, f8, R, seq); });
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    const unsigned char amin = REF ? 0 : (unsigned char)row_amin;
     if (!REF && amin_out != nullptr && threadIdx.x == 0) amin_out[bh] = amin;
     float acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    {
-        // wave w takes the token groups w, w + 16, ... (128 tokens each): neighbouring waves, neighbouring rows
-        constexpr int GT = 2 * (D == 256 ? 32 : 64);
-        const int64_t row0 = (int64_t)bh * ma.g.max_seq_len;
-        v_accumulate_range<D, REF>(v_first_8 + row0 * D, v_mid_4 + row0 * (D / 2), v_last_4 + row0 * (D / 2), R,
-                                   ma.probs + (int64_t)bh * ma.g.row_stride, amin, wave * GT, R, acc,
-                                   v_levels_out != nullptr ? v_levels_out + (int64_t)bh * R : nullptr, NW);
-    }
+    const unsigned short *prow = ma.probs + (int64_t)bh * ma.g.row_stride;
+    v_stream_run<D, REF, NR, PF>(ring, f8, m4, l4, R, prow, amin, seq, acc);
+    if (v_levels_out != nullptr)
+        for (int t = threadIdx.x; t < R; t += NT) v_levels_out[(int64_t)bh * R + t] = (uint8_t)(REF ? 0 : v_level(amin, prow[t]));
     v_fold_lanes<D, NW>(acc, wave_part);
     __syncthreads();
     for (int d = threadIdx.x; d < D; d += NT) {
@@ -885,6 +960,8 @@ static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
     l.total = l.v_chunks + up((size_t)B * sizeof(int));
     return l;
 }
+
+constexpr int tail_rows_per_cu = 2, tail_max_tokens = 8192;
 
 template <int D>
 static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint8_t *vm4, uint8_t *vl4, uint8_t *kcm,
@@ -1051,6 +1128,30 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
     }
     mark(1, st);
+    // Second half of the step in one launch (see tail_step_kernel)
+    // It is used when the (batch, head) pairs spread evenly over the compute units (every unit gets the same one or
+    // two rows) and the rows are not long: measured on MI355X with 32 heads x 128, against the three launches it
+    // replaces: 30.2 vs 34.8 us per step at batch 8 x 1024 tokens, 76.0 vs 78.7 at 8 x 4096, 141.6 vs 145.9 at
+    // 16 x 4096; level at 32 x 4096 and behind at 8 x 16384 (one workgroup per unit streams at 4.5 TB/s, the V pass
+    // of many small workgroups at 6).
+    const int cus = compute_units();
+    bool tail = cus > 0 && (B * Hq) % cus == 0 && (B * Hq) / cus <= tail_rows_per_cu && R <= tail_max_tokens;
+    { AKV_TUNE("AKV_TUNE_TAIL", v); if (has_v) tail = v != 0; }
+    tail = tail && n_blocks >= 1 && geo.G == 1 && !ragged && !(literal_broadcast && !ref);
+    if (tail) {
+        if (ref)
+            hipLaunchKernelGGL((tail_step_kernel<D, true, 4, 3>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
+                               reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out);
+        else
+            hipLaunchKernelGGL((tail_step_kernel<D, false, 4, 3>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
+                               reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out);
+        mark(2, st);
+        mark(3, st);
+        mark(4, st);
+        mark(5, st);
+        mark(6, st);
+        return check_launch("decode_step(tail)");
+    }
     {
         // threads per (batch, head) row: a thread keeps 32 scores in registers between the softmax passes, so
         // rows above 8192 / 16384 tokens get 512 / 1024 threads (512 and 1024 measure level with 256 at 4096 tokens)

@@ -25,6 +25,19 @@ int check_launch(const char *what) {
 
 int g_tune_epoch = 0;
 
+int compute_units() {
+    // per device: a process may use several
+    static int cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+        cached[dev] = n > 0 ? n : -1;
+    }
+    return cached[dev] > 0 ? cached[dev] : 0;
+}
+
 }  // namespace akv
 
 extern "C" int akv_reload_tuning(void) {

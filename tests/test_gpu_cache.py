@@ -202,16 +202,19 @@ def test_fused_step_rejects_bad_state():
 
 
 @pytest.mark.parametrize("reference", [False, True])
-def test_one_launch_step_matches_the_four_launch_step(monkeypatch, reference):
-    """AKV_TUNE_MONO=1 runs the whole step as one kernel (one 16-wave workgroup per (batch, head)); it must
-    agree with the four-launch step: identical fetch levels and threshold, outputs within 1e-3."""
+@pytest.mark.parametrize("switch,D,k_block", [("AKV_TUNE_MONO", 128, 64), ("AKV_TUNE_TAIL", 128, 64), ("AKV_TUNE_TAIL", 128, 256),
+                                              ("AKV_TUNE_TAIL", 64, 64), ("AKV_TUNE_TAIL", 256, 64)])
+def test_one_launch_step_matches_the_four_launch_step(monkeypatch, reference, switch, D, k_block):
+    """AKV_TUNE_MONO=1 runs the whole step as one kernel (one 16-wave workgroup per (batch, head)), AKV_TUNE_TAIL=1
+    everything after the K pass as one kernel (one 8-wave workgroup per (batch, head)); both must agree with the
+    four-launch step: identical fetch levels and threshold, outputs within 1e-3."""
     from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
-    B, H, D, prefill, steps = 2, 8, 128, 1100, 70
+    B, H, prefill, steps = 2, 8, 1100, 70
     q, k, v = make_qkv(B, prefill + steps, H, D, seed=123)
     rng = np.random.default_rng(8)
     caches = []
     for _ in range(2):
-        c = QuantizedCache_AlignedKV(cfg(H, D), B, prefill + steps + 64, "cuda", torch.half)
+        c = QuantizedCache_AlignedKV(cfg(H, D), B, prefill + steps + 64, "cuda", torch.half, k_block=k_block)
         c.reference = reference
         c.key_cache[0].save(dev(k[:, :prefill]), 0, prefill)
         c.value_cache[0].save(dev(v[:, :prefill]), 0, prefill)
@@ -221,10 +224,10 @@ def test_one_launch_step_matches_the_four_launch_step(monkeypatch, reference):
     lib = load_library()
     for t in range(prefill, prefill + steps):
         qt = dev(rng.standard_normal((B, 1, H, D)).astype(np.float16))
-        monkeypatch.setenv("AKV_TUNE_MONO", "0")
+        monkeypatch.setenv(switch, "0")
         lib.akv_reload_tuning()      # the switches are read once and again after this call
         o4 = caches[0].auto_compute(qt, dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None)
-        monkeypatch.setenv("AKV_TUNE_MONO", "1")
+        monkeypatch.setenv(switch, "1")
         lib.akv_reload_tuning()
         o1 = caches[1].auto_compute(qt, dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None)
         assert (o4.float() - o1.float()).abs().max().item() <= 1e-3
@@ -236,5 +239,5 @@ def test_one_launch_step_matches_the_four_launch_step(monkeypatch, reference):
     k0, k1 = caches[0].key_cache[0], caches[1].key_cache[0]
     assert torch.equal(k0.k_cache_first_8, k1.k_cache_first_8) and torch.equal(k0.k_cache_last_4, k1.k_cache_last_4)
     assert k0.reststartpos == k1.reststartpos == (prefill + steps) // 64 * 64
-    monkeypatch.delenv("AKV_TUNE_MONO")
+    monkeypatch.delenv(switch)
     lib.akv_reload_tuning()
