@@ -133,6 +133,9 @@ constexpr int kSkip = 0x7fffffff;   // an offset no plane slice reaches
 // these: the eight XCDs have separate L2 caches that are only reconciled at kernel boundaries, and a
 // device-wide fence (write back + invalidate of a whole L2) costs far more than the few bytes exchanged.
 constexpr int kDeviceScope = 1 << 4;
+// Plane bytes are read once per step: non-temporal loads (they do not displace what the compute unit's cache holds
+// and are not kept in it).  Measured on the V planes at batch 8 x 32 heads x 4096 tokens: 25.2 instead of 26.8 us.
+constexpr int kStream = 1 << 1;
 __device__ __forceinline__ void store_u16_device(const __amdgpu_buffer_rsrc_t r, int byte_off, unsigned short v) {
     __builtin_amdgcn_raw_buffer_store_b16((short)v, r, byte_off, 0, kDeviceScope);
 }

@@ -39,7 +39,7 @@ __device__ __forceinline__ void k_issue_half_h(KHalfTile<HG> &t, const __amdgpu_
     const int lane = threadIdx.x & 63;
 #pragma unroll
     for (int g = 0; g < HG; ++g)
-        t.h[g] = __builtin_amdgcn_raw_buffer_load_b128(rH, blk * (D * 64) + (g0 + g) * 1024 + lane * 16, 0, 0);
+        t.h[g] = __builtin_amdgcn_raw_buffer_load_b128(rH, blk * (D * 64) + (g0 + g) * 1024 + lane * 16, 00, kStream);
 }
 
 template <int D, int HG>
@@ -52,8 +52,8 @@ __device__ __forceinline__ void k_issue_half_ml(KHalfTile<HG> &t, const __amdgpu
         const int gg = g0 + g;
         const int mo = ((need_mid >> gg) & 1u) ? blk * (D * 32) + gg * 512 + lane * 8 : kSkip;
         const int lo = ((need_last >> gg) & 1u) ? blk * (D * 32) + gg * 512 + lane * 8 : kSkip;
-        t.m[g] = __builtin_amdgcn_raw_buffer_load_b64(rM, mo, 0, 0);
-        t.l[g] = __builtin_amdgcn_raw_buffer_load_b64(rL, lo, 0, 0);
+        t.m[g] = __builtin_amdgcn_raw_buffer_load_b64(rM, mo, 00, kStream);
+        t.l[g] = __builtin_amdgcn_raw_buffer_load_b64(rL, lo, 00, kStream);
     }
 }
 
@@ -164,7 +164,7 @@ __device__ __forceinline__ void k256_issue_h(KHalfTile<HG> &t, const __amdgpu_bu
 #pragma unroll
     for (int g = 0; g < HG; ++g) {
         const int c = 4 * (g0 + g) + cs;
-        t.h[g] = __builtin_amdgcn_raw_buffer_load_b128(rH, blk * (D * 256) + c * 256 + piece * 16, 0, 0);
+        t.h[g] = __builtin_amdgcn_raw_buffer_load_b128(rH, blk * (D * 256) + c * 256 + piece * 16, 00, kStream);
     }
 }
 
@@ -177,8 +177,8 @@ __device__ __forceinline__ void k256_issue_ml(KHalfTile<HG> &t, const __amdgpu_b
     for (int g = 0; g < HG; ++g) {
         const int gg = g0 + g, c = 4 * gg + cs;
         const int off = blk * (D * 128) + c * 128 + piece * 8;
-        t.m[g] = __builtin_amdgcn_raw_buffer_load_b64(rM, ((need_mid >> gg) & 1u) ? off : kSkip, 0, 0);
-        t.l[g] = __builtin_amdgcn_raw_buffer_load_b64(rL, ((need_last >> gg) & 1u) ? off : kSkip, 0, 0);
+        t.m[g] = __builtin_amdgcn_raw_buffer_load_b64(rM, ((need_mid >> gg) & 1u) ? off : kSkip, 00, kStream);
+        t.l[g] = __builtin_amdgcn_raw_buffer_load_b64(rL, ((need_last >> gg) & 1u) ? off : kSkip, 00, kStream);
     }
 }
 
@@ -277,7 +277,7 @@ __device__ __forceinline__ void v_issue_half_h(VHighPart<HV> &t, const __amdgpu_
 #pragma unroll
     for (int u = 0; u < HV; ++u) {
         const int tok = base + u * TPL + tl;
-        t.h[u] = __builtin_amdgcn_raw_buffer_load_b128(rH, tok < t_end ? tok * D + cl * 16 : kSkip, 0, 0);
+        t.h[u] = __builtin_amdgcn_raw_buffer_load_b128(rH, tok < t_end ? tok * D + cl * 16 : kSkip, 0, kStream);
     }
 }
 
@@ -293,8 +293,8 @@ __device__ __forceinline__ void v_issue_half_ml(VLowPart<HV> &t, const __amdgpu_
         const int tok = base + u * TPL + tl;
         const bool valid = tok < t_end;
         const int level = REF ? 0 : v_level(amin, (unsigned short)sb[u]);
-        t.m[u] = __builtin_amdgcn_raw_buffer_load_b64(rM, (valid && level < 2) ? tok * (D / 2) + cl * 8 : kSkip, 0, 0);
-        t.l[u] = __builtin_amdgcn_raw_buffer_load_b64(rL, (valid && level == 0) ? tok * (D / 2) + cl * 8 : kSkip, 0, 0);
+        t.m[u] = __builtin_amdgcn_raw_buffer_load_b64(rM, (valid && level < 2) ? tok * (D / 2) + cl * 8 : kSkip, 00, kStream);
+        t.l[u] = __builtin_amdgcn_raw_buffer_load_b64(rL, (valid && level == 0) ? tok * (D / 2) + cl * 8 : kSkip, 00, kStream);
         t.cm[u] = level == 2 ? 0x88888888u : 0u;
         t.cl[u] = level == 1 ? 0x88888888u : 0u;
     }
@@ -497,6 +497,7 @@ __device__ __forceinline__ void v_stream_run(VRing<D, NR> &ring, const uint8_t *
                                              float *acc) {
     using S = VStream<D>;
     static_assert(NR % 2 == 0, "the two nibble buffers alternate with the ring slots");
+    static_assert(NR >= 4, "the levels of half tile k + 1 are looked at before half tile k + NR - 1 is requested");
     constexpr int HV = S::HV;
     const int lane = threadIdx.x & 63, tl = lane / S::LPR;
     const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
@@ -517,7 +518,7 @@ __device__ __forceinline__ void v_stream_run(VRing<D, NR> &ring, const uint8_t *
     bool fine_now = v_half_is_fine<REF, HV>(ring.sb[0], amin);
     if (fine_now) v_issue_half_ml<D, REF, HV>(nib[0], rM, rL, seq.half(0) * S::HT, n_tokens, ring.sb[0], amin);
     __builtin_amdgcn_sched_barrier(0);
-    for (int i0 = 0; i0 < seq.n_per_wave; i0 += NR) {
+    auto round = [&](int i0) {
 #pragma unroll
         for (int k = 0; k < NR; ++k) {
             // nibble rows of the next half tile first, then the newest probabilities and high bytes
@@ -533,6 +534,13 @@ __device__ __forceinline__ void v_stream_run(VRing<D, NR> &ring, const uint8_t *
             __builtin_amdgcn_sched_barrier(0);
             fine_now = fine_next;
         }
+    };
+    // The first round stands outside the loop: the compiler derives the number of loads that may stay in flight at
+    // a wait from every path that reaches it, and the path from the set-up above (fewer requests behind the one
+    // waited for) would otherwise hold every round of the loop to the depth of the first.
+    if (seq.n_per_wave > 0) {
+        round(0);
+        for (int i0 = NR; i0 < seq.n_per_wave; i0 += NR) round(i0);
     }
 }
 

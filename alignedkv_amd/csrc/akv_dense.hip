@@ -70,7 +70,7 @@ __global__ __launch_bounds__(256) void dense_k_pass_kernel(const unsigned short 
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int t = base + u * 4 + tl;
-            kv[u] = __builtin_amdgcn_raw_buffer_load_b128(rK, t < t_end ? t * (D * 2) + cl * 16 : kSkip, 0, 0);
+            kv[u] = __builtin_amdgcn_raw_buffer_load_b128(rK, t < t_end ? t * (D * 2) + cl * 16 : kSkip, 00, kStream);
         }
     };
     auto finish = [&](const u32x4 *kv, int base) {
@@ -218,7 +218,7 @@ __global__ __launch_bounds__(256) void dense_v_pass_kernel(const unsigned short 
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
             const int t = base + u * 4 + tl;
-            vv[u] = __builtin_amdgcn_raw_buffer_load_b128(rV, t < t_end ? t * (D * 2) + cl * 16 : kSkip, 0, 0);
+            vv[u] = __builtin_amdgcn_raw_buffer_load_b128(rV, t < t_end ? t * (D * 2) + cl * 16 : kSkip, 00, kStream);
             sb[u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < t_end ? t * 2 : kSkip, 0, 0);
         }
     };

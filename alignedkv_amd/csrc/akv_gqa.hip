@@ -173,8 +173,8 @@ __device__ __forceinline__ void v_group_issue(VHalfTile<HV> &t, const __amdgpu_b
         int level = 2;   // finest level any head of the group asks for
 #pragma unroll
         for (int h = 0; h < GH; ++h) level = min(level, REF ? 0 : v_level(amin[h], (unsigned short)p.s[h][half * HV + u]));
-        t.m[u] = __builtin_amdgcn_raw_buffer_load_b64(rM, (valid && level < 2) ? tok * (D / 2) + cl * 8 : kSkip, 0, 0);
-        t.l[u] = __builtin_amdgcn_raw_buffer_load_b64(rL, (valid && level == 0) ? tok * (D / 2) + cl * 8 : kSkip, 0, 0);
+        t.m[u] = __builtin_amdgcn_raw_buffer_load_b64(rM, (valid && level < 2) ? tok * (D / 2) + cl * 8 : kSkip, 00, kStream);
+        t.l[u] = __builtin_amdgcn_raw_buffer_load_b64(rL, (valid && level == 0) ? tok * (D / 2) + cl * 8 : kSkip, 00, kStream);
     }
 }
 

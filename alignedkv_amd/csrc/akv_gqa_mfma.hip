@@ -77,15 +77,15 @@ struct KTaskTile {   // one channel group: 4 channels x SL slots per lane
 template <int NB>
 __device__ __forceinline__ void load_bytes(u32 *dst, const __amdgpu_buffer_rsrc_t r, int off) {
     if constexpr (NB == 16) {
-        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, off, 00, kStream);
         dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
     } else if constexpr (NB == 8) {
-        const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0);
+        const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(r, off, 00, kStream);
         dst[0] = v.x; dst[1] = v.y;
     } else if constexpr (NB == 4) {
-        dst[0] = __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0);
+        dst[0] = __builtin_amdgcn_raw_buffer_load_b32(r, off, 00, kStream);
     } else {
-        dst[0] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0);
+        dst[0] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, off, 00, kStream);
     }
 }
 
