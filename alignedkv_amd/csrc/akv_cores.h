@@ -461,21 +461,37 @@ struct VSeq {
     __device__ __forceinline__ int half(int i) const { return i < n_per_wave ? i * n_waves + wave : n_halves; }
 };
 
+// High bytes of half tile `half`: one address per lane, the HV rows at constant distances from it.  A half tile past the
+// end of the row (VSeq::half returns n_halves for those) lies outside the buffer resource: the loads return zeros and
+// fetch nothing, no select per row is needed (the rows of a sequence are whole 64-token blocks, so a half tile is
+// inside or outside as a whole).
+template <int D>
+__device__ __forceinline__ void v_stream_issue_high(VHighPart<VStream<D>::HV> &t, const __amdgpu_buffer_rsrc_t rH, int half) {
+    using S = VStream<D>;
+    const int lane = threadIdx.x & 63;
+    const int vo = (half * S::HT + lane / S::LPR) * D + (lane % S::LPR) * 16;
+#pragma unroll
+    for (int u = 0; u < S::HV; ++u) t.h[u] = __builtin_amdgcn_raw_buffer_load_b128(rH, vo + u * (S::TPL * D), 0, kStream);
+}
+
+template <int D>
+__device__ __forceinline__ void v_stream_issue_probs(u32 *sb, const __amdgpu_buffer_rsrc_t rS, int half) {
+    using S = VStream<D>;
+    const int lane = threadIdx.x & 63;
+    const int vo = (half * S::HT + lane / S::LPR) * 2;
+#pragma unroll
+    for (int u = 0; u < S::HV; ++u)
+        sb[u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, vo + u * (S::TPL * 2), 0, 0);
+}
+
 // requests half tile `half` (tokens half * HT ...) into ring slot k
 template <int D, int NR>
 __device__ __forceinline__ void v_stream_issue(VRing<D, NR> &ring, int k, const __amdgpu_buffer_rsrc_t rH,
-                                               const __amdgpu_buffer_rsrc_t rS, int half, int n_tokens) {
-    using S = VStream<D>;
-    const int lane = threadIdx.x & 63, tl = lane / S::LPR;
-    const int base = half * S::HT;
+                                               const __amdgpu_buffer_rsrc_t rS, int half) {
     // the probabilities first: loads return in order, and the fetch levels of a half tile are looked at one half
     // tile before its high bytes are needed
-#pragma unroll
-    for (int u = 0; u < S::HV; ++u) {
-        const int t = base + u * S::TPL + tl;
-        ring.sb[k][u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < n_tokens ? t * 2 : kSkip, 0, 0);
-    }
-    v_issue_half_h<D, S::HV>(ring.hi[k], rH, base, n_tokens);
+    v_stream_issue_probs<D>(ring.sb[k], rS, half);
+    v_stream_issue_high<D>(ring.hi[k], rH, half);
 }
 
 // the first PF half tiles of the wave: before anything the caller has to do first (they depend on nothing but
@@ -483,11 +499,10 @@ __device__ __forceinline__ void v_stream_issue(VRing<D, NR> &ring, int k, const 
 // the high bytes of the half tiles PF .. NR - 2)
 template <int D, int NR, int PF>
 __device__ __forceinline__ void v_stream_prefetch(VRing<D, NR> &ring, const uint8_t *f8, int n_tokens, const VSeq &seq) {
-    using S = VStream<D>;
     static_assert(PF <= NR - 1, "the ring keeps one slot for the half tile being multiplied");
     const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
 #pragma unroll
-    for (int k = 0; k < PF; ++k) v_issue_half_h<D, S::HV>(ring.hi[k], rH, seq.half(k) * S::HT, n_tokens);
+    for (int k = 0; k < PF; ++k) v_stream_issue_high<D>(ring.hi[k], rH, seq.half(k));
     __builtin_amdgcn_sched_barrier(0);
 }
 
@@ -499,21 +514,15 @@ __device__ __forceinline__ void v_stream_run(VRing<D, NR> &ring, const uint8_t *
     static_assert(NR % 2 == 0, "the two nibble buffers alternate with the ring slots");
     static_assert(NR >= 4, "the levels of half tile k + 1 are looked at before half tile k + NR - 1 is requested");
     constexpr int HV = S::HV;
-    const int lane = threadIdx.x & 63, tl = lane / S::LPR;
     const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
     const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_tokens * (D / 2));
     const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_tokens * (D / 2));
     const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)n_tokens * 2);
 #pragma unroll
-    for (int k = PF; k < NR - 1; ++k) v_issue_half_h<D, HV>(ring.hi[k], rH, seq.half(k) * S::HT, n_tokens);
+    for (int k = PF; k < NR - 1; ++k) v_stream_issue_high<D>(ring.hi[k], rH, seq.half(k));
     // probabilities of the half tiles requested so far
 #pragma unroll
-    for (int k = 0; k < NR - 1; ++k)
-#pragma unroll
-        for (int u = 0; u < HV; ++u) {
-            const int t = seq.half(k) * S::HT + u * S::TPL + tl;
-            ring.sb[k][u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < n_tokens ? t * 2 : kSkip, 0, 0);
-        }
+    for (int k = 0; k < NR - 1; ++k) v_stream_issue_probs<D>(ring.sb[k], rS, seq.half(k));
     VLowPart<HV> nib[2];
     bool fine_now = v_half_is_fine<REF, HV>(ring.sb[0], amin);
     if (fine_now) v_issue_half_ml<D, REF, HV>(nib[0], rM, rL, seq.half(0) * S::HT, n_tokens, ring.sb[0], amin);
@@ -526,7 +535,7 @@ __device__ __forceinline__ void v_stream_run(VRing<D, NR> &ring, const uint8_t *
             const bool fine_next = v_half_is_fine<REF, HV>(ring.sb[kn], amin);
             if (fine_next)
                 v_issue_half_ml<D, REF, HV>(nib[(k + 1) & 1], rM, rL, seq.half(i0 + k + 1) * S::HT, n_tokens, ring.sb[kn], amin);
-            v_stream_issue<D, NR>(ring, (k + NR - 1) % NR, rH, rS, seq.half(i0 + k + NR - 1), n_tokens);
+            v_stream_issue<D, NR>(ring, (k + NR - 1) % NR, rH, rS, seq.half(i0 + k + NR - 1));
             __builtin_amdgcn_sched_barrier(0);
             if (fine_now) v_compute_half<HV>(acc, ring.hi[k], nib[k & 1], ring.sb[k]);
             else v_compute_half_coarse<HV>(acc, ring.hi[k], ring.sb[k]);
