@@ -29,7 +29,7 @@ HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
 # HBM bytes per launch of the K pass at the default workload, from the rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE runs summarised in profiles/decode_step_c2_hbm_traffic.txt (256-token K blocks) and decode_step_c2_k_block64_hbm_traffic.txt (FETCH_SIZE scaled x2.0 by the
 # known-size copy kernel, WRITE_SIZE x1.0): 222.4 MiB read + 2.0 MiB written.
-MEASURED_K_PASS_TRAFFIC = {(8, 32, 128, 4096, "outlier", 64): int((222.3 + 2.0) * (1 << 20)),
+MEASURED_K_PASS_TRAFFIC = {(8, 32, 128, 4096, "outlier", 64): int((222.4 + 2.0) * (1 << 20)),
                            (8, 32, 128, 4096, "outlier", 256): int((198.0 + 2.0) * (1 << 20))}
 
 
