@@ -259,4 +259,66 @@ class _AlignedKVModule:
                                           int(bool(reference)), int(bool(literal_broadcast)), _stream_ptr(dev)), lib)
 
 
+class PreparedDecodeStep:
+    """akv_decode_step_gqa for one layer of a multi-head cache with everything that does not change between its steps
+    checked and converted once: plane, column-maximum, rest-buffer, score and workspace pointers and the geometry.
+    A call checks only the three token tensors and the output.  Made by `cuda_module.prepare_decode_step`; `key`
+    lets the owner notice that one of the captured tensors was replaced (then it prepares again)."""
+
+    def __init__(self, lib, static_head, static_mid, geometry, tok_bytes, device, stream, key, keep):
+        self._fn = lib.akv_decode_step_gqa
+        self._lib = lib
+        self._head = static_head        # 10 pointers: planes, column maxima, rest buffers
+        self._mid = static_mid          # scores, probs, row_stride, workspace, workspace bytes
+        self._geo = geometry            # bsz, q heads, kv heads, n_max_blocks, max_seq_len, head_dim, d_block, k_block, top_max_k
+        self._tok = tok_bytes
+        self.device = device
+        self.stream = stream
+        self.key = key
+        self._keep = keep               # the tensors behind the pointers
+
+    def __call__(self, q, k_new, v_new, out, mask, mask_stride, cur_len, reference, literal_broadcast,
+                 k_levels_out=None, v_levels_out=None, amin_out=None):
+        tok = self._tok
+        for t in (q, k_new, v_new, out):
+            if t.dtype != torch.uint8 or t.numel() != tok or not t.is_contiguous() or t.device != self.device:
+                raise RuntimeError("decode step: q, k_new, v_new and out must be contiguous uint8 views of "
+                                   f"{tok} bytes on {self.device}")
+        rc = self._fn(*self._head, q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), _ptr(mask), mask_stride,
+                      out.data_ptr(), *self._mid, _ptr(k_levels_out), _ptr(v_levels_out), _ptr(amin_out), *self._geo,
+                      cur_len, None, int(bool(reference)), int(bool(literal_broadcast)), self.stream)
+        if rc != 0:
+            check(rc, self._lib)
+
+
+def _prepare_decode_step(self, k_planes, v_planes, k_exp_column_max, v_exp_column_max, restk, restv, scores, probs,
+                         bsz, n_kv_heads, n_max_blocks, max_seq_len, head_dim, d_block, k_block, top_max_k, key=None):
+    """The checks of `decode_step_gqa` on the per-layer tensors of a multi-head cache, once; returns a
+    PreparedDecodeStep bound to the current stream of their device (a call on another stream needs another one).
+    n_max_blocks counts K plane blocks of k_block tokens."""
+    lib = load_library()
+    dev = k_planes[0].device
+    kplane = bsz * n_kv_heads * n_max_blocks * head_dim * k_block
+    vplane = bsz * n_kv_heads * max_seq_len * head_dim
+    tok = bsz * n_kv_heads * head_dim * 2
+    for name, t, n in (("k_first_8", k_planes[0], kplane), ("k_mid_4", k_planes[1], kplane // 2),
+                       ("k_last_4", k_planes[2], kplane // 2), ("v_first_8", v_planes[0], vplane),
+                       ("v_mid_4", v_planes[1], vplane // 2), ("v_last_4", v_planes[2], vplane // 2),
+                       ("k_exp_column_max", k_exp_column_max, tok // 2), ("v_exp_column_max", v_exp_column_max, tok // 2),
+                       ("restk", restk, tok * d_block), ("restv", restv, tok * d_block)):
+        _require(name, t, n, dev)
+    row_stride = scores.shape[-1] // 2
+    _require("scores", scores, bsz * n_kv_heads * row_stride * 2, dev)
+    _require("probs", probs, bsz * n_kv_heads * row_stride * 2, dev)
+    need = lib.akv_decode_step_workspace_bytes(bsz, n_kv_heads, head_dim, max_seq_len)
+    ws = self._workspace(dev, need)
+    head = tuple(_ptr(t) for t in (*k_planes, *v_planes, k_exp_column_max, v_exp_column_max, restk, restv))
+    mid = (_ptr(scores), _ptr(probs), row_stride, _ptr(ws), ws.numel())
+    geo = (bsz, n_kv_heads, n_kv_heads, n_max_blocks, max_seq_len, head_dim, d_block, k_block, top_max_k)
+    keep = (k_planes, v_planes, k_exp_column_max, v_exp_column_max, restk, restv, scores, probs, ws)
+    return PreparedDecodeStep(lib, head, mid, geo, tok, dev, _stream_ptr(dev), key, keep)
+
+
+_AlignedKVModule.prepare_decode_step = _prepare_decode_step
+
 cuda_module = _AlignedKVModule()

@@ -89,11 +89,12 @@ class PlaneCacheBase(torch.nn.Module):
 
     def _advance_after_fused_step(self):
         """Host counters after the fused step appended one token (and flushed a full rest buffer)."""
-        self.current_cache_len += 1
-        self._restlen += 1
-        if self._restlen == column_block:
-            self._restlen = 0
-            self.reststartpos += column_block
+        d = self.__dict__     # plain integers: no need for torch.nn.Module.__setattr__ on every step
+        d["current_cache_len"] += 1
+        d["_restlen"] += 1
+        if d["_restlen"] == column_block:
+            d["_restlen"] = 0
+            d["reststartpos"] += column_block
 
     def _zero_state(self):
         # the reference leaves the rest buffer untouched here (extension/k_cache_file.py:62-67); a prefill

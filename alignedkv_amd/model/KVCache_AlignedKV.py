@@ -8,7 +8,9 @@ from typing import List, Optional
 import torch
 import torch.nn.functional as F
 
+from ..extension._plane_cache import column_block
 from ..extension.k_cache_file import K_Cache_Class
+from ..extension.KV_cache_cpp_extention import _stream_ptr, cuda_module
 from ..extension.v_cache_file import V_Cache_Class
 
 def _cache_base():
@@ -70,6 +72,7 @@ class QuantizedCache_AlignedKV(_HFCache):
         self._device = device
         self._scores = None
         self._probs = None
+        self._prepared = {}
 
     def update(self, key_states, value_states, layer_idx, cache_kwargs=None):
         raise Exception("This function is not used in AlignedKV")
@@ -120,49 +123,61 @@ class QuantizedCache_AlignedKV(_HFCache):
             return False
         return mask.reshape(mask.shape[0], mask.shape[-1]).contiguous().view(torch.uint8)
 
+    def _prepared_step(self, layer_id: int, device):
+        """The fused step of a layer with its per-layer arguments checked once (PreparedDecodeStep); prepared again
+        when a rest buffer or a column-maximum tensor was replaced (the unfused path and a prefill do that) or the
+        current stream changed."""
+        kc, vc = self.key_cache[layer_id], self.value_cache[layer_id]
+        key = (kc._rest.data_ptr(), vc._rest.data_ptr(), kc._colmax.data_ptr(), vc._colmax.data_ptr(), _stream_ptr(device))
+        st = self._prepared.get(layer_id)
+        if st is None or st.key != key:
+            B, H = self.max_batch_size, self.num_key_value_heads
+            if self._scores is None:
+                width = (kc.n_max_blocks + 1) * column_block
+                self._scores = torch.empty((B, H, width), dtype=torch.half, device=device)
+                self._probs = torch.empty((B, H, width), dtype=torch.half, device=device)
+            st = cuda_module.prepare_decode_step(
+                (kc.k_cache_first_8, kc.k_cache_mid_4, kc.k_cache_last_4),
+                (vc.v_cache_first_8, vc.v_cache_mid_4, vc.v_cache_last_4),
+                kc._colmax, vc._colmax, kc._rest.view(torch.uint8), vc._rest.view(torch.uint8),
+                self._scores.view(torch.uint8), self._probs.view(torch.uint8), B, H, kc.k_n_max_blocks,
+                self.max_cache_len, self.head_dim, column_block, kc.k_block, vc.top_max_k, key=key)
+            self._prepared[layer_id] = st
+        return st
+
     def decoding_fused(self, q, k, v, start_pos: int, mask2d, layer_id: int):
-        """One decode step through akv_decode_step; same state transitions as decoding_k + decoding_v."""
-        from ..extension.KV_cache_cpp_extention import cuda_module
-        from ..extension._plane_cache import column_block
+        """One decode step through akv_decode_step_gqa; same state transitions as decoding_k + decoding_v."""
         kc, vc = self.key_cache[layer_id], self.value_cache[layer_id]
         kc._check_save(k, start_pos, 1, "new_k")
         vc._check_save(v, start_pos, 1, "new_v")
         assert tuple(q.shape) == tuple(k.shape), f"q.shape: {tuple(q.shape)} != {tuple(k.shape)}"
+        assert kc.reststartpos + kc._restlen == start_pos
         B, H, D = self.max_batch_size, self.num_key_value_heads, self.head_dim
-        if self._scores is None:
-            width = (kc.n_max_blocks + 1) * column_block
-            self._scores = torch.empty((B, H, width), dtype=torch.half, device=q.device)
-            self._probs = torch.empty((B, H, width), dtype=torch.half, device=q.device)
+        step = self._prepared_step(layer_id, q.device)
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         out = torch.empty_like(q)
-        flushed = kc.reststartpos + (column_block if kc._restlen + 1 == column_block else 0)
         klv = vlv = amin = None
         if kc.record_levels or vc.record_levels:
+            flushed = kc.reststartpos + (column_block if kc._restlen + 1 == column_block else 0)
             klv = torch.empty((B, H, D), dtype=torch.uint8, device=q.device)
             vlv = torch.empty((B, H, flushed), dtype=torch.uint8, device=q.device) if flushed else None
             amin = torch.empty((B, H), dtype=torch.uint8, device=q.device)
-        if kc.k_block == column_block:
-            cuda_module.decode_step(
-                (kc.k_cache_first_8, kc.k_cache_mid_4, kc.k_cache_last_4),
-                (vc.v_cache_first_8, vc.v_cache_mid_4, vc.v_cache_last_4),
-                kc._colmax, vc._colmax, kc._rest.view(torch.uint8), vc._rest.view(torch.uint8),
-                q.view(torch.uint8), k.view(torch.uint8), v.view(torch.uint8), mask2d, out.view(torch.uint8),
-                self._scores.view(torch.uint8), self._probs.view(torch.uint8), B, H, kc.n_max_blocks, self.max_cache_len,
-                D, column_block, vc.top_max_k, start_pos, kc.reststartpos, kc._restlen, self.reference,
-                self.literal_broadcast, klv, vlv, amin)
+        mask_stride = 0
+        if mask2d is not None:
+            if mask2d.shape[1] < 2 * (start_pos + 1):
+                raise RuntimeError(f"mask: shape {tuple(mask2d.shape)} does not cover {start_pos + 1} halves")
+            mask_stride = 0 if mask2d.shape[0] == 1 else mask2d.stride(0) // 2
+        if q.device != torch.device("cuda", torch.cuda.current_device()):
+            with torch.cuda.device(q.device):
+                step(q.view(torch.uint8), k.view(torch.uint8), v.view(torch.uint8), out.view(torch.uint8), mask2d,
+                     mask_stride, start_pos, self.reference, self.literal_broadcast, klv, vlv, amin)
         else:
-            assert kc.reststartpos + kc._restlen == start_pos
-            cuda_module.decode_step_gqa(
-                (kc.k_cache_first_8, kc.k_cache_mid_4, kc.k_cache_last_4),
-                (vc.v_cache_first_8, vc.v_cache_mid_4, vc.v_cache_last_4),
-                kc._colmax, vc._colmax, kc._rest.view(torch.uint8), vc._rest.view(torch.uint8),
-                q.view(torch.uint8), k.view(torch.uint8), v.view(torch.uint8), mask2d, out.view(torch.uint8),
-                self._scores.view(torch.uint8), self._probs.view(torch.uint8), B, H, H, kc.k_n_max_blocks,
-                self.max_cache_len, D, column_block, vc.top_max_k, start_pos, None, self.reference, klv, vlv, amin,
-                k_block=kc.k_block, literal_broadcast=self.literal_broadcast)
+            step(q.view(torch.uint8), k.view(torch.uint8), v.view(torch.uint8), out.view(torch.uint8), mask2d,
+                 mask_stride, start_pos, self.reference, self.literal_broadcast, klv, vlv, amin)
         kc._advance_after_fused_step()
         vc._advance_after_fused_step()
-        kc.last_levels, vc.last_levels, vc.last_alignment_min = klv, vlv, amin
+        if klv is not None:
+            kc.last_levels, vc.last_levels, vc.last_alignment_min = klv, vlv, amin
         return out
 
     def decoding(self, q, k, v, start_pos: int, seqlen: int, mask, layer_id: int):
