@@ -126,6 +126,15 @@ __device__ __forceinline__ u32 rebuild_bits(u32 hi, u32 mid_nibble, u32 last_nib
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, u32 num_bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)num_bytes, 0x00020000);
 }
+// x / d for many x and one d: r = 1 / d once (a correctly rounded division), then per x a product and one
+// correction step, three instructions instead of the ten of a division.  The result equals x / d as the division
+// instruction sequence rounds it (checked on the host for 2e7 pairs with x in (0, 1], d in [1, 4096]); values too small
+// for fp16 are not looked at by the callers.
+__device__ __forceinline__ float div_by(float x, float d, float r) {
+    const float q = x * r;
+    return fmaf(fmaf(-q, d, x), r, q);
+}
+
 constexpr int kSkip = 0x7fffffff;   // an offset no plane slice reaches
 
 // Cache-policy bits of buffer loads/stores on gfx950: sc1 = device (agent) scope.  Data that one

@@ -183,16 +183,17 @@ __global__ __launch_bounds__(256) void dense_middle_kernel(DenseMiddleArgs a) {
         for (int j = 0; j < 4; ++j) sum += expf(lo_half_to_float(ww[j]) - m) + expf(hi_half_to_float(ww[j]) - m);
     });
     sum = d_block_reduce(sum, false, red);
+    const float rsum = 1.0f / sum;
     each([&](int i, const u32x4 w) {
         const u32 ww[4] = {w.x, w.y, w.z, w.w};
         u32 o[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j)
-            o[j] = (u32)float_to_half_bits(expf(lo_half_to_float(ww[j]) - m) / sum) |
-                   ((u32)float_to_half_bits(expf(hi_half_to_float(ww[j]) - m) / sum) << 16);
+            o[j] = (u32)float_to_half_bits(div_by(expf(lo_half_to_float(ww[j]) - m), sum, rsum)) |
+                   ((u32)float_to_half_bits(div_by(expf(hi_half_to_float(ww[j]) - m), sum, rsum)) << 16);
         *reinterpret_cast<u32x4 *>(prow + i * 8) = (u32x4){o[0], o[1], o[2], o[3]};
     });
-    if (t_tail <= n) prow[t_tail] = float_to_half_bits(expf(x_tail - m) / sum);
+    if (t_tail <= n) prow[t_tail] = float_to_half_bits(div_by(expf(x_tail - m), sum, rsum));
 }
 
 // V pass, head_dim 128: lane = 8 channels of one token, 4 tokens per wave-wide load, 8 loads in flight.

@@ -544,6 +544,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
             }
         const float et = tid < nrest ? expf(xt - m) : 0.f;
         sum = block_reduce<NW>(sum + et, false, red);
+        const float rsum = 1.0f / sum;
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
             const int i = tid + NT * v;
@@ -551,7 +552,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
                 u32 out[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const u32 p0 = float_to_half_bits(x[v][2 * j] / sum), p1 = float_to_half_bits(x[v][2 * j + 1] / sum);
+                    const u32 p0 = float_to_half_bits(div_by(x[v][2 * j], sum, rsum)), p1 = float_to_half_bits(div_by(x[v][2 * j + 1], sum, rsum));
                     out[j] = p0 | (p1 << 16);
                     const u32 grp = 0xffffu - (u32)(i >> 2);     // token / 32 = vector index / 4
                     best[2 * j] = max(best[2 * j], (p0 << 16) | grp);
@@ -562,7 +563,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
             }
         }
         if (tid < nrest) {
-            const unsigned short p = float_to_half_bits(et / sum);
+            const unsigned short p = float_to_half_bits(div_by(et, sum, rsum));
             prow[R + tid] = p;
             tail_p[tid] = half_bits_to_float(p);
         }
@@ -582,12 +583,13 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
         }
         const float et = tid < nrest ? expf(xt - m) : 0.f;
         sum = block_reduce<NW>(sum + et, false, red);
+        const float rsum = 1.0f / sum;
         for (int i = tid; i < nvec; i += NT) {
             decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
             u32 out[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const u32 p0 = float_to_half_bits(expf(x[2 * j] - m) / sum), p1 = float_to_half_bits(expf(x[2 * j + 1] - m) / sum);
+                const u32 p0 = float_to_half_bits(div_by(expf(x[2 * j] - m), sum, rsum)), p1 = float_to_half_bits(div_by(expf(x[2 * j + 1] - m), sum, rsum));
                 out[j] = p0 | (p1 << 16);
                 const u32 grp = 0xffffu - (u32)(i >> 2);
                 best[2 * j] = max(best[2 * j], (p0 << 16) | grp);
@@ -597,7 +599,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
             *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
         }
         if (tid < nrest) {
-            const unsigned short p = float_to_half_bits(et / sum);
+            const unsigned short p = float_to_half_bits(div_by(et, sum, rsum));
             prow[R + tid] = p;
             tail_p[tid] = half_bits_to_float(p);
         }
