@@ -159,10 +159,15 @@ def test_save_assertions_mirror_the_reference():
         kc.save(x[:, :2], 8, 2)
 
 
-def test_fused_step_with_mask_and_reference_flag():
+@pytest.mark.parametrize("tail", ["0", "1"])
+def test_fused_step_with_mask_and_reference_flag(monkeypatch, tail):
     """The fused step with an additive fp16 mask ([B,1,1,L], -inf on a few positions of one sequence)
-    equals the unfused op sequence on the same cache contents, in aligned and in reference mode."""
+    equals the unfused op sequence on the same cache contents, in aligned and in reference mode; as four launches
+    and with everything after the K pass in one."""
+    from alignedkv_amd import load_library
     from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
+    monkeypatch.setenv("AKV_TUNE_TAIL", tail)
+    load_library().akv_reload_tuning()
     B, H, D, prefill = 2, 4, 128, 150
     q, k, v = make_qkv(B, prefill + 4, H, D, seed=31)
     rng = np.random.default_rng(3)
@@ -181,6 +186,31 @@ def test_fused_step_with_mask_and_reference_flag():
             assert torch.isfinite(outs[0]).all()
             assert (outs[0].float() - outs[1].float()).abs().max().item() <= 2e-3
             assert caches[0]._probs[1, :, 3:40].abs().max().item() == 0.0
+    monkeypatch.delenv("AKV_TUNE_TAIL")
+    load_library().akv_reload_tuning()
+
+
+def test_step_on_as_many_rows_as_compute_units_matches_the_op_sequence():
+    """batch x heads = 256: the shape for which the library itself chooses the two-launch step on a 256-unit part.
+    Whatever it chooses, the fused step must agree with the unfused op sequence across a flush."""
+    from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
+    B, H, D, prefill, steps = 8, 32, 128, 190, 4
+    _, k, v = make_qkv(B, prefill + steps, H, D, seed=77)
+    q = np.random.default_rng(78).standard_normal((B, prefill + steps, H, D)).astype(np.float16)
+    caches = []
+    for fused in (True, False):
+        c = QuantizedCache_AlignedKV(cfg(H, D), B, 320, "cuda", torch.half, k_block=256 if fused else 64)
+        c.fused = fused
+        c.key_cache[0].save(dev(k[:, :prefill]), 0, prefill)
+        c.value_cache[0].save(dev(v[:, :prefill]), 0, prefill)
+        c.key_cache[0].record_levels = c.value_cache[0].record_levels = True
+        caches.append(c)
+    for t in range(prefill, prefill + steps):
+        outs = [c.auto_compute(dev(q[:, t:t + 1]), dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None) for c in caches]
+        assert (outs[0].float() - outs[1].float()).abs().max().item() <= 2e-3
+        assert torch.equal(caches[0].key_cache[0].last_levels, caches[1].key_cache[0].last_levels)
+        flips = (caches[0].value_cache[0].last_levels != caches[1].value_cache[0].last_levels).float().mean().item()
+        assert flips <= 0.01
 
 
 def test_fused_step_rejects_bad_state():
