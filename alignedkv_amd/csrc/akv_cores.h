@@ -424,21 +424,7 @@ __device__ __forceinline__ void v_accumulate(VFirstTile<D> &ft, const uint8_t *f
     }
 }
 
-// Tokens [t_begin, t_end) in groups of two batches (128 tokens, 64 for head_dim 256): any range length.
-template <int D, bool REF>
-__device__ __forceinline__ void v_accumulate_range(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_tokens,
-                                                   const unsigned short *s_row, unsigned char amin, int t_begin,
-                                                   int t_end, float *acc, uint8_t *levels_row, int group_stride = 1) {
-    constexpr int GT = 2 * (D == 256 ? 32 : 64);
-    for (int g = t_begin; g < t_end; g += GT * group_stride) {
-        VFirstTile<D> ft;
-        v_prefetch_first<D>(ft, f8, n_tokens, g, t_end);
-        v_accumulate<D, REF, 2>(ft, f8, m4, l4, n_tokens, s_row, amin, g, min(g + GT, t_end), acc, levels_row);
-    }
-}
-
-// One wave streams the half tiles first_half, first_half + half_stride, ... of a row of V planes (a half tile = HT
-// tokens): a ring of NR half tiles of high bytes, each requested together with its probabilities NR - 1 half tiles
+// One wave streams its share of the half tiles of a row of V planes (VSeq; a half tile = HT tokens): a ring of NR half tiles of high bytes, each requested together with its probabilities NR - 1 half tiles
 // before it is multiplied (neither depends on a fetch level); the nibble rows of a half tile with a token below
 // level 2 are requested one half tile ahead, before the newest high bytes, so that waiting for them does not wait
 // for those.  For callers that give a wave a long range: v_accumulate keeps one half tile in flight and leaves the

@@ -715,105 +715,6 @@ __global__ __launch_bounds__(NT) void fused_middle_kernel(MiddleArgs a) {
     middle_body<D, NT>(a, blockIdx.x);
 }
 
-// Middle stage, V pass and final sum of one (batch, head) by one workgroup of 16 waves.
-template <int D, bool REF>
-__device__ __forceinline__ void row_tail(const uint8_t *__restrict__ v_first_8, const uint8_t *__restrict__ v_mid_4,
-                                         const uint8_t *__restrict__ v_last_4, const MiddleArgs &ma,
-                                         unsigned short *__restrict__ out, uint8_t *__restrict__ v_levels_out,
-                                         uint8_t *__restrict__ amin_out, float (*wave_part)[D]) {
-    constexpr int NT = 1024, NW = NT / 64;
-    const int wave = threadIdx.x >> 6;
-    const int bh = blockIdx.x;
-    // ---- middle: append, tail scores, softmax, probe, threshold, tail output
-    middle_body<D, NT>(ma, bh);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
-    // ---- V pass: wave w accumulates tokens [w*tpw, (w+1)*tpw)
-    int R, nrest_unused;
-    seq_state(ma.g, bh / ma.g.Hq, R, nrest_unused);
-    const unsigned char amin = REF ? 0 : ma.amin[bh];
-    if (!REF && amin_out != nullptr && threadIdx.x == 0) amin_out[bh] = amin;
-    float acc[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    {
-        // wave w takes the token groups w, w + 16, ... (128 tokens each): neighbouring waves, neighbouring rows
-        constexpr int GT = 2 * (D == 256 ? 32 : 64);
-        const int64_t row0 = (int64_t)bh * ma.g.max_seq_len;
-        v_accumulate_range<D, REF>(v_first_8 + row0 * D, v_mid_4 + row0 * (D / 2), v_last_4 + row0 * (D / 2), R,
-                                   ma.probs + (int64_t)bh * ma.g.row_stride, amin, wave * GT, R, acc,
-                                   v_levels_out != nullptr ? v_levels_out + (int64_t)bh * R : nullptr, NW);
-    }
-    v_fold_lanes<D, NW>(acc, wave_part);
-    __syncthreads();
-    for (int d = threadIdx.x; d < D; d += NT) {
-        float sum = 0.f;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) sum += wave_part[w][d];
-        const float o16 = half_bits_to_float(float_to_half_bits(sum));
-        out[(int64_t)bh * D + d] = float_to_half_bits(o16 + half_bits_to_float(ma.otail[(int64_t)bh * D + d]));
-    }
-}
-
-
-// ------------------------------------------------------------------------------------------------
-// Whole step in one launch: one workgroup of 16 waves per (batch, head) runs the K pass, the middle
-// stage and the V pass back to back.  Used when there are about as many (batch, head) pairs as compute
-// units: nothing is exchanged between workgroups (no partial sums, no second and third launch with
-// their ramp-up and drain), scores and probabilities never leave the compute unit's caches.
-// grid (B*H), 1024 threads.
-// ------------------------------------------------------------------------------------------------
-template <int D, bool REF>
-__global__ __launch_bounds__(1024) void mono_step_kernel(
-    const uint8_t *__restrict__ k_first_8, const uint8_t *__restrict__ k_mid_4, const uint8_t *__restrict__ k_last_4,
-    const uint8_t *__restrict__ v_first_8, const uint8_t *__restrict__ v_mid_4, const uint8_t *__restrict__ v_last_4,
-    MiddleArgs ma, unsigned short *__restrict__ out, uint8_t *__restrict__ k_levels_out,
-    uint8_t *__restrict__ v_levels_out, uint8_t *__restrict__ amin_out, int n_blocks, int n_max_blocks, float scale) {
-    constexpr int CB = 64;
-    constexpr int NG = D / 16;
-    constexpr int NT = 1024, NW = NT / 64;
-    __shared__ float wave_part[NW][D];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int bh = blockIdx.x;
-    // ---- K pass: wave w scores blocks [w*bpw, (w+1)*bpw)
-    {
-        // wave w takes blocks w, w + 16, ...: at any time the 16 waves stream 16 neighbouring blocks
-        const int first_blk = wave;
-        const int end_blk = n_blocks;
-        const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
-        KHalfTile<D / 32> ta;
-        k_prefetch_first<D>(ta, k_first_8 + plane_off * 2, n_blocks, first_blk);
-        float qf[NG];
-        u32 esum[NG];
-        u32 mx = 0;
-#pragma unroll
-        for (int g = 0; g < NG; ++g) {
-            const int c = g * 16 + (lane >> 2);
-            const u32 qb = ma.q[(int64_t)bh * D + c];
-            qf[g] = half_bits_to_float(qb);
-            const u32 cm = max((u32)ma.kcm[(int64_t)bh * D + c], exp_field(ma.k_new[(int64_t)bh * D + c]));
-            esum[g] = (exp_field(qb) + cm) & 0xffu;
-            mx = max(mx, esum[g]);
-        }
-#pragma unroll
-        for (int m = 4; m <= 32; m <<= 1) mx = max(mx, (u32)__shfl_xor((int)mx, m, 64));
-        u32 need_mid = 0, need_last = 0;
-#pragma unroll
-        for (int g = 0; g < NG; ++g) {
-            const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)esum[g]);
-            need_mid |= (lv < 2 ? 1u : 0u) << g;
-            need_last |= (lv == 0 ? 1u : 0u) << g;
-            if (k_levels_out != nullptr && wave == 0 && (lane & 3) == 0)
-                k_levels_out[(int64_t)bh * D + g * 16 + (lane >> 2)] = (uint8_t)lv;
-        }
-        k_score_blocks<D>(ta, k_first_8 + plane_off * 2, k_mid_4 + plane_off, k_last_4 + plane_off, n_blocks, first_blk,
-                          end_blk, qf, need_mid, need_last, ma.scores + (int64_t)bh * ma.g.row_stride, scale, NW);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __syncthreads();
-    row_tail<D, REF>(v_first_8, v_mid_4, v_last_4, ma, out, v_levels_out, amin_out, wave_part);
-}
-
 // Second half of a step in one launch: the middle stage, the V pass and the final sum for one (batch, head) per
 // workgroup of 8 waves, after a K pass that ran as a launch of its own.  With about as many (batch, head) pairs as
 // compute units (or a multiple of them) every unit streams one row of V planes from start to end: no partial sums,
@@ -1075,28 +976,6 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     ma.kcm = kcm; ma.vcm = vcm; ma.toe = toe; ma.amin = amin; ma.v_first_8 = vf8;
     ma.g = geo; ma.mask_stride = mask_stride; ma.top_k = top_k; ma.persist = persist;
     mark(0, st);
-    // One launch for the whole step: opt-in (AKV_TUNE_MONO=1), multi-head uniform-length caches only.  It
-    // measures level with the four launches at batch 8 x 32 heads x 4096 tokens on MI355X.
-    bool mono = false;
-    { AKV_TUNE("AKV_TUNE_MONO", v); if (has_v) mono = v != 0; }
-    mono = mono && n_blocks >= 1 && geo.G == 1 && !ragged && kb == 64 && !(literal_broadcast && !ref);
-    if (mono) {
-        if (ref)
-            hipLaunchKernelGGL((mono_step_kernel<D, true>), dim3(B * Hq), dim3(1024), 0, st, kf8, km4, kl4, vf8, vm4, vl4,
-                               ma, reinterpret_cast<unsigned short *>(out), k_levels_out, v_levels_out, amin_out,
-                               n_blocks, n_max_blocks, scale);
-        else
-            hipLaunchKernelGGL((mono_step_kernel<D, false>), dim3(B * Hq), dim3(1024), 0, st, kf8, km4, kl4, vf8, vm4, vl4,
-                               ma, reinterpret_cast<unsigned short *>(out), k_levels_out, v_levels_out, amin_out,
-                               n_blocks, n_max_blocks, scale);
-        mark(1, st);
-        mark(2, st);
-        mark(3, st);
-        mark(4, st);
-        mark(5, st);
-        mark(6, st);
-        return check_launch("decode_step(mono)");
-    }
     if (n_blocks > 0 && matrix) {
         int rc = AKV_OK;
         if constexpr (D <= 128)
