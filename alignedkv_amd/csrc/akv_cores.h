@@ -539,6 +539,107 @@ __device__ __forceinline__ void v_stream_run(VRing<D, NR> &ring, const uint8_t *
     }
 }
 
+// The same with the rare tokens below level 2 taken out of the loop.  Every half tile is multiplied at level 2 (high
+// bytes only: no nibble loads, no branch on the levels and no wait for them in the pipeline); a lane whose token is
+// below level 2 appends (token, probability) to the wave's list in LDS, and after the loop the wave walks the list,
+// TPL tokens at a time, and adds p * (value at the token's level - value at level 2).  Both values are fp16 numbers,
+// so the result differs from multiplying the token at its level only by fp32 rounding.  With ~1 % of the tokens below
+// level 2, 25-80 % of the 32-token half tiles hold one; taking those half tiles' nibble rows inside the loop held the
+// wave up by about 0.7 us each (measured), which left the rows of a step up to 8 us apart.
+// list: LDS, room for every token of the wave (n_per_wave * HT entries).
+template <int D, int NR, int PF>
+__device__ __forceinline__ void v_stream_run_deferred(VRing<D, NR> &ring, const uint8_t *f8, const uint8_t *m4,
+                                                      const uint8_t *l4, int n_tokens, const unsigned short *s_row,
+                                                      unsigned char amin, const VSeq &seq, float *acc, u32 *list) {
+    using S = VStream<D>;
+    static_assert(NR >= 2, "one slot is multiplied while the others travel");
+    constexpr int HV = S::HV;
+    const int lane = threadIdx.x & 63, tl = lane / S::LPR, cl = lane % S::LPR;
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_tokens * (D / 2));
+    const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_tokens * (D / 2));
+    const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)n_tokens * 2);
+#pragma unroll
+    for (int k = PF; k < NR - 1; ++k) v_stream_issue_high<D>(ring.hi[k], rH, seq.half(k));
+#pragma unroll
+    for (int k = 0; k < NR - 1; ++k) v_stream_issue_probs<D>(ring.sb[k], rS, seq.half(k));
+    __builtin_amdgcn_sched_barrier(0);
+    int count = 0;   // entries in the list (wave-uniform)
+    auto round = [&](int i0) {
+#pragma unroll
+        for (int k = 0; k < NR; ++k) {
+            v_stream_issue<D, NR>(ring, (k + NR - 1) % NR, rH, rS, seq.half(i0 + k + NR - 1));
+            __builtin_amdgcn_sched_barrier(0);
+            // tokens of this half tile below level 2 (one lane per token notes it: the first of its row)
+            bool fine[HV];
+            bool any = false;
+#pragma unroll
+            for (int u = 0; u < HV; ++u) {
+                fine[u] = cl == 0 && v_level(amin, (unsigned short)ring.sb[k][u]) < 2 && ring.sb[k][u] != 0u;
+                any = any || fine[u];
+            }
+            if (__builtin_amdgcn_ballot_w64(any) != 0ull) {
+                const int base = seq.half(i0 + k) * S::HT + tl;
+#pragma unroll
+                for (int u = 0; u < HV; ++u) {
+                    const unsigned long long m = __builtin_amdgcn_ballot_w64(fine[u]);
+                    const int before = (int)__builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u));
+                    if (fine[u]) list[count + before] = (u32)(base + u * S::TPL) | (ring.sb[k][u] << 16);
+                    count += __builtin_popcountll(m);
+                }
+            }
+            v_compute_half_coarse<HV>(acc, ring.hi[k], ring.sb[k]);
+            pin_accumulators(acc);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    if (seq.n_per_wave > 0) {
+        round(0);
+        for (int i0 = NR; i0 < seq.n_per_wave; i0 += NR) round(i0);
+    }
+    // the listed tokens, TPL per step (lane group tl takes entry e0 + tl), one step requested ahead
+    struct Step {
+        u32x4 h;
+        u32x2 m, l;
+        u32 cm, cl;
+        float p;
+    };
+    auto request = [&](Step &st, int e0) {
+        const int e = e0 + tl;
+        const bool on = e < count;
+        const u32 entry = on ? list[e] : 0u;
+        const int tok = (int)(entry & 0xffffu);
+        const u32 pb = entry >> 16;
+        const int level = v_level(amin, (unsigned short)pb);
+        st.h = __builtin_amdgcn_raw_buffer_load_b128(rH, on ? tok * D + cl * 16 : kSkip, 0, kStream);
+        st.m = __builtin_amdgcn_raw_buffer_load_b64(rM, (on && level < 2) ? tok * (D / 2) + cl * 8 : kSkip, 0, kStream);
+        st.l = __builtin_amdgcn_raw_buffer_load_b64(rL, (on && level == 0) ? tok * (D / 2) + cl * 8 : kSkip, 0, kStream);
+        st.cm = level == 2 ? 0x88888888u : 0u;
+        st.cl = level == 1 ? 0x88888888u : 0u;
+        st.p = on ? half_bits_to_float(pb) : 0.f;
+    };
+    auto apply = [&](const Step &st) {
+        fma8(acc, st.h.x, st.h.y, st.m.x | st.cm, st.l.x | st.cl, st.p);
+        fma8(acc + 8, st.h.z, st.h.w, st.m.y | st.cm, st.l.y | st.cl, st.p);
+        fma8_even_odd(acc, st.h.x, st.h.y, 0x80808080u, 0x80808080u, -st.p);
+        fma8_even_odd(acc + 8, st.h.z, st.h.w, 0x80808080u, 0x80808080u, -st.p);
+    };
+    if (count > 0) {
+        Step a, b;
+        request(a, 0);
+        for (int e0 = 0; e0 < count; e0 += 2 * S::TPL) {
+            request(b, e0 + S::TPL);
+            __builtin_amdgcn_sched_barrier(0);
+            apply(a);
+            __builtin_amdgcn_sched_barrier(0);
+            request(a, e0 + 2 * S::TPL);
+            __builtin_amdgcn_sched_barrier(0);
+            apply(b);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+}
+
 // Folds the token lanes of a wave together and adds the 4 waves of the workgroup:
 // out[d] (d < D) = sum over all 256 lanes of their acc for channel d.  wave_part: LDS [4][D].
 template <int D, int NW = 4>

@@ -715,19 +715,21 @@ __global__ __launch_bounds__(NT) void fused_middle_kernel(MiddleArgs a) {
     middle_body<D, NT>(a, blockIdx.x);
 }
 
+constexpr int tail_rows_per_cu = 2, tail_max_tokens = 8192;
+
 // Second half of a step in one launch: the middle stage, the V pass and the final sum for one (batch, head) per
 // workgroup of 8 waves, after a K pass that ran as a launch of its own.  With about as many (batch, head) pairs as
 // compute units (or a multiple of them) every unit streams one row of V planes from start to end: no partial sums,
 // no combine launch, and the first high-byte tiles of every wave travel while the middle stage runs.
 // grid (B*H), 512 threads.
-template <int D, bool REF, int NR, int PF>
-__global__ __launch_bounds__(512) void tail_step_kernel(const uint8_t *__restrict__ v_first_8,
+template <int D, bool REF, int NR, int PF, int NT>
+__global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict__ v_first_8,
                                                         const uint8_t *__restrict__ v_mid_4,
                                                         const uint8_t *__restrict__ v_last_4, MiddleArgs ma,
                                                         unsigned short *__restrict__ out,
                                                         uint8_t *__restrict__ v_levels_out,
                                                         uint8_t *__restrict__ amin_out) {
-    constexpr int NT = 512, NW = NT / 64;
+    constexpr int NW = NT / 64;
     __shared__ float wave_part[NW][D];
     __shared__ u32 row_amin;
     const int wave = threadIdx.x >> 6;
@@ -751,7 +753,13 @@ __global__ __launch_bounds__(512) void tail_step_kernel(const uint8_t *__restric
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
     const unsigned short *prow = ma.probs + (int64_t)bh * ma.g.row_stride;
-    v_stream_run<D, REF, NR, PF>(ring, f8, m4, l4, R, prow, amin, seq, acc);
+    if constexpr (REF) {
+        v_stream_run<D, REF, NR, PF>(ring, f8, m4, l4, R, prow, amin, seq, acc);
+    } else {
+        // (a row has at most tail_max_tokens flushed tokens: tail_max_tokens / NW per wave)
+        __shared__ u32 fine_list[NW][tail_max_tokens / NW];
+        v_stream_run_deferred<D, NR, PF>(ring, f8, m4, l4, R, prow, amin, seq, acc, fine_list[wave]);
+    }
     if (v_levels_out != nullptr)
         for (int t = threadIdx.x; t < R; t += NT) v_levels_out[(int64_t)bh * R + t] = (uint8_t)(REF ? 0 : v_level(amin, prow[t]));
     v_fold_lanes<D, NW>(acc, wave_part);
@@ -863,8 +871,6 @@ static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
     l.total = l.v_chunks + up((size_t)B * sizeof(int));
     return l;
 }
-
-constexpr int tail_rows_per_cu = 2, tail_max_tokens = 8192;
 
 template <int D>
 static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint8_t *vm4, uint8_t *vl4, uint8_t *kcm,
@@ -1016,15 +1022,17 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     // 16 x 4096; level at 32 x 4096 and behind at 8 x 16384 (one workgroup per unit streams at 4.5 TB/s, the V pass
     // of many small workgroups at 6).
     const int cus = compute_units();
-    bool tail = cus > 0 && (B * Hq) % cus == 0 && (B * Hq) / cus <= tail_rows_per_cu && R <= tail_max_tokens;
+    bool tail = cus > 0 && (B * Hq) % cus == 0 && (B * Hq) / cus <= tail_rows_per_cu;
     { AKV_TUNE("AKV_TUNE_TAIL", v); if (has_v) tail = v != 0; }
-    tail = tail && n_blocks >= 1 && geo.G == 1 && !ragged && !(literal_broadcast && !ref);
+    tail = tail && n_blocks >= 1 && R <= tail_max_tokens && geo.G == 1 && !ragged && !(literal_broadcast && !ref);
     if (tail) {
+        // ring depth 2 (one half tile per wave in flight besides the one being multiplied): measured faster than 3, 4,
+        // 6 and 8 (29.9 / 30.9 / 30.3 / 32.1 / 32.1 us); 16 waves per workgroup measured 1 us slower than 8
         if (ref)
-            hipLaunchKernelGGL((tail_step_kernel<D, true, 4, 3>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
+            hipLaunchKernelGGL((tail_step_kernel<D, true, 4, 3, 512>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
                                reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out);
         else
-            hipLaunchKernelGGL((tail_step_kernel<D, false, 4, 3>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
+            hipLaunchKernelGGL((tail_step_kernel<D, false, 2, 1, 512>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
                                reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out);
         mark(2, st);
         mark(3, st);
