@@ -357,6 +357,73 @@ __device__ __forceinline__ bool v_half_is_fine(const u32 *sb, unsigned char amin
     return __builtin_amdgcn_ballot_w64(any) != 0ull;
 }
 
+// ---- tokens below level 2, taken out of the streaming loops -----------------------------------------
+// With ~1 % of the tokens below level 2, 25-80 % of the 32-token half tiles hold one; fetching those half tiles' nibble
+// rows inside the pipeline holds a wave up by about 0.7 us each (measured).  The loops therefore multiply every token
+// at level 2 (high bytes only); a lane whose token is below level 2 appends (token, probability) to the wave's list in
+// LDS, and the wave then adds p * (value at the token's level - value at level 2) for the listed tokens, TPL at a
+// time.  Both values are fp16 numbers, so the result differs from multiplying the token at its level only by fp32
+// rounding.
+template <int D>
+struct VListed {
+    static constexpr int LPR = D / 16, TPL = 64 / LPR;
+    struct Step {
+        u32x4 h;
+        u32x2 m, l;
+        u32 cm, cl;
+        float p;
+    };
+    // Appends the lanes' tokens flagged `fine` (one lane per token: the first of its row) to list[count...].
+    static __device__ __forceinline__ void append(u32 *list, int &count, bool fine, int tok, u32 prob_bits) {
+        const unsigned long long m = __builtin_amdgcn_ballot_w64(fine);
+        if (m == 0ull) return;
+        const int before = (int)__builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u));
+        if (fine) list[count + before] = (u32)tok | (prob_bits << 16);
+        count += __builtin_popcountll(m);
+    }
+    // lane group tl takes entry e0 + tl; an entry holds its token relative to tok_base in 16 bits
+    static __device__ __forceinline__ void request(Step &st, const u32 *list, int count, int e0, const __amdgpu_buffer_rsrc_t rH,
+                                                   const __amdgpu_buffer_rsrc_t rM, const __amdgpu_buffer_rsrc_t rL,
+                                                   unsigned char amin, int tok_base) {
+        const int lane = threadIdx.x & 63, tl = lane / LPR, cl = lane % LPR;
+        const int e = e0 + tl;
+        const bool on = e < count;
+        const u32 entry = on ? list[e] : 0u;
+        const int tok = tok_base + (int)(entry & 0xffffu);
+        const u32 pb = entry >> 16;
+        const int level = v_level(amin, (unsigned short)pb);
+        st.h = __builtin_amdgcn_raw_buffer_load_b128(rH, on ? tok * D + cl * 16 : kSkip, 0, kStream);
+        st.m = __builtin_amdgcn_raw_buffer_load_b64(rM, (on && level < 2) ? tok * (D / 2) + cl * 8 : kSkip, 0, kStream);
+        st.l = __builtin_amdgcn_raw_buffer_load_b64(rL, (on && level == 0) ? tok * (D / 2) + cl * 8 : kSkip, 0, kStream);
+        st.cm = level == 2 ? 0x88888888u : 0u;
+        st.cl = level == 1 ? 0x88888888u : 0u;
+        st.p = on ? half_bits_to_float(pb) : 0.f;
+    }
+    static __device__ __forceinline__ void apply(float *acc, const Step &st) {
+        fma8(acc, st.h.x, st.h.y, st.m.x | st.cm, st.l.x | st.cl, st.p);
+        fma8(acc + 8, st.h.z, st.h.w, st.m.y | st.cm, st.l.y | st.cl, st.p);
+        fma8_even_odd(acc, st.h.x, st.h.y, 0x80808080u, 0x80808080u, -st.p);
+        fma8_even_odd(acc + 8, st.h.z, st.h.w, 0x80808080u, 0x80808080u, -st.p);
+    }
+    // the whole list; `first` holds the entries 0 .. TPL - 1, requested by the caller earlier
+    static __device__ __forceinline__ void apply_all(float *acc, Step &first, const u32 *list, int count,
+                                                     const __amdgpu_buffer_rsrc_t rH, const __amdgpu_buffer_rsrc_t rM,
+                                                     const __amdgpu_buffer_rsrc_t rL, unsigned char amin, int tok_base) {
+        if (count <= 0) return;
+        Step other;
+        for (int e0 = 0; e0 < count; e0 += 2 * TPL) {
+            request(other, list, count, e0 + TPL, rH, rM, rL, amin, tok_base);
+            __builtin_amdgcn_sched_barrier(0);
+            apply(acc, first);
+            __builtin_amdgcn_sched_barrier(0);
+            request(first, list, count, e0 + 2 * TPL, rH, rM, rL, amin, tok_base);
+            __builtin_amdgcn_sched_barrier(0);
+            apply(acc, other);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+};
+
 template <int D, bool REF, int NIT>
 __device__ __forceinline__ void v_accumulate(VFirstTile<D> &ft, const uint8_t *f8, const uint8_t *m4, const uint8_t *l4,
                                              int n_tokens, const unsigned short *s_row, unsigned char amin, int t_begin,
@@ -444,7 +511,11 @@ struct VRing {
 // neighbouring rows).  Past the wave's share: n_halves (nothing is fetched).
 struct VSeq {
     int wave, n_waves, n_per_wave, n_halves;
-    __device__ __forceinline__ int half(int i) const { return i < n_per_wave ? i * n_waves + wave : n_halves; }
+    int first = 0;   // the wave's share starts at its first-th half tile (a caller that has done the ones before)
+    __device__ __forceinline__ int half(int i) const {
+        return i + first < n_per_wave ? (i + first) * n_waves + wave : n_halves;
+    }
+    __device__ __forceinline__ int left() const { return n_per_wave - first; }
 };
 
 // High bytes of half tile `half`: one address per lane, the HV rows at constant distances from it.  A half tile past the
@@ -471,8 +542,8 @@ __device__ __forceinline__ void v_stream_issue_probs(u32 *sb, const __amdgpu_buf
 }
 
 // requests half tile `half` (tokens half * HT ...) into ring slot k
-template <int D, int NR>
-__device__ __forceinline__ void v_stream_issue(VRing<D, NR> &ring, int k, const __amdgpu_buffer_rsrc_t rH,
+template <int D, int NRING>
+__device__ __forceinline__ void v_stream_issue(VRing<D, NRING> &ring, int k, const __amdgpu_buffer_rsrc_t rH,
                                                const __amdgpu_buffer_rsrc_t rS, int half) {
     // the probabilities first: loads return in order, and the fetch levels of a half tile are looked at one half
     // tile before its high bytes are needed
@@ -533,42 +604,71 @@ __device__ __forceinline__ void v_stream_run(VRing<D, NR> &ring, const uint8_t *
     // The first round stands outside the loop: the compiler derives the number of loads that may stay in flight at
     // a wait from every path that reaches it, and the path from the set-up above (fewer requests behind the one
     // waited for) would otherwise hold every round of the loop to the depth of the first.
-    if (seq.n_per_wave > 0) {
+    if (seq.left() > 0) {
         round(0);
-        for (int i0 = NR; i0 < seq.n_per_wave; i0 += NR) round(i0);
+        for (int i0 = NR; i0 < seq.left(); i0 += NR) round(i0);
     }
 }
 
-// The same with the rare tokens below level 2 taken out of the loop.  Every half tile is multiplied at level 2 (high
-// bytes only: no nibble loads, no branch on the levels and no wait for them in the pipeline); a lane whose token is
-// below level 2 appends (token, probability) to the wave's list in LDS, and after the loop the wave walks the list,
-// TPL tokens at a time, and adds p * (value at the token's level - value at level 2).  Both values are fp16 numbers,
-// so the result differs from multiplying the token at its level only by fp32 rounding.  With ~1 % of the tokens below
-// level 2, 25-80 % of the 32-token half tiles hold one; taking those half tiles' nibble rows inside the loop held the
-// wave up by about 0.7 us each (measured), which left the rows of a step up to 8 us apart.
-// list: LDS, room for every token of the wave (n_per_wave * HT entries).
-template <int D, int NR, int PF>
-__device__ __forceinline__ void v_stream_run_deferred(VRing<D, NR> &ring, const uint8_t *f8, const uint8_t *m4,
-                                                      const uint8_t *l4, int n_tokens, const unsigned short *s_row,
-                                                      unsigned char amin, const VSeq &seq, float *acc, u32 *list) {
+// Number of the wave's tokens below level 2: the probabilities of the wave's half tiles, 16 bytes per lane and load;
+// for rows of at most 64 * 16 * 8 / 2 tokens per wave.
+template <int D>
+__device__ __forceinline__ int v_stream_count_fine(const unsigned short *s_row, int n_tokens, unsigned char amin, const VSeq &seq) {
     using S = VStream<D>;
-    static_assert(NR >= 2, "one slot is multiplied while the others travel");
+    constexpr int UPH = S::HT * 2 / 16;    // 16-byte units of probabilities per half tile
+    const int lane = threadIdx.x & 63;
+    const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)n_tokens * 2);
+    typedef short i16x2_t __attribute__((ext_vector_type(2)));
+    typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+    const unsigned short a16 = (unsigned short)((unsigned)amin << 10);
+    const u16x2_t a2 = {a16, a16};
+    const i16x2_t c8 = {0x0800, 0x0800};
+    int n = 0;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int f = lane + 64 * j, i = f / UPH, part = f % UPH;
+        const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(rS, (seq.half(i) * S::HT + part * 8) * 2, 0, 0);
+        const u32 ww[4] = {w.x, w.y, w.z, w.w};
+        const bool on = seq.half(i) < seq.n_halves;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            union { u32 u; u16x2_t v; } x;
+            x.u = ww[k];
+            union { u16x2_t u; i16x2_t s; } d;
+            d.u = a2 - x.v;                                    // wraps like the reference's `short` arithmetic
+            union { i16x2_t v; u32 u; } t;
+            t.v = __builtin_elementwise_sub_sat(d.s, c8);      // negative <=> diff < 0x0800 <=> level < 2
+            n += on ? __builtin_popcount((t.u >> 15) & 0x00010001u) : 0;
+        }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) n += __shfl_xor(n, m, 64);
+    return n;
+}
+
+// The same with the tokens below level 2 taken out of the loop (VListed); the caller adds the listed tokens at the end
+// (v_stream_apply_list).  For rows where they are rare: a listed token costs a second fetch of its high bytes and a
+// share of a memory round trip of its own (at one token in nine the pass takes 52 instead of 30 us).
+// list: LDS, room for every token of the wave (n_per_wave * HT entries); count: its length.
+template <int D, int NR, int PF, int NRING>
+__device__ __forceinline__ void v_stream_run_deferred(VRing<D, NRING> &ring, const uint8_t *f8, int n_tokens,
+                                                     const unsigned short *s_row, unsigned char amin, const VSeq &seq,
+                                                     float *acc, u32 *list, int &count) {
+    using S = VStream<D>;
+    static_assert(NR >= 2 && NR <= NRING, "one slot is multiplied while the others travel");
     constexpr int HV = S::HV;
     const int lane = threadIdx.x & 63, tl = lane / S::LPR, cl = lane % S::LPR;
     const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
-    const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_tokens * (D / 2));
-    const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_tokens * (D / 2));
     const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)n_tokens * 2);
 #pragma unroll
     for (int k = PF; k < NR - 1; ++k) v_stream_issue_high<D>(ring.hi[k], rH, seq.half(k));
 #pragma unroll
     for (int k = 0; k < NR - 1; ++k) v_stream_issue_probs<D>(ring.sb[k], rS, seq.half(k));
     __builtin_amdgcn_sched_barrier(0);
-    int count = 0;   // entries in the list (wave-uniform)
     auto round = [&](int i0) {
 #pragma unroll
         for (int k = 0; k < NR; ++k) {
-            v_stream_issue<D, NR>(ring, (k + NR - 1) % NR, rH, rS, seq.half(i0 + k + NR - 1));
+            v_stream_issue<D, NRING>(ring, (k + NR - 1) % NR, rH, rS, seq.half(i0 + k + NR - 1));
             __builtin_amdgcn_sched_barrier(0);
             // tokens of this half tile below level 2 (one lane per token notes it: the first of its row)
             bool fine[HV];
@@ -581,63 +681,28 @@ __device__ __forceinline__ void v_stream_run_deferred(VRing<D, NR> &ring, const 
             if (__builtin_amdgcn_ballot_w64(any) != 0ull) {
                 const int base = seq.half(i0 + k) * S::HT + tl;
 #pragma unroll
-                for (int u = 0; u < HV; ++u) {
-                    const unsigned long long m = __builtin_amdgcn_ballot_w64(fine[u]);
-                    const int before = (int)__builtin_amdgcn_mbcnt_hi((u32)(m >> 32), __builtin_amdgcn_mbcnt_lo((u32)m, 0u));
-                    if (fine[u]) list[count + before] = (u32)(base + u * S::TPL) | (ring.sb[k][u] << 16);
-                    count += __builtin_popcountll(m);
-                }
+                for (int u = 0; u < HV; ++u) VListed<D>::append(list, count, fine[u], base + u * S::TPL, ring.sb[k][u]);
             }
             v_compute_half_coarse<HV>(acc, ring.hi[k], ring.sb[k]);
             pin_accumulators(acc);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
-    if (seq.n_per_wave > 0) {
+    if (seq.left() > 0) {
         round(0);
-        for (int i0 = NR; i0 < seq.n_per_wave; i0 += NR) round(i0);
+        for (int i0 = NR; i0 < seq.left(); i0 += NR) round(i0);
     }
-    // the listed tokens, TPL per step (lane group tl takes entry e0 + tl), one step requested ahead
-    struct Step {
-        u32x4 h;
-        u32x2 m, l;
-        u32 cm, cl;
-        float p;
-    };
-    auto request = [&](Step &st, int e0) {
-        const int e = e0 + tl;
-        const bool on = e < count;
-        const u32 entry = on ? list[e] : 0u;
-        const int tok = (int)(entry & 0xffffu);
-        const u32 pb = entry >> 16;
-        const int level = v_level(amin, (unsigned short)pb);
-        st.h = __builtin_amdgcn_raw_buffer_load_b128(rH, on ? tok * D + cl * 16 : kSkip, 0, kStream);
-        st.m = __builtin_amdgcn_raw_buffer_load_b64(rM, (on && level < 2) ? tok * (D / 2) + cl * 8 : kSkip, 0, kStream);
-        st.l = __builtin_amdgcn_raw_buffer_load_b64(rL, (on && level == 0) ? tok * (D / 2) + cl * 8 : kSkip, 0, kStream);
-        st.cm = level == 2 ? 0x88888888u : 0u;
-        st.cl = level == 1 ? 0x88888888u : 0u;
-        st.p = on ? half_bits_to_float(pb) : 0.f;
-    };
-    auto apply = [&](const Step &st) {
-        fma8(acc, st.h.x, st.h.y, st.m.x | st.cm, st.l.x | st.cl, st.p);
-        fma8(acc + 8, st.h.z, st.h.w, st.m.y | st.cm, st.l.y | st.cl, st.p);
-        fma8_even_odd(acc, st.h.x, st.h.y, 0x80808080u, 0x80808080u, -st.p);
-        fma8_even_odd(acc + 8, st.h.z, st.h.w, 0x80808080u, 0x80808080u, -st.p);
-    };
-    if (count > 0) {
-        Step a, b;
-        request(a, 0);
-        for (int e0 = 0; e0 < count; e0 += 2 * S::TPL) {
-            request(b, e0 + S::TPL);
-            __builtin_amdgcn_sched_barrier(0);
-            apply(a);
-            __builtin_amdgcn_sched_barrier(0);
-            request(a, e0 + 2 * S::TPL);
-            __builtin_amdgcn_sched_barrier(0);
-            apply(b);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
+}
+
+template <int D>
+__device__ __forceinline__ void v_stream_apply_list(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_tokens,
+                                                    unsigned char amin, float *acc, const u32 *list, int count) {
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_tokens * (D / 2));
+    const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_tokens * (D / 2));
+    typename VListed<D>::Step first;
+    VListed<D>::request(first, list, count, 0, rH, rM, rL, amin, 0);
+    VListed<D>::apply_all(acc, first, list, count, rH, rM, rL, amin, 0);
 }
 
 // Folds the token lanes of a wave together and adds the 4 waves of the workgroup:

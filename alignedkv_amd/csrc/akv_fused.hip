@@ -756,9 +756,19 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     if constexpr (REF) {
         v_stream_run<D, REF, NR, PF>(ring, f8, m4, l4, R, prow, amin, seq, acc);
     } else {
-        // (a row has at most tail_max_tokens flushed tokens: tail_max_tokens / NW per wave)
+        // Few tokens below level 2 (the usual case): they are taken out of the loop, which then keeps one half tile
+        // per wave in flight (measured faster than 2, 3, 5 and 7: 29.9 / 30.9 / 30.3 / 32.1 / 32.1 us at batch 8 x 32
+        // heads x 4096 tokens).  More than one in 16 among the wave's tokens (flat attention): the loop that takes
+        // their nibble rows along with the half tiles, ring of NR.  (A row has at most tail_max_tokens flushed tokens.)
         __shared__ u32 fine_list[NW][tail_max_tokens / NW];
-        v_stream_run_deferred<D, NR, PF>(ring, f8, m4, l4, R, prow, amin, seq, acc, fine_list[wave]);
+        const int n_fine = v_stream_count_fine<D>(prow, R, amin, seq);
+        if (n_fine * 16 <= seq.n_per_wave * VStream<D>::HT) {
+            int count = 0;
+            v_stream_run_deferred<D, 2, PF, NR>(ring, f8, R, prow, amin, seq, acc, fine_list[wave], count);
+            v_stream_apply_list<D>(f8, m4, l4, R, amin, acc, fine_list[wave], count);
+        } else {
+            v_stream_run<D, REF, NR, PF>(ring, f8, m4, l4, R, prow, amin, seq, acc);
+        }
     }
     if (v_levels_out != nullptr)
         for (int t = threadIdx.x; t < R; t += NT) v_levels_out[(int64_t)bh * R + t] = (uint8_t)(REF ? 0 : v_level(amin, prow[t]));
@@ -1026,13 +1036,12 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     { AKV_TUNE("AKV_TUNE_TAIL", v); if (has_v) tail = v != 0; }
     tail = tail && n_blocks >= 1 && R <= tail_max_tokens && geo.G == 1 && !ragged && !(literal_broadcast && !ref);
     if (tail) {
-        // ring depth 2 (one half tile per wave in flight besides the one being multiplied): measured faster than 3, 4,
-        // 6 and 8 (29.9 / 30.9 / 30.3 / 32.1 / 32.1 us); 16 waves per workgroup measured 1 us slower than 8
+        // (16 waves per workgroup measured 1 us slower than 8)
         if (ref)
             hipLaunchKernelGGL((tail_step_kernel<D, true, 4, 3, 512>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
                                reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out);
         else
-            hipLaunchKernelGGL((tail_step_kernel<D, false, 2, 1, 512>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
+            hipLaunchKernelGGL((tail_step_kernel<D, false, 4, 1, 512>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
                                reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out);
         mark(2, st);
         mark(3, st);
