@@ -190,6 +190,45 @@ def test_fused_step_with_mask_and_reference_flag(monkeypatch, tail):
     load_library().akv_reload_tuning()
 
 
+@pytest.mark.parametrize("D,q_scale", [(128, 1.0), (128, 0.0), (128, 0.05), (256, 1.0), (256, 0.05), (64, 0.05)])
+def test_two_launch_step_at_its_longest_row_and_with_flat_attention(monkeypatch, D, q_scale):
+    """8192 flushed tokens (the longest row the two-launch step takes: every wave's list of tokens below level 2 can
+    fill up) and queries scaled towards zero (flat attention: a large share of the tokens is below level 2, the waves
+    take the loop that fetches nibble rows with the half tiles).  Against the four-launch step on the same cache."""
+    from alignedkv_amd import load_library
+    from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
+    B, H, prefill, steps = 1, 4, 8192 - 64, 66
+    _, k, v = make_qkv(B, prefill + steps, H, D, seed=5)
+    q = (q_scale * np.random.default_rng(6).standard_normal((B, steps, H, D))).astype(np.float16)
+    lib = load_library()
+    caches = []
+    for _ in range(2):
+        c = QuantizedCache_AlignedKV(cfg(H, D), B, prefill + steps + 64, "cuda", torch.half, k_block=256 if D <= 128 else 64)
+        c.key_cache[0].save(dev(k[:, :prefill]), 0, prefill)
+        c.value_cache[0].save(dev(v[:, :prefill]), 0, prefill)
+        c.key_cache[0].record_levels = c.value_cache[0].record_levels = True
+        caches.append(c)
+    fine_share = 0.0
+    for s in range(steps):
+        t = prefill + s
+        outs = []
+        for tail, c in zip(("0", "1"), caches):
+            monkeypatch.setenv("AKV_TUNE_TAIL", tail)
+            lib.akv_reload_tuning()
+            outs.append(c.auto_compute(dev(q[:, s:s + 1]), dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None))
+        assert (outs[0].float() - outs[1].float()).abs().max().item() <= 1e-3
+        # the two softmax stages add the row up with 4 and with 8 waves: a probability can differ in its last bit, and
+        # with flat attention many tokens sit next to a level threshold
+        flips = (caches[0].value_cache[0].last_levels != caches[1].value_cache[0].last_levels).float().mean().item()
+        assert flips <= 2e-3
+        assert torch.equal(caches[0].value_cache[0].last_alignment_min, caches[1].value_cache[0].last_alignment_min)
+        fine_share = max(fine_share, (caches[1].value_cache[0].last_levels < 2).float().mean().item())
+    if q_scale < 1.0:
+        assert fine_share > 1 / 16, "the inputs are meant to put the waves on the loop for frequent tokens below level 2"
+    monkeypatch.delenv("AKV_TUNE_TAIL")
+    lib.akv_reload_tuning()
+
+
 def test_step_on_as_many_rows_as_compute_units_matches_the_op_sequence():
     """batch x heads = 256: the shape for which the library itself chooses the two-launch step on a 256-unit part.
     Whatever it chooses, the fused step must agree with the unfused op sequence across a flush."""
