@@ -42,17 +42,24 @@ __device__ __forceinline__ u32 low_bits_excess(u32 w, u32 keep, u32 put) {
     return as_u32(as_f16x2(w) - as_f16x2((w & keep) | put));
 }
 
+// the substitution bits of levels 1 and 2 for a pair of fp16 values, kept in vector registers
+struct LevelPuts {
+    u32 put1 = 0x00080008u, put2 = 0x00800080u;
+    __device__ __forceinline__ void pin() { asm volatile("" : "+v"(put1), "+v"(put2)); }
+};
+
 // acc += A x B0  (+ C1 x B1 + C2 x B2 unless every plane is read)
 template <bool REF>
-__device__ __forceinline__ void mfma_levels(f32x4 &acc, u32 a_lo, u32 a_hi, f16x4 b0, f16x4 b1, f16x4 b2) {
+__device__ __forceinline__ void mfma_levels(f32x4 &acc, u32 a_lo, u32 a_hi, f16x4 b0, f16x4 b1, f16x4 b2, u32 put1,
+                                            u32 put2) {
+    // put1 = 0x00080008, put2 = 0x00800080 in vector registers (LevelPuts): (w & keep) | put is then one v_and_or_b32
+    // (an instruction takes one literal constant)
     acc = __builtin_amdgcn_mfma_f32_16x16x16f16(as_f16x4(a_lo, a_hi), b0, acc, 0, 0, 0);
     if (!REF) {
         acc = __builtin_amdgcn_mfma_f32_16x16x16f16(
-            as_f16x4(low_bits_excess(a_lo, 0xFFF0FFF0u, 0x00080008u), low_bits_excess(a_hi, 0xFFF0FFF0u, 0x00080008u)), b1,
-            acc, 0, 0, 0);
+            as_f16x4(low_bits_excess(a_lo, 0xFFF0FFF0u, put1), low_bits_excess(a_hi, 0xFFF0FFF0u, put1)), b1, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x16f16(
-            as_f16x4(low_bits_excess(a_lo, 0xFF00FF00u, 0x00800080u), low_bits_excess(a_hi, 0xFF00FF00u, 0x00800080u)), b2,
-            acc, 0, 0, 0);
+            as_f16x4(low_bits_excess(a_lo, 0xFF00FF00u, put2), low_bits_excess(a_hi, 0xFF00FF00u, put2)), b2, acc, 0, 0, 0);
     }
 }
 
@@ -111,7 +118,7 @@ __device__ __forceinline__ void kt_issue(KTaskTile<SL> &t, const __amdgpu_buffer
 
 template <bool REF, int SL>
 __device__ __forceinline__ void kt_compute(f32x4 *acc, const KTaskTile<SL> &t, int kg, u32 need_mid, u32 need_last, f16x4 b0,
-                                           f16x4 b1, f16x4 b2) {
+                                           f16x4 b1, f16x4 b2, const LevelPuts &lp) {
     constexpr int NX = (SL + 7) / 8;       // units of 8 slots (one unit of 4 for SL == 4)
     constexpr int NP = SL == 4 ? 2 : 4;    // slot pairs per unit
 #pragma unroll
@@ -141,8 +148,8 @@ __device__ __forceinline__ void kt_compute(f32x4 *acc, const KTaskTile<SL> &t, i
             const u32 a23_s0 = __builtin_amdgcn_perm(w[3][p], w[2][p], 0x05040100u);
             const u32 a01_s2 = __builtin_amdgcn_perm(w[1][p], w[0][p], 0x07060302u);
             const u32 a23_s2 = __builtin_amdgcn_perm(w[3][p], w[2][p], 0x07060302u);
-            mfma_levels<REF>(acc[s0], a01_s0, a23_s0, b0, b1, b2);
-            mfma_levels<REF>(acc[s0 + 2], a01_s2, a23_s2, b0, b1, b2);
+            mfma_levels<REF>(acc[s0], a01_s0, a23_s0, b0, b1, b2, lp.put1, lp.put2);
+            mfma_levels<REF>(acc[s0 + 2], a01_s2, a23_s2, b0, b1, b2, lp.put1, lp.put2);
         }
     }
 }
@@ -291,6 +298,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && 
         lv1 = v.x; lv2 = v.y; need_mid = v.z; need_last = v.w;
     }
 
+    LevelPuts puts;
+    puts.pin();
     // Software pipeline: AHEAD channel-group tiles in flight while one is multiplied.
     KTaskTile<SL> t[AHEAD + 1];
 #pragma unroll
@@ -316,7 +325,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && 
             const u32 m2b = ((lv2 >> (4 * kg + 2)) & 1u ? 0xFFFFu : 0u) | ((lv2 >> (4 * kg + 3)) & 1u ? 0xFFFF0000u : 0u);
             const u32 na = qp[kg][0] ^ 0x80008000u, nb = qp[kg][1] ^ 0x80008000u;     // -q
             kt_compute<REF, SL>(acc, t[kg % (AHEAD + 1)], kg, need_mid, need_last, as_f16x4(qp[kg][0], qp[kg][1]),
-                                as_f16x4(na & m1a, nb & m1b), as_f16x4(na & m2a, nb & m2b));
+                                as_f16x4(na & m1a, nb & m1b), as_f16x4(na & m2a, nb & m2b), puts);
             __builtin_amdgcn_sched_barrier(0);
         }
         // lane (j, ig): acc[s][r] = score of slot s of token set 4 ig + r for query head j
@@ -531,6 +540,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     f32x4 acc[CPP];
 #pragma unroll
     for (int i = 0; i < CPP; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    LevelPuts puts;
+    puts.pin();
 
     u32x2 pn[4], pnn[4];
     VMacroOps oc, on;
@@ -560,7 +571,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
                 const u32 n2a = na & ((l2 & 1u ? 0xFFFFu : 0u) | (l2 & 2u ? 0xFFFF0000u : 0u));
                 const u32 n2b = nb & ((l2 & 4u ? 0xFFFFu : 0u) | (l2 & 8u ? 0xFFFF0000u : 0u));
                 kt_compute<REF, CPP>(acc, t[si], 0, (oc.need >> (4 * si)) & 0xfu, (oc.need >> (16 + 4 * si)) & 0xfu,
-                                     as_f16x4(oc.p[si].x, oc.p[si].y), as_f16x4(n1a, n1b), as_f16x4(n2a, n2b));
+                                     as_f16x4(oc.p[si].x, oc.p[si].y), as_f16x4(n1a, n1b), as_f16x4(n2a, n2b), puts);
             } else {
                 kt_compute_coarse<CPP>(acc, t[si], as_f16x4(oc.p[si].x, oc.p[si].y));
             }
