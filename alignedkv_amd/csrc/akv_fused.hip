@@ -919,6 +919,10 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     const bool grouped = group_heads(geo.G) > 1;
     bool matrix = geo.G >= 2 && geo.G <= 16 && D <= 128;   // (the 32-bit level masks hold 128 channels)
     { AKV_TUNE("AKV_TUNE_MFMA", v); if (has_v) matrix = matrix && v != 0; }
+    if (kb != 64 && geo.G > 1 && !matrix) {
+        set_error("decode_step: grouped-query heads over K plane blocks of %d tokens need the matrix-core K pass", kb);
+        return AKV_ERR_INVALID;
+    }
     const int n_kblocks = (R + kb - 1) / kb;    // K plane blocks that hold tokens (the last one may be partly filled)
     const int bpw = kb == 256 ? k256_blocks_per_wave(B, Hq, n_kblocks) : k_blocks_per_wave(B, Hq, n_blocks);
     bool matrix_v = matrix;
@@ -1167,8 +1171,9 @@ extern "C" int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t
     AKV_REQUIRE(head_dim == 64 || head_dim == 128 || head_dim == 256,
                 "decode_step: head_dim %d not supported by the fused step (64, 128, 256); use the five ops", head_dim);
     AKV_REQUIRE(d_block == 64, "decode_step: d_block %d not supported by the fused step (64); use the five ops", d_block);
-    AKV_REQUIRE(k_block == 64 || (k_block == 256 && n_q_heads == n_kv_heads && head_dim <= 128),
-                "decode_step: k_block %d: K plane blocks are 64 tokens, or 256 for multi-head caches with head_dim 64 or 128", k_block);
+    AKV_REQUIRE(k_block == 64 || (k_block == 256 && head_dim <= 128 && n_q_heads / n_kv_heads <= 16),
+                "decode_step: k_block %d: K plane blocks are 64 tokens, or 256 for head_dim 64 or 128 and at most 16 query "
+                "heads per KV head", k_block);
     AKV_REQUIRE(top_max_k == 32, "decode_step: top_max_k %d not supported by the fused step (32)", top_max_k);
     AKV_REQUIRE(bsz <= 65535 && n_kv_heads <= 65535, "decode_step: bsz/heads exceed the grid limit 65535");
     AKV_REQUIRE(cur_len >= 0 && cur_len + 1 <= max_seq_len, "decode_step: cache full (%d of %d tokens)", cur_len, max_seq_len);

@@ -96,21 +96,25 @@ __device__ __forceinline__ void load_bytes(u32 *dst, const __amdgpu_buffer_rsrc_
     }
 }
 
-template <int D, int SL>
+// KSH: log2 of 64-token blocks per K plane block (0: plane blocks of 64 tokens, 2: of 256).  blk counts 64-token
+// blocks either way; in a 256-token plane block a channel's row holds the slots of four of them side by side.
+template <int D, int SL, int KSH>
 __device__ __forceinline__ void kt_issue(KTaskTile<SL> &t, const __amdgpu_buffer_rsrc_t rH, const __amdgpu_buffer_rsrc_t rM,
                                          const __amdgpu_buffer_rsrc_t rL, int blk, int kg, u32 need_mid, u32 need_last) {
     constexpr int PB = 64 / SL;   // pieces per block
+    constexpr int KB = 64 << KSH;
     const int lane = threadIdx.x & 63;
     const int piece = (lane & 15) % PB, cs = lane >> 4;
+    const int kblk = blk >> KSH, sub = blk & ((1 << KSH) - 1);
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int c = 16 * kg + 4 * r + cs;
-        load_bytes<SL>(t.h[r], rH, blk * (D * 64) + c * 64 + piece * SL);
+        load_bytes<SL>(t.h[r], rH, kblk * (D * KB) + c * KB + sub * 64 + piece * SL);
     }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int c = 16 * kg + 4 * r + cs;
-        const int off = blk * (D * 32) + c * 32 + piece * (SL / 2);
+        const int off = kblk * (D * KB / 2) + c * (KB / 2) + sub * 32 + piece * (SL / 2);
         load_bytes<SL / 2>(t.m[r], rM, ((need_mid >> (4 * kg + r)) & 1u) ? off : kSkip);
         load_bytes<SL / 2>(t.l[r], rL, ((need_last >> (4 * kg + r)) & 1u) ? off : kSkip);
     }
@@ -251,7 +255,7 @@ __device__ __forceinline__ void kt_compute_coarse(f32x4 *acc, const KTaskTile<SL
     }
 }
 
-template <int D, bool REF, int SL, int AHEAD>
+template <int D, bool REF, int SL, int AHEAD, int KSH>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && AHEAD == 3 ? 3 : 1))) void mfma_k_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const u32 *__restrict__ prep, unsigned short *__restrict__ scores, StepGeom geo, int tasks_per_wave, float scale,
@@ -275,10 +279,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && 
     const int end_task = min(first_task + tasks_per_wave, n_tasks);
     if (first_task >= n_tasks) return;     // past the end of this sequence (no barrier in this kernel)
 
-    const int64_t plane_off = (int64_t)bh_kv * geo.n_max_blocks * (D * (CB / 2));
-    const __amdgpu_buffer_rsrc_t rH = make_rsrc(first_8 + plane_off * 2, (u32)n_blocks * (D * CB));
-    const __amdgpu_buffer_rsrc_t rM = make_rsrc(mid_4 + plane_off, (u32)n_blocks * (D * CB / 2));
-    const __amdgpu_buffer_rsrc_t rL = make_rsrc(last_4 + plane_off, (u32)n_blocks * (D * CB / 2));
+    // geo.n_max_blocks counts K plane blocks (of 64 << KSH tokens); the resources end with the last one that holds tokens
+    constexpr int KB = CB << KSH;
+    const int n_kblocks = (n_blocks + (1 << KSH) - 1) >> KSH;
+    const int64_t plane_off = (int64_t)bh_kv * geo.n_max_blocks * (D * (KB / 2));
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(first_8 + plane_off * 2, (u32)n_kblocks * (D * KB));
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(mid_4 + plane_off, (u32)n_kblocks * (D * KB / 2));
+    const __amdgpu_buffer_rsrc_t rL = make_rsrc(last_4 + plane_off, (u32)n_kblocks * (D * KB / 2));
     const __amdgpu_buffer_rsrc_t rS = make_rsrc(scores, scores_bytes);
     const int blk_sel = (lane & 15) / PB;
 
@@ -303,7 +310,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && 
     // Software pipeline: AHEAD channel-group tiles in flight while one is multiplied.
     KTaskTile<SL> t[AHEAD + 1];
 #pragma unroll
-    for (int i = 0; i < AHEAD; ++i) kt_issue<D, SL>(t[i], rH, rM, rL, first_task * NBT + blk_sel, i, need_mid, need_last);
+    for (int i = 0; i < AHEAD; ++i) kt_issue<D, SL, KSH>(t[i], rH, rM, rL, first_task * NBT + blk_sel, i, need_mid, need_last);
     __builtin_amdgcn_sched_barrier(0);
     for (int task = first_task; task < end_task; ++task) {
         f32x4 acc[SL];
@@ -317,7 +324,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && 
 #pragma unroll
         for (int kg = 0; kg < KG; ++kg) {
             const int kn = kg + AHEAD;
-            kt_issue<D, SL>(t[kn % (AHEAD + 1)], rH, rM, rL, kn < KG ? blk : next_blk, kn % KG, need_mid, need_last);
+            kt_issue<D, SL, KSH>(t[kn % (AHEAD + 1)], rH, rM, rL, kn < KG ? blk : next_blk, kn % KG, need_mid, need_last);
             __builtin_amdgcn_sched_barrier(0);
             const u32 m1a = ((lv1 >> (4 * kg)) & 1u ? 0xFFFFu : 0u) | ((lv1 >> (4 * kg + 1)) & 1u ? 0xFFFF0000u : 0u);
             const u32 m1b = ((lv1 >> (4 * kg + 2)) & 1u ? 0xFFFFu : 0u) | ((lv1 >> (4 * kg + 3)) & 1u ? 0xFFFF0000u : 0u);
@@ -360,6 +367,7 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
                        hipStream_t st, PassShape *shape_only) {
     int sl = 8;
     { AKV_TUNE("AKV_TUNE_K_SL", v); if (has_v) sl = v == 16 ? 16 : (v == 4 ? 4 : 8); }
+    if (geo.kb == 256) sl = 8;
     const int nbt = sl / 4;
     const int n_tasks = (n_blocks + nbt - 1) / nbt;
     int tpw = 1;
@@ -381,17 +389,18 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
     int rc = check_launch("decode_step(mfma k_prepare)");
     if (rc != AKV_OK) return rc;
     dim3 grid((n_tasks + 4 * tpw - 1) / (4 * tpw), geo.Hkv, B);
-#define AKV_MK(RF, SLL, AH)                                                                                          \
-    hipLaunchKernelGGL((mfma_k_pass_kernel<D, RF, SLL, AH>), grid, dim3(256), 0, st, f8, m4, l4, prep, scores, geo, tpw, \
-                       scale, (u32)scores_bytes)
+#define AKV_MK(RF, SLL, AH, KSH)                                                                                     \
+    hipLaunchKernelGGL((mfma_k_pass_kernel<D, RF, SLL, AH, KSH>), grid, dim3(256), 0, st, f8, m4, l4, prep, scores, geo, \
+                       tpw, scale, (u32)scores_bytes)
     int ahead = 3;
     { AKV_TUNE("AKV_TUNE_K_AHEAD", v); if (has_v) ahead = v; }
     constexpr int DEEP = (D / 16) % 8 == 0 ? 7 : 3;
-    if (sl == 16) { if (ref) AKV_MK(true, 16, 1); else AKV_MK(false, 16, 1); }
-    else if (sl == 8 && ahead == 7) { if (ref) AKV_MK(true, 8, DEEP); else AKV_MK(false, 8, DEEP); }
-    else if (sl == 8) { if (ref) AKV_MK(true, 8, 3); else AKV_MK(false, 8, 3); }
-    else if (ahead == 7) { if (ref) AKV_MK(true, 4, DEEP); else AKV_MK(false, 4, DEEP); }
-    else { if (ref) AKV_MK(true, 4, 3); else AKV_MK(false, 4, 3); }
+    if (geo.kb == 256) { if (ref) AKV_MK(true, 8, 3, 2); else AKV_MK(false, 8, 3, 2); }   // (the default tile shape only)
+    else if (sl == 16) { if (ref) AKV_MK(true, 16, 1, 0); else AKV_MK(false, 16, 1, 0); }
+    else if (sl == 8 && ahead == 7) { if (ref) AKV_MK(true, 8, DEEP, 0); else AKV_MK(false, 8, DEEP, 0); }
+    else if (sl == 8) { if (ref) AKV_MK(true, 8, 3, 0); else AKV_MK(false, 8, 3, 0); }
+    else if (ahead == 7) { if (ref) AKV_MK(true, 4, DEEP, 0); else AKV_MK(false, 4, DEEP, 0); }
+    else { if (ref) AKV_MK(true, 4, 3, 0); else AKV_MK(false, 4, 3, 0); }
 #undef AKV_MK
     return check_launch("decode_step(mfma k_pass)");
 }

@@ -17,17 +17,21 @@ from ..extension.KV_cache_cpp_extention import cuda_module
 
 class RaggedGQACache:
     def __init__(self, n_layers: int, bsz: int, max_seq_len: int, n_q_heads: int, n_kv_heads: int, head_dim: int,
-                 device="cuda", literal_colmax: bool = True):
-        assert n_q_heads % n_kv_heads == 0
+                 device="cuda", literal_colmax: bool = True, k_block: int = column_block):
+        """k_block: tokens per block of the K planes (64, or 256 for head_dim 64 / 128 and 2 to 16 query heads per KV
+        head: a nibble row of a channel is then a whole 128-byte line)."""
+        assert n_q_heads % n_kv_heads == 0 and k_block in (column_block, 4 * column_block)
         self.n_layers, self.bsz, self.max_seq_len = n_layers, bsz, max_seq_len
         self.n_q_heads, self.n_kv_heads, self.head_dim = n_q_heads, n_kv_heads, head_dim
-        self.n_max_blocks = cdiv(max_seq_len, column_block)
+        self.k_block = k_block
+        self.n_max_blocks = cdiv(max_seq_len, k_block)     # K plane blocks
         self.literal_colmax = literal_colmax
         self.reference = False
         self.record_levels = False
         z = lambda *shape: torch.zeros(shape, dtype=torch.uint8, device=device)
         B, H, D, cb, NB = bsz, n_kv_heads, head_dim, column_block, self.n_max_blocks
-        self.k_planes = [(z(B, H, NB, D, cb), z(B, H, NB, D, cb // 2), z(B, H, NB, D, cb // 2)) for _ in range(n_layers)]
+        self.k_planes = [(z(B, H, NB, D, k_block), z(B, H, NB, D, k_block // 2), z(B, H, NB, D, k_block // 2))
+                         for _ in range(n_layers)]
         self.v_planes = [(z(B, H, max_seq_len, D), z(B, H, max_seq_len, D // 2), z(B, H, max_seq_len, D // 2))
                          for _ in range(n_layers)]
         self.k_colmax = [z(B, 1, H, D) for _ in range(n_layers)]
@@ -36,7 +40,7 @@ class RaggedGQACache:
         self.restv = [torch.zeros((B, cb, H, D), dtype=torch.half, device=device) for _ in range(n_layers)]
         self.seq_lens = [torch.zeros(B, dtype=torch.int32, device=device) for _ in range(n_layers)]
         self.len_bound = [0] * n_layers          # host-side upper bound of seq_lens (sizes the launches)
-        width = (NB + 1) * cb
+        width = (cdiv(max_seq_len, cb) + 1) * cb
         self.scores = torch.empty((B, n_q_heads, width), dtype=torch.half, device=device)
         self.probs = torch.empty((B, n_q_heads, width), dtype=torch.half, device=device)
         self.last_k_levels = self.last_v_levels = self.last_alignment_min = None
@@ -56,7 +60,10 @@ class RaggedGQACache:
         tail = S % cb
         kp = [p[b:b + 1] for p in self.k_planes[layer]]
         vp = [p[b:b + 1] for p in self.v_planes[layer]]
-        cuda_module.k_cache_save(*kp, k.view(torch.uint8), 1, H, S // cb, self.n_max_blocks, D, cb, 0, S)
+        if S - tail:
+            # whole 64-token tiles; with 256-token blocks the last block may be partly filled
+            cuda_module.k_cache_save(*kp, k[:, :S - tail].contiguous().view(torch.uint8), 1, H, cdiv(S - tail, self.k_block),
+                                     self.n_max_blocks, D, self.k_block, 0, S - tail)
         cuda_module.v_cache_save(*vp, v.view(torch.uint8), 1, H, self.max_seq_len, D, 0, S - tail)
         self.k_colmax[layer][b:b + 1] = self._colmax(k)
         self.v_colmax[layer][b:b + 1] = self._colmax(v)
@@ -87,7 +94,8 @@ class RaggedGQACache:
                                     q.view(torch.uint8), k.view(torch.uint8), v.view(torch.uint8), mask2d,
                                     out.view(torch.uint8), self.scores.view(torch.uint8), self.probs.view(torch.uint8),
                                     B, Hq, Hkv, self.n_max_blocks, self.max_seq_len, D, column_block, 32, bound,
-                                    self.seq_lens[layer], self.reference, klv, vlv if flushed else None, amin)
+                                    self.seq_lens[layer], self.reference, klv, vlv if flushed else None, amin,
+                                    k_block=self.k_block)
         if not fixed_bound:
             self.len_bound[layer] = bound + 1
         self.last_k_levels, self.last_v_levels, self.last_alignment_min = klv, vlv, amin

@@ -44,9 +44,10 @@ def parse():
     ap.add_argument("--cache-len", type=int, default=4096)
     ap.add_argument("--layers", type=int, default=4, help="caches the steps rotate over")
     ap.add_argument("--k-kind", default="outlier", choices=["outlier", "lognormal"])
-    ap.add_argument("--k-block", type=int, default=256, choices=[64, 256],
+    ap.add_argument("--k-block", type=int, default=None, choices=[64, 256],
                     help="tokens per block of the K planes (the ops' d_block): 256 = a nibble row is a whole 128-byte line, "
-                         "64 = the block length the reference's Python classes use")
+                         "64 = the block length the reference's Python classes use.  Default: 256 for c2, 64 for c3 (with "
+                         "grouped heads nearly every row is fetched anyway and 64-token blocks measure 9 us faster)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=10)
     ap.add_argument("--seed", type=int, default=0)
@@ -57,7 +58,10 @@ def parse():
     ap.add_argument("--c3-len", type=int, default=0, help="c3 only: one length for every sequence instead of U[2048, 8192]")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB copy kernel (known size, for scaling hardware byte counters)")
-    return ap.parse_args()
+    a = ap.parse_args()
+    if a.k_block is None:
+        a.k_block = 256 if a.workload == "c2" else 64
+    return a
 
 
 def make_layer_inputs(torch, B, L, H, D, seed, k_kind):
@@ -236,7 +240,7 @@ def bench_c3(a):
     lens = np.random.default_rng(a.seed + 3).integers(2048, 8193, B)
     if a.c3_len:
         lens[:] = a.c3_len
-    cache = RaggedGQACache(a.layers, B, Lmax, Hq, Hkv, D)
+    cache = RaggedGQACache(a.layers, B, Lmax, Hq, Hkv, D, k_block=a.k_block)
     for layer in range(a.layers):
         for b in range(B):
             k, v = make_layer_inputs(torch, 1, int(lens[b]), Hkv, D, a.seed + 100 * layer + b, "outlier")
@@ -304,7 +308,7 @@ def bench_c3(a):
            "ms_per_step": round(sec * 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
            "dtype": "f32", "data": "synthetic",
            "config": {"workload": "C3: batch 32, 32 query heads over 8 KV heads x 128, %d cached tokens in total, "
-                                  "%d layers rotated" % (int(lens.sum()), a.layers)},
+                                  "%d layers rotated, K plane blocks of %d tokens" % (int(lens.sum()), a.layers, a.k_block)},
            "kv_plane_bytes_union_of_group_levels": int(kv_bytes), "dense_fp16_bytes": int(dense),
            "bytes_vs_dense": round(kv_bytes / dense, 4),
            "effective_hbm_gbps": round(kv_bytes / sec / 1e9, 1), "pct_hbm_peak": round(100 * kv_bytes / sec / 1e9 / HBM_PEAK_GBPS, 1),

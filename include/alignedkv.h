@@ -168,8 +168,8 @@ AKV_API int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_las
  * then an upper bound of them (it sizes the launches), a sequence flushes its rest buffer on the step that
  * fills it, and the step increments every entry of seq_lens on the device.
  * k_block: tokens per block of the K planes, [bsz, n_kv_heads, n_max_blocks, head_dim, k_block] (the d_block of
- * akv_k_cache_save / akv_k_cache_compute).  64 is the reference's layout.  256 (multi-head, head_dim 64 or 128)
- * makes a channel's nibble row a whole 128-byte line, so a skipped row saves exactly its bytes in HBM traffic;
+ * akv_k_cache_save / akv_k_cache_compute).  64 is the reference's layout.  256 (head_dim 64 or 128; multi-head, or 2 to
+ * 16 query heads per KV head) makes a channel's nibble row a whole 128-byte line, so a skipped row saves exactly its bytes in HBM traffic;
  * tokens still enter the planes 64 at a time (d_block, the length of the rest buffers), as whole tiles inside a block.
  */
 AKV_API int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,

@@ -18,19 +18,24 @@ def dev(a):
                                                    (4, 16, 2, [63, 127, 128, 1], 66, 128), (2, 8, 1, [300, 190], 5, 128),
                                                    (2, 8, 2, [500, 321], 4, 64), (2, 12, 4, [260, 700], 3, 64),
                                                    (2, 8, 2, [450, 130], 4, 256), (1, 6, 2, [1100], 2, 128),
-                                                   (2, 40, 2, [200, 330], 2, 128)])
+                                                   (2, 40, 2, [200, 330], 2, 128),
+                                                   # K plane blocks of 256 tokens (negative head_dim marks them)
+                                                   (3, 8, 2, [130, 64, 7], 70, -128), (2, 16, 1, [700, 255], 66, -128),
+                                                   (2, 12, 4, [260, 900], 3, -64)])
 def test_gqa_ragged_step_matches_per_sequence_oracle(B, Hq, Hkv, lens, steps, D):
     from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
+    kb = 256 if D < 0 else 64
+    D = abs(D)
     G = Hq // Hkv
     Lmax = max(lens) + steps + 5
     _, k, v = make_qkv(B, Lmax, Hkv, D, seed=sum(lens), n_outliers=4)
     rng = np.random.default_rng(Hq)
-    cache = RaggedGQACache(1, B, Lmax, Hq, Hkv, D)
+    cache = RaggedGQACache(1, B, Lmax, Hq, Hkv, D, k_block=kb)
     cache.record_levels = True
     oracles = []
     for b in range(B):
         cache.prefill(0, b, dev(k[b:b + 1, :lens[b]]), dev(v[b:b + 1, :lens[b]]))
-        oc = O.OracleCache(1, Lmax, Hq, D)
+        oc = O.OracleCache(1, Lmax, Hq, D, k_block=kb)
         oc.save(np.repeat(k[b:b + 1, :lens[b]], G, axis=2), np.repeat(v[b:b + 1, :lens[b]], G, axis=2), 0, lens[b])
         oracles.append(oc)
     flips = total = 0
@@ -59,7 +64,7 @@ def test_gqa_ragged_step_matches_per_sequence_oracle(B, Hq, Hkv, lens, steps, D)
     # planes of every KV head hold what the oracle holds for the query heads of its group
     for b in range(B):
         oc = oracles[b]
-        nb = oc.rest_start // 64
+        nb = O.cdiv(oc.rest_start, kb)
         for i in range(3):
             got = cache.k_planes[0][i][b, :, :nb].cpu().numpy()
             assert np.array_equal(got, oc.k_planes[i][0, ::G, :nb])
@@ -199,6 +204,13 @@ def test_unsupported_combinations_are_refused_before_launch():
         step(k_block=128)
     step()   # and the supported call goes through
     assert c.seq_lens[0].cpu().tolist() == [1, 1]
+    # 256-token K blocks: up to 16 query heads per KV head, head_dim up to 128
+    for hq, d in ((40, 128), (8, 256)):
+        c2 = RaggedGQACache(1, B, 256, hq, Hkv, d, k_block=256)
+        q2 = torch.zeros((B, 1, hq, d), dtype=torch.half, device="cuda")
+        kv2 = torch.zeros((B, 1, Hkv, d), dtype=torch.half, device="cuda")
+        with pytest.raises(RuntimeError, match="k_block|K plane blocks"):
+            c2.decode(0, q2, kv2, kv2)
 
 
 @pytest.mark.parametrize("Hq,Hkv", [(8, 8), (8, 2)])
