@@ -252,6 +252,49 @@ def test_step_on_as_many_rows_as_compute_units_matches_the_op_sequence():
         assert flips <= 0.01
 
 
+def test_fused_step_against_op_sequence_on_random_shapes(monkeypatch):
+    """A fixed sample of shapes (batch, heads, head_dim, prompt length, K block, launches of the step): the fused step
+    against the reference's sequence of ops and framework kernels on a second cache, token by token across flushes."""
+    from alignedkv_amd import load_library
+    from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
+    lib = load_library()
+    rng = np.random.default_rng(2024)
+    for case in range(24):
+        B = int(rng.integers(1, 5))
+        H = int(rng.choice([1, 2, 3, 4, 8]))
+        D = int(rng.choice([64, 128, 256]))
+        prefill = int(rng.integers(1, 700))
+        steps = int(rng.integers(1, 6)) if case % 3 else int(64 - prefill % 64 + rng.integers(0, 3))
+        kb = 256 if (D <= 128 and rng.integers(0, 2)) else 64
+        tail = str(int(rng.integers(0, 2)))
+        q_scale = float(rng.choice([1.0, 1.0, 0.1]))
+        monkeypatch.setenv("AKV_TUNE_TAIL", tail)
+        lib.akv_reload_tuning()
+        _, k, v = make_qkv(B, prefill + steps, H, D, seed=100 + case)
+        q = (q_scale * rng.standard_normal((B, steps, H, D))).astype(np.float16)
+        caches = []
+        for fused in (True, False):
+            c = QuantizedCache_AlignedKV(cfg(H, D), B, prefill + steps + 64, "cuda", torch.half, k_block=kb if fused else 64)
+            c.fused = fused
+            c.key_cache[0].save(dev(k[:, :prefill]), 0, prefill)
+            c.value_cache[0].save(dev(v[:, :prefill]), 0, prefill)
+            c.key_cache[0].record_levels = c.value_cache[0].record_levels = True
+            caches.append(c)
+        what = f"case {case}: B={B} H={H} D={D} prefill={prefill} steps={steps} k_block={kb} tail={tail} q_scale={q_scale}"
+        for s in range(steps):
+            t = prefill + s
+            outs = [c.auto_compute(dev(q[:, s:s + 1]), dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None) for c in caches]
+            assert (outs[0].float() - outs[1].float()).abs().max().item() <= 2e-3, what
+            if caches[1].key_cache[0].reststartpos:
+                assert torch.equal(caches[0].key_cache[0].last_levels, caches[1].key_cache[0].last_levels), what
+                a, b = caches[0].value_cache[0].last_levels, caches[1].value_cache[0].last_levels
+                assert (a != b).float().mean().item() <= 0.02, what
+        for i, name in enumerate(("v_cache_first_8", "v_cache_mid_4", "v_cache_last_4")):
+            assert torch.equal(getattr(caches[0].value_cache[0], name), getattr(caches[1].value_cache[0], name)), what
+    monkeypatch.delenv("AKV_TUNE_TAIL")
+    lib.akv_reload_tuning()
+
+
 def test_fused_step_rejects_bad_state():
     from alignedkv_amd.extension.KV_cache_cpp_extention import cuda_module as m
     B, H, D, cb, Lmax = 1, 2, 128, 64, 128
