@@ -1035,8 +1035,17 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     // replaces: 30.2 vs 34.8 us per step at batch 8 x 1024 tokens, 76.0 vs 78.7 at 8 x 4096, 141.6 vs 145.9 at
     // 16 x 4096; level at 32 x 4096 and behind at 8 x 16384 (one workgroup per unit streams at 4.5 TB/s, the V pass
     // of many small workgroups at 6).
+    // With fewer rows than compute units a row's workgroup streams alone at about 45 GB/s, while the V pass of many
+    // small workgroups needs 4 us or the time of its bytes at 5 TB/s and then two more launches (2.5 us): measured
+    // with 32 heads x 128 at batch 1 x 1024 tokens 21.7 vs 23.9 us per step, 2 x 2048: 25.5 vs 26.3, 4 x 4096: 43.7
+    // vs 45.6, but 1 x 4096: 30.3 vs 27.0.
     const int cus = compute_units();
-    bool tail = cus > 0 && (B * Hq) % cus == 0 && (B * Hq) / cus <= tail_rows_per_cu;
+    const int rows = B * Hq;
+    bool tail = cus > 0 && rows % cus == 0 && rows / cus <= tail_rows_per_cu;
+    if (cus > 0 && rows < cus) {
+        const float row_us = (float)R * D / 45e3f, passes_us = fmaxf(4.f, (float)rows * R * D / 5e6f) + 2.5f;
+        tail = row_us < passes_us;
+    }
     { AKV_TUNE("AKV_TUNE_TAIL", v); if (has_v) tail = v != 0; }
     tail = tail && n_blocks >= 1 && R <= tail_max_tokens && geo.G == 1 && !ragged && !(literal_broadcast && !ref);
     if (tail) {

@@ -26,11 +26,11 @@ namespace akv {
 __global__ __launch_bounds__(256) void k_save_blocks_kernel(
     uint8_t *__restrict__ first_8, uint8_t *__restrict__ mid_4, uint8_t *__restrict__ last_4,
     const unsigned short *__restrict__ k_new, int n_max_blocks, int H, int D, int cb, int tile_slots,
-    int start_pos, int n_tokens, int seqlen) {
+    int start_pos, int n_tokens, int seqlen, int first_tile) {
     extern __shared__ unsigned short tile[];   // [tile_slots][D + 2]
     const int pitch = D + 2;
     const int h = blockIdx.y, b = blockIdx.z;
-    const int t0 = blockIdx.x * tile_slots;                       // first source token of this tile
+    const int t0 = (first_tile + blockIdx.x) * tile_slots;        // first source token of this tile
     const int pos = start_pos + t0;                               // its position in the cache (a multiple of tile_slots)
     const int z = pos / cb, slot0 = pos - z * cb;                 // destination block and first slot in it
     const int nv = min(tile_slots, n_tokens - t0);                // valid tokens of this tile
@@ -82,6 +82,74 @@ __global__ __launch_bounds__(256) void k_save_blocks_kernel(
             for (int i = 0; i < nbytes; ++i) {
                 m4[(int64_t)d * (cb >> 1) + (j >> 1) + i] = (uint8_t)(mw >> (8 * i));
                 l4[(int64_t)d * (cb >> 1) + (j >> 1) + i] = (uint8_t)(lw >> (8 * i));
+            }
+        }
+    }
+}
+
+// The same bytes for whole tiles of ts tokens (64, 128 or 256: as many as divide the block) when D is a multiple of 8 and
+// everything is 16-byte aligned.  LDS holds the tile as it comes (16-byte vectors of 8 channels of one token) and is
+// read back in the same vectors, 8 tokens x 8 channels per thread, which the thread turns into the plane words of its 8
+// channels in registers: 16 LDS operations of 16 bytes per 128 elements instead of 96 of 2 bytes.  The vector index
+// within a token's row is XOR-ed with a function of the token so that the reads spread over the banks.  Thread
+// (o, jg) = (channel octet, group of 8 slots): the ts/8 threads of an octet write ts contiguous bytes of each first_8
+// row and ts/2 of each nibble row -- with blocks of 256 tokens a whole row at once (tiles of 64 slots left every 128-byte
+// line to four workgroups: 2.8 TB/s read + write, against 4.3 with blocks of 64 tokens).
+// A workgroup takes dc of the D channels.  grid (tiles * D / dc, H, B); ts * dc / 64 threads; dynamic LDS 2 ts dc bytes.
+__global__ __launch_bounds__(256) void k_save_tiles_kernel(uint8_t *__restrict__ first_8, uint8_t *__restrict__ mid_4,
+                                                          uint8_t *__restrict__ last_4, const u32x4 *__restrict__ k_new,
+                                                          int n_max_blocks, int H, int D, int cb, int ts, int dc, int start_pos,
+                                                          int first_token, int seqlen) {
+    extern __shared__ u32x4 tile_vec[];        // [ts tokens][dc / 8 vectors]
+    const int octs = D >> 3, wo = dc >> 3;     // vectors per token: in memory, in this workgroup's share
+    const int chunks = D / dc;
+    const int tile_idx = blockIdx.x / chunks, chunk = blockIdx.x - tile_idx * chunks;
+    const int swz = (wo & (wo - 1)) == 0 ? wo - 1 : 0;
+    const int swz_mul = wo >= 16 ? 2 : 1;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int t0 = first_token + tile_idx * ts;
+    const int pos = start_pos + t0;
+    const int z = pos / cb, slot0 = pos - z * cb;
+    for (int idx = threadIdx.x; idx < ts * wo; idx += blockDim.x) {
+        const int j = idx / wo, o = idx - j * wo;
+        tile_vec[j * wo + (o ^ (((j >> 3) * swz_mul) & swz))] = k_new[(((int64_t)b * seqlen + t0 + j) * H + h) * octs + chunk * wo + o];
+    }
+    __syncthreads();
+    const int64_t blk_base = (((int64_t)b * H + h) * n_max_blocks + z) * (int64_t)D * (cb >> 1);
+    uint8_t *f8 = first_8 + blk_base * 2 + slot0;
+    uint8_t *m4 = mid_4 + blk_base + (slot0 >> 1);
+    uint8_t *l4 = last_4 + blk_base + (slot0 >> 1);
+    const int groups = ts >> 3;
+    for (int task = threadIdx.x; task < groups * wo; task += blockDim.x) {
+        const int o = task / groups, jg = task - o * groups;
+        u32 x[8][4];                           // [token 8 jg + i][channel pair c]: channels 8 o + 2 c (low half), + 1 (high half)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const u32x4 v = tile_vec[(8 * jg + i) * wo + (o ^ ((jg * swz_mul) & swz))];
+            x[i][0] = v.x; x[i][1] = v.y; x[i][2] = v.z; x[i][3] = v.w;
+        }
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            // high bytes: [even channel of token a, of token b, odd channel of token a, of token b]
+            const u32 h01 = __builtin_amdgcn_perm(x[1][c], x[0][c], 0x07030501u), h23 = __builtin_amdgcn_perm(x[3][c], x[2][c], 0x07030501u);
+            const u32 h45 = __builtin_amdgcn_perm(x[5][c], x[4][c], 0x07030501u), h67 = __builtin_amdgcn_perm(x[7][c], x[6][c], 0x07030501u);
+            // low bytes of the even slots and of the odd slots, same arrangement
+            const u32 e02 = __builtin_amdgcn_perm(x[2][c], x[0][c], 0x06020400u), e46 = __builtin_amdgcn_perm(x[6][c], x[4][c], 0x06020400u);
+            const u32 o13 = __builtin_amdgcn_perm(x[3][c], x[1][c], 0x06020400u), o57 = __builtin_amdgcn_perm(x[7][c], x[5][c], 0x06020400u);
+#pragma unroll
+            for (int par = 0; par < 2; ++par) {
+                const u32 sel = par ? 0x07060302u : 0x05040100u;
+                const int ch = chunk * dc + 8 * o + 2 * c + par;
+                u32x2 hw;
+                hw.x = __builtin_amdgcn_perm(h23, h01, sel);       // slots 8 jg + 0..3
+                hw.y = __builtin_amdgcn_perm(h67, h45, sel);       // slots 8 jg + 4..7
+                const u32 ev = __builtin_amdgcn_perm(e46, e02, sel);   // low bytes of slots 0, 2, 4, 6
+                const u32 od = __builtin_amdgcn_perm(o57, o13, sel);   // of slots 1, 3, 5, 7
+                const u32 mw = (ev & 0xF0F0F0F0u) | ((od >> 4) & 0x0F0F0F0Fu);
+                const u32 lw = ((ev << 4) & 0xF0F0F0F0u) | (od & 0x0F0F0F0Fu);
+                *reinterpret_cast<u32x2 *>(f8 + (int64_t)ch * cb + 8 * jg) = hw;
+                *reinterpret_cast<u32 *>(m4 + (int64_t)ch * (cb >> 1) + 4 * jg) = mw;
+                *reinterpret_cast<u32 *>(l4 + (int64_t)ch * (cb >> 1) + 4 * jg) = lw;
             }
         }
     }
@@ -278,10 +346,40 @@ int launch_k_save_blocks(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, cons
                     d_block);
         size_t lds = (size_t)tile_slots * (d_head + 2) * sizeof(unsigned short);
         AKV_REQUIRE(lds <= 64 * 1024, "k_cache_save: d_head=%d too large for the staging tile (%zu bytes)", d_head, lds);
-        hipLaunchKernelGGL(k_save_blocks_kernel, dim3((n_tokens + tile_slots - 1) / tile_slots, n_kv_heads, bsz), dim3(256), lds,
-                           st, first_8, mid_4, last_4, reinterpret_cast<const unsigned short *>(k_new), n_max_blocks,
-                           n_kv_heads, d_head, d_block, tile_slots, start_pos, n_tokens, seqlen);
-        return check_launch("k_cache_save");
+        // whole tiles of 16-byte aligned data take the vector kernel (first tiles as long as divide the block, then of
+        // 64 tokens), what remains the general one
+        const bool vec = tile_slots == 64 && d_block % 64 == 0 && d_head % 8 == 0 && ((uintptr_t)k_new & 15) == 0 &&
+                         (((uintptr_t)first_8 | (uintptr_t)mid_4 | (uintptr_t)last_4) & 7) == 0;
+        const int n_tiles = (n_tokens + tile_slots - 1) / tile_slots;
+        int n_vec = 0;       // 64-token tiles done by the vector kernel
+        if (vec) {
+            int done = 0;    // tokens
+            const int big = d_block % 256 == 0 ? 256 : (d_block % 128 == 0 ? 128 : 64);
+            for (int ts = big; ts >= 64; ts = ts > 64 ? 64 : 0) {
+                if (ts != 64 && (start_pos + done) % ts != 0) continue;
+                const int n = (n_tokens - done) / ts;
+                if (n == 0) continue;
+                // channels per workgroup: a divisor of d_head (in whole vectors) that keeps the tile within 32 KiB
+                int dc = d_head;
+                while (dc > 8 && (2 * ts * dc > 32 * 1024 || d_head % dc != 0 || dc % 8 != 0)) dc -= 8;
+                if (2 * ts * dc > 64 * 1024) continue;
+                const int threads = min(256, (ts * dc / 64 + 63) / 64 * 64);
+                hipLaunchKernelGGL(k_save_tiles_kernel, dim3(n * (d_head / dc), n_kv_heads, bsz), dim3(threads), (size_t)2 * ts * dc, st,
+                                   first_8, mid_4, last_4, reinterpret_cast<const u32x4 *>(k_new), n_max_blocks, n_kv_heads, d_head,
+                                   d_block, ts, dc, start_pos, done, seqlen);
+                int rc = check_launch("k_cache_save(tiles)");
+                if (rc != AKV_OK) return rc;
+                done += n * ts;
+            }
+            n_vec = done / 64;
+        }
+        if (n_tiles > n_vec) {
+            hipLaunchKernelGGL(k_save_blocks_kernel, dim3(n_tiles - n_vec, n_kv_heads, bsz), dim3(256), lds, st, first_8, mid_4,
+                               last_4, reinterpret_cast<const unsigned short *>(k_new), n_max_blocks, n_kv_heads, d_head,
+                               d_block, tile_slots, start_pos, n_tokens, seqlen, n_vec);
+            return check_launch("k_cache_save");
+        }
+        return AKV_OK;
     }
     if (seqlen == 1) {
         const int blk = start_pos / d_block;

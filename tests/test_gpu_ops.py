@@ -40,7 +40,8 @@ def v_planes_dev(B, H, Lmax, D):
 @pytest.mark.parametrize("B,H,D,cb,S,start_blk", [
     (2, 4, 128, 64, 256, 0), (1, 4, 128, 64, 200, 0), (2, 2, 128, 64, 64, 3),
     (2, 3, 8, 8, 24, 0), (1, 2, 64, 64, 128, 1), (1, 1, 256, 64, 64, 0), (1, 2, 20, 16, 48, 0),
-    (1, 2, 128, 256, 512, 0)])
+    (1, 2, 128, 256, 512, 0), (1, 2, 64, 256, 768, 1), (1, 2, 256, 256, 512, 0), (1, 2, 72, 128, 384, 0),
+    (2, 2, 128, 128, 384, 1), (1, 1, 24, 192, 384, 0), (1, 3, 328, 256, 256, 0)])
 def test_k_cache_save_bit_exact(mod, B, H, D, cb, S, start_blk):
     rng = np.random.default_rng(S + D)
     kb = rng.integers(0, 65536, (B, S, H, D)).astype(np.uint16)
@@ -49,6 +50,23 @@ def test_k_cache_save_bit_exact(mod, B, H, D, cb, S, start_blk):
     O.k_cache_save(*want, kb, S // cb, cb, start_blk * cb, S)
     got = k_planes_dev(B, H, Lmax, D, cb)
     mod.k_cache_save(*got, u8(kb), B, H, S // cb, Lmax // cb, D, cb, start_blk * cb, S)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.cpu().numpy(), w)
+
+
+def test_k_cache_save_from_a_source_that_is_not_16_byte_aligned(mod):
+    """The vector kernel wants 16-byte aligned tokens; any other source takes the general kernel, same bytes."""
+    B, H, D, cb, S = 1, 2, 128, 64, 128
+    rng = np.random.default_rng(5)
+    kb = rng.integers(0, 65536, (B, S, H, D)).astype(np.uint16)
+    want = O.k_planes_alloc(B, H, 4 * cb, D, cb)
+    O.k_cache_save(*want, kb, S // cb, cb, 0, S)
+    buf = torch.zeros(kb.nbytes + 8, dtype=torch.uint8, device="cuda")
+    src = buf[8:]
+    assert src.data_ptr() % 16 == 8
+    src.copy_(torch.from_numpy(kb.view(np.uint8).reshape(-1)))
+    got = k_planes_dev(B, H, 4 * cb, D, cb)
+    mod.k_cache_save(*got, src, B, H, S // cb, 4, D, cb, 0, S)
     for g, w in zip(got, want):
         assert np.array_equal(g.cpu().numpy(), w)
 
