@@ -365,9 +365,12 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
                        const unsigned short *q, const unsigned short *k_new, unsigned short *scores,
                        uint8_t *levels_out, u32 *prep, const StepGeom &geo, int B, int n_blocks, bool ref, float scale,
                        hipStream_t st, PassShape *shape_only) {
-    int sl = 8;
-    { AKV_TUNE("AKV_TUNE_K_SL", v); if (has_v) sl = v == 16 ? 16 : (v == 4 ? 4 : 8); }
-    if (geo.kb == 256) sl = 8;
+    // Slots per lane.  K blocks of 256 tokens: 16, so that the 16 lanes of a token-set group read a channel's whole row
+    // of a block (256 B of first_8, 128 B of a nibble plane); measured at batch 32, 32 over 8 heads, lengths 2048..8192:
+    // 62.5 us, against 78 with 8 slots per lane (half rows) and 68.8 with blocks of 64 tokens and 8 slots.  Three tiles
+    // ahead instead of one (one wave per SIMD instead of two) measured 75.7 us, two tasks per wave 69.1.
+    int sl = geo.kb == 256 ? 16 : 8;
+    { AKV_TUNE("AKV_TUNE_K_SL", v); if (has_v) sl = v == 16 ? 16 : (v == 4 && geo.kb != 256 ? 4 : 8); }
     const int nbt = sl / 4;
     const int n_tasks = (n_blocks + nbt - 1) / nbt;
     int tpw = 1;
@@ -395,7 +398,8 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
     int ahead = 3;
     { AKV_TUNE("AKV_TUNE_K_AHEAD", v); if (has_v) ahead = v; }
     constexpr int DEEP = (D / 16) % 8 == 0 ? 7 : 3;
-    if (geo.kb == 256) { if (ref) AKV_MK(true, 8, 3, 2); else AKV_MK(false, 8, 3, 2); }   // (the default tile shape only)
+    if (geo.kb == 256 && sl == 16) { if (ref) AKV_MK(true, 16, 1, 2); else AKV_MK(false, 16, 1, 2); }
+    else if (geo.kb == 256) { if (ref) AKV_MK(true, 8, 3, 2); else AKV_MK(false, 8, 3, 2); }
     else if (sl == 16) { if (ref) AKV_MK(true, 16, 1, 0); else AKV_MK(false, 16, 1, 0); }
     else if (sl == 8 && ahead == 7) { if (ref) AKV_MK(true, 8, DEEP, 0); else AKV_MK(false, 8, DEEP, 0); }
     else if (sl == 8) { if (ref) AKV_MK(true, 8, 3, 0); else AKV_MK(false, 8, 3, 0); }

@@ -44,10 +44,9 @@ def parse():
     ap.add_argument("--cache-len", type=int, default=4096)
     ap.add_argument("--layers", type=int, default=4, help="caches the steps rotate over")
     ap.add_argument("--k-kind", default="outlier", choices=["outlier", "lognormal"])
-    ap.add_argument("--k-block", type=int, default=None, choices=[64, 256],
-                    help="tokens per block of the K planes (the ops' d_block): 256 = a nibble row is a whole 128-byte line, "
-                         "64 = the block length the reference's Python classes use.  Default: 256 for c2, 64 for c3 (with "
-                         "grouped heads nearly every row is fetched anyway and 64-token blocks measure 9 us faster)")
+    ap.add_argument("--k-block", type=int, default=256, choices=[64, 256],
+                    help="tokens per block of the K planes (the ops' d_block): 256 (default) = a nibble row is a whole "
+                         "128-byte line, 64 = the block length the reference's Python classes use")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=10)
     ap.add_argument("--seed", type=int, default=0)
@@ -59,8 +58,6 @@ def parse():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB copy kernel (known size, for scaling hardware byte counters)")
     a = ap.parse_args()
-    if a.k_block is None:
-        a.k_block = 256 if a.workload == "c2" else 64
     return a
 
 
