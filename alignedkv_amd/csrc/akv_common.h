@@ -158,6 +158,11 @@ __device__ __forceinline__ u32x4 load_b128_device(const __amdgpu_buffer_rsrc_t r
     return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, kDeviceScope);
 }
 
+// Index of the wave in its workgroup as a scalar: what is derived from it (a wave's share of the tokens, loop bounds,
+// validity of a tile) then lives in scalar registers, loops over it are uniform loops and the conditions cost no
+// vector instructions.  (threadIdx.x >> 6 alone is a per-lane value to the compiler.)
+__device__ __forceinline__ int wave_index() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
 __device__ __forceinline__ float wave_xor_add(float v, int mask) { return v + __shfl_xor(v, mask, 64); }
 
 }  // namespace akv

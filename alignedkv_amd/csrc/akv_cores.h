@@ -712,7 +712,7 @@ __device__ __forceinline__ void v_fold_lanes(float *acc, float (*wave_part)[D]) 
     // leaves wave_part[wave][d] = this wave's sum for channel d (caller synchronises)
     constexpr int LPR = D / 16;
     constexpr int NV = LPR == 16 ? 4 : (LPR == 8 ? 2 : 1);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     int ch = (lane % LPR) * 16;
     reduce_scatter_step<16>(acc, 32);
     ch += (lane & 32) ? 8 : 0;
@@ -734,7 +734,7 @@ template <int D>
 __device__ __forceinline__ void v_fold_workgroup(float *acc, float (*wave_part)[D], float *out) {
     constexpr int LPR = D / 16;
     constexpr int NV = LPR == 16 ? 4 : (LPR == 8 ? 2 : 1);   // sums left per lane
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     int ch = (lane % LPR) * 16;
     reduce_scatter_step<16>(acc, 32);
     ch += (lane & 32) ? 8 : 0;

@@ -248,7 +248,7 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     float scale) {
     constexpr int CB = 64;
     constexpr int NG = D / 16;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     int bx, hkv, b, chunk, gq;
     if (!step_block(geo, bx, hkv, b)) return;
     decode_group_block(geo.G, bx, chunk, gq);
@@ -307,7 +307,7 @@ __global__ __launch_bounds__(256) void fused_k_pass256_kernel(
     float scale) {
     constexpr int KB = 256;
     constexpr int NG = D / 4;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     int chunk, h, b;
     if (!step_block(geo, chunk, h, b)) return;
     const int bh = b * geo.Hq + h;
@@ -732,7 +732,7 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     constexpr int NW = NT / 64;
     __shared__ float wave_part[NW][D];
     __shared__ u32 row_amin;
-    const int wave = threadIdx.x >> 6;
+    const int wave = wave_index();
     const int bh = blockIdx.x;
     int R, nrest_unused;
     seq_state(ma.g, bh / ma.g.Hq, R, nrest_unused);
@@ -807,7 +807,7 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
     uint8_t *__restrict__ levels_out, int levels_stride, uint8_t *__restrict__ amin_out, StepGeom geo,
     int tokens_per_wave, int n_chunks) {
     __shared__ float wave_part[4][D];
-    const int wave = threadIdx.x >> 6;
+    const int wave = wave_index();
     int bx, hkv, b, chunk, gq;
     if (!step_block(geo, bx, hkv, b)) return;
     decode_group_block(geo.G, bx, chunk, gq);

@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void group_k_pass_kernel(
     constexpr int CB = 64;
     constexpr int NG = D / 16;
     constexpr int HG = NG / 2;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     int chunk, by, b;
     if (!step_block(geo, chunk, by, b)) return;
     const int n_sub = geo.G / GH;
@@ -214,7 +214,7 @@ __global__ __launch_bounds__(256) void group_v_pass_kernel(
     constexpr int U = VGroupProbs<D, REF, GH>::U, HV = U / 2;
     constexpr int ST = U * TPL;               // tokens per step of two half tiles
     __shared__ float wave_part[4][D];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     int chunk, by, b;
     if (!step_block(geo, chunk, by, b)) return;
     const int n_sub = geo.G / GH;

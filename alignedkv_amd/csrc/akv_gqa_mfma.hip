@@ -265,7 +265,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && 
     constexpr int PB = 64 / SL;    // pieces (token sets) per block
     constexpr int NBT = 16 / PB;   // blocks per task
     static_assert(KG % (AHEAD + 1) == 0, "the tile ring is rotated by unrolling");
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     int chunk, hkv, b;
     if (!step_block(geo, chunk, hkv, b)) return;
     const int G = geo.G;
@@ -508,7 +508,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     constexpr int CPP = D / 16;        // channels per lane
     constexpr int MACRO = 64;          // tokens per macro step: 4 tiles of 16 tokens
     __shared__ float fold[4][4][D];    // [wave][head of the pass][channel]
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     int chunk, hkv, b;
     if (!step_block(geo, chunk, hkv, b)) return;
     const int G = geo.G;

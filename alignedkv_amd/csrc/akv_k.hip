@@ -190,7 +190,7 @@ __global__ __launch_bounds__(256) void k_compute_cb64_kernel(
     int blocks_per_wave, float scale) {
     constexpr int CB = 64;
     constexpr int NG = D / 16;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     const int h = blockIdx.y, b = blockIdx.z;
     const int bh = b * H + h;
     const int first_blk = (blockIdx.x * 4 + wave) * blocks_per_wave;
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(256) void k_compute_cb256_kernel(
     int blocks_per_wave, float scale) {
     constexpr int CB = 256;
     constexpr int NG = D / 4;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_index();
     const int h = blockIdx.y, b = blockIdx.z;
     const int bh = b * H + h;
     const int first_blk = (blockIdx.x * 4 + wave) * blocks_per_wave;

@@ -110,7 +110,7 @@ __global__ __launch_bounds__(256) void v_compute_tuned_kernel(
     uint8_t *__restrict__ levels_out, int H, int max_seq_len, int s_last_dim, int n_tokens, int tokens_per_wave,
     int n_chunks) {
     __shared__ float wave_part[4][D];
-    const int wave = threadIdx.x >> 6;
+    const int wave = wave_index();
     const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     const int bh = b * H + h;
     const int t_begin = (chunk * 4 + wave) * tokens_per_wave;
