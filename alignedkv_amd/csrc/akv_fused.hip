@@ -356,6 +356,87 @@ __global__ __launch_bounds__(256) void fused_k_pass256_kernel(
                          need_mid, need_last, scores + (int64_t)bh * geo.row_stride, R, scale);
 }
 
+// The same pass for short caches: one workgroup per 256-token block, its four waves take a quarter of the channels each
+// and add their partial scores through LDS.  With a whole block per wave a cache of 1024 tokens x 32 heads gives the
+// pass 128 waves of 48 KiB each (8.1 us per step at batch 1); split like this it has 512 waves of 12 KiB, all loads
+// of a wave in flight at once.  grid (n_kblocks, H, B), 256 threads.
+template <int D, bool REF>
+__global__ __launch_bounds__(256) void fused_k_pass256_split_kernel(
+    const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
+    const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
+    unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, StepGeom geo, float scale) {
+    constexpr int KB = 256;
+    constexpr int NG = D / 4;      // load groups of 4 channels
+    constexpr int HG = 4;          // groups per half tile
+    constexpr int GW = NG / 4;     // groups per wave
+    constexpr int NT = GW / HG;    // half tiles per wave
+    static_assert(GW % HG == 0 && NG <= 32, "head_dim 64 or 128");
+    const int lane = threadIdx.x & 63, wave = wave_index();
+    int blk, h, b;
+    if (!step_block(geo, blk, h, b)) return;
+    const int bh = b * geo.Hq + h;
+    int R, nrest;
+    seq_state(geo, b, R, nrest);
+    const int n_blocks = (R + KB - 1) / KB;     // the last one may be partly filled
+    if (blk >= n_blocks) return;
+    const int64_t plane_off = (int64_t)bh * geo.n_max_blocks * (D * (KB / 2));
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(first_8 + plane_off * 2, (u32)n_blocks * (D * KB));
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(mid_4 + plane_off, (u32)n_blocks * (D * KB / 2));
+    const __amdgpu_buffer_rsrc_t rL = make_rsrc(last_4 + plane_off, (u32)n_blocks * (D * KB / 2));
+    const int g_first = wave * GW;
+    KHalfTile<HG> t[NT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) k256_issue_h<D, HG>(t[i], rH, blk, g_first + HG * i);
+    __builtin_amdgcn_sched_barrier(0);
+    __shared__ u32 staged[D];      // [channel]: q bits | exponent sum << 16
+    __shared__ float part[4][KB];  // [wave][slot]: partial scores
+    for (int c = threadIdx.x; c < D; c += 256) {
+        const u32 qb = q[(int64_t)bh * D + c];
+        // column max including the token appended by this step
+        const u32 cm = max((u32)kcm[(int64_t)bh * D + c], exp_field(k_new[(int64_t)bh * D + c]));
+        staged[c] = qb | (((exp_field(qb) + cm) & 0xffu) << 16);
+    }
+    __syncthreads();
+    u32 mx = 0;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) mx = max(mx, staged[4 * g + (lane >> 4)] >> 16);
+    mx = max(mx, (u32)__shfl_xor((int)mx, 16, 64));
+    mx = max(mx, (u32)__shfl_xor((int)mx, 32, 64));
+    float qf[GW];
+    u32 need_mid = 0, need_last = 0;   // bit g: of the wave's group g
+#pragma unroll
+    for (int g = 0; g < GW; ++g) {
+        const u32 w = staged[4 * (g_first + g) + (lane >> 4)];
+        qf[g] = lo_half_to_float(w);
+        const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)(w >> 16));
+        need_mid |= (lv < 2 ? 1u : 0u) << g;
+        need_last |= (lv == 0 ? 1u : 0u) << g;
+        if (levels_out != nullptr && blk == 0 && (lane & 15) == 0)
+            levels_out[(int64_t)bh * D + 4 * (g_first + g) + (lane >> 4)] = (uint8_t)lv;
+    }
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+        k256_issue_ml<D, HG>(t[i], rM, rL, blk, g_first + HG * i, need_mid << g_first, need_last << g_first);
+    __builtin_amdgcn_sched_barrier(0);
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NT; ++i) k_compute_half<HG>(acc, t[i], HG * i, qf, need_mid, need_last);
+    reduce_scatter_step<16>(acc, 32);
+    reduce_scatter_step<8>(acc, 16);
+    const int slot = (lane & 15) * 16 + ((lane & 32) ? 8 : 0) + ((lane & 16) ? 4 : 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part[wave][slot + i] = acc[i];
+    __syncthreads();
+    const int token = blk * KB + threadIdx.x;
+    if (token < R) {
+        const float sum = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+        // device scope: the workgroup that runs the softmax for this (batch, head) may sit on another XCD
+        store_u16_device(make_rsrc(scores + (int64_t)bh * geo.row_stride, (u32)R * 2), token * 2, float_to_half_bits(sum * scale));
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // middle.  grid (B*H), 256 threads.
 // ------------------------------------------------------------------------------------------------
@@ -924,7 +1005,12 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         return AKV_ERR_INVALID;
     }
     const int n_kblocks = (R + kb - 1) / kb;    // K plane blocks that hold tokens (the last one may be partly filled)
-    const int bpw = kb == 256 ? k256_blocks_per_wave(B, Hq, n_kblocks) : k_blocks_per_wave(B, Hq, n_blocks);
+    // short caches: a block per workgroup instead of per wave while that still fits the machine at once (16 waves per
+    // compute unit)
+    bool k_split = kb == 256 && geo.G == 1 && D <= 128 && !ragged && compute_units() > 0 &&
+                   (int64_t)B * Hq * n_kblocks <= 4 * compute_units();
+    { AKV_TUNE("AKV_TUNE_K_SPLIT", v); if (has_v) k_split = k_split && v != 0; }
+    const int bpw = k_split ? 1 : (kb == 256 ? k256_blocks_per_wave(B, Hq, n_kblocks) : k_blocks_per_wave(B, Hq, n_blocks));
     bool matrix_v = matrix;
     { AKV_TUNE("AKV_TUNE_MFMA_V", v); if (has_v) matrix_v = matrix_v && v != 0; }
     VPlan p = v_plan(B, grouped ? Hq / group_heads(geo.G) : Hq, D, R);
@@ -943,7 +1029,8 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
             int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo, B, n_blocks, ref, scale, st, &ks);
             if (rc != AKV_OK) return rc;
         } else {
-            ks = PassShape{group_grid_x((n_kblocks + 4 * bpw - 1) / (4 * bpw), geo.G), Hkv, 4 * bpw * kb};
+            if (k_split) ks = PassShape{n_kblocks, Hkv, kb};
+            else ks = PassShape{group_grid_x((n_kblocks + 4 * bpw - 1) / (4 * bpw), geo.G), Hkv, 4 * bpw * kb};
         }
         if (matrix_v) vs = PassShape{p.n_chunks, Hkv, p.chunk_tokens};
         else vs = PassShape{grouped ? p.n_chunks : group_grid_x(p.n_chunks, geo.G), grouped ? Hkv * (geo.G / group_heads(geo.G)) : Hkv,
@@ -1004,6 +1091,18 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
     } else if (n_blocks > 0 && grouped) {
         int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo_k, B, n_blocks, ref, scale, st);
+        if (rc != AKV_OK) return rc;
+    } else if (n_blocks > 0 && kb == 256 && k_split) {
+        dim3 grid(ks.grid_x, ks.grid_y, B);
+        if constexpr (D <= 128) {
+            if (ref)
+                hipLaunchKernelGGL((fused_k_pass256_split_kernel<D, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
+                                   k_levels_out, geo_k, scale);
+            else
+                hipLaunchKernelGGL((fused_k_pass256_split_kernel<D, false>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
+                                   k_levels_out, geo_k, scale);
+        }
+        int rc = check_launch("decode_step(k_pass256 split)");
         if (rc != AKV_OK) return rc;
     } else if (n_blocks > 0 && kb == 256) {
         dim3 grid(ks.grid_x, ks.grid_y, B);
