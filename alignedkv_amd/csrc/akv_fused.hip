@@ -124,8 +124,15 @@ __device__ __forceinline__ void build_task_maps(const StepGeom &geo, const TaskM
 // planes (same bytes as k_save_blocks_kernel / v_save_vec8_kernel).  kPreSplit workgroups per (batch, KV head):
 // the first appends, and a flush is shared between them (16 tokens of V and a quarter of the channels of K each;
 // the token of this step is taken from the step's inputs, so no workgroup waits for the append).
-// grid (B*Hkv*kPreSplit [+ 2*B for the task maps]), 256 threads.
+// grid (B*Hkv*kPreSplit [+ ceil(B*Hkv/4) for the set-up of the matrix-core K pass] [+ 2*B for the task maps]), 256 threads.
 constexpr int kPreSplit = 4;
+// what the matrix-core K pass wants set up per (batch, KV head) (mfma_k_prepare); words == nullptr: nothing
+struct KPrepare {
+    const unsigned short *q;
+    u32 *words;
+    uint8_t *levels_out;
+    int ref;
+};
 template <int D>
 __global__ __launch_bounds__(256) void fused_pre_kernel(uint8_t *__restrict__ kf8, uint8_t *__restrict__ km4,
                                                         uint8_t *__restrict__ kl4, uint8_t *__restrict__ vf8,
@@ -134,14 +141,25 @@ __global__ __launch_bounds__(256) void fused_pre_kernel(uint8_t *__restrict__ kf
                                                         const unsigned short *__restrict__ v_new,
                                                         unsigned short *__restrict__ restk, unsigned short *__restrict__ restv,
                                                         uint8_t *__restrict__ kcm, uint8_t *__restrict__ vcm, StepGeom geo,
-                                                        TaskMaps maps, int B) {
+                                                        TaskMaps maps, int B, KPrepare prep) {
     constexpr int CB = 64, S = kPreSplit, DS = D / S, TS = CB / S;
     static_assert(DS % 8 == 0, "a workgroup's share of the channels is a whole number of 16-byte vectors");
     __shared__ unsigned short tile[CB][DS + 2];
     __shared__ int map_scratch[8];
     const int n_bh = B * geo.Hkv;
-    if ((int)blockIdx.x >= n_bh * S) {   // the extra workgroups: task maps of the K pass and of the V pass
-        build_task_maps(geo, maps, B, map_scratch, (int)blockIdx.x - n_bh * S);
+    const int n_prep = prep.words != nullptr ? (n_bh + 3) / 4 : 0;
+    if ((int)blockIdx.x >= n_bh * S + n_prep) {   // the last workgroups: task maps of the K pass and of the V pass
+        build_task_maps(geo, maps, B, map_scratch, (int)blockIdx.x - n_bh * S - n_prep);
+        return;
+    }
+    if ((int)blockIdx.x >= n_bh * S) {   // set-up of the matrix-core K pass, a wave per (batch, KV head)
+        if constexpr (D <= 128) {
+            const int bh_kv = ((int)blockIdx.x - n_bh * S) * 4 + wave_index();
+            if (bh_kv < n_bh) {
+                if (prep.ref) mfma_k_prepare<D, true>(kcm, prep.q, k_new, prep.words, prep.levels_out, geo, bh_kv);
+                else mfma_k_prepare<D, false>(kcm, prep.q, k_new, prep.words, prep.levels_out, geo, bh_kv);
+            }
+        }
         return;
     }
     const int bh = blockIdx.x / S, sub = blockIdx.x - bh * S, b = bh / geo.Hkv, h = bh - b * geo.Hkv;
@@ -1048,6 +1066,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     }
 
     int persist = 1;
+    bool k_prepared = false;     // the set-up of the matrix-core K pass was done by the first kernel
     if (ragged) {
         // per-sequence lengths live on the device: one small kernel appends every token and flushes the rest
         // buffers that fill up with it; its last 2*B workgroups write the task maps
@@ -1057,8 +1076,12 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         maps.v_chunks = v_chunks;
         maps.k = ks;
         maps.v = vs;
-        hipLaunchKernelGGL((fused_pre_kernel<D>), dim3(B * Hkv * kPreSplit + (mapped ? 2 * B : 0)), dim3(256), 0, st, kf8, km4, kl4, vf8, vm4,
-                           vl4, k16, v16, rk16, rv16, kcm, vcm, geo, maps, B);
+        KPrepare prep = {q16, nullptr, k_levels_out, ref ? 1 : 0};
+        if (n_blocks > 0 && matrix) prep.words = reinterpret_cast<u32 *>(ws + lay.prep);
+        k_prepared = prep.words != nullptr;
+        const int n_prep = k_prepared ? (B * Hkv + 3) / 4 : 0;
+        hipLaunchKernelGGL((fused_pre_kernel<D>), dim3(B * Hkv * kPreSplit + n_prep + (mapped ? 2 * B : 0)), dim3(256), 0, st, kf8, km4,
+                           kl4, vf8, vm4, vl4, k16, v16, rk16, rv16, kcm, vcm, geo, maps, B, prep);
         int rc = check_launch("decode_step(pre)");
         if (rc != AKV_OK) return rc;
         persist = 0;
@@ -1087,7 +1110,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         int rc = AKV_OK;
         if constexpr (D <= 128)
             rc = launch_mfma_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, reinterpret_cast<u32 *>(ws + lay.prep),
-                                       geo_k, B, n_blocks, ref, scale, st);
+                                       geo_k, B, n_blocks, ref, scale, st, nullptr, k_prepared);
         if (rc != AKV_OK) return rc;
     } else if (n_blocks > 0 && grouped) {
         int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo_k, B, n_blocks, ref, scale, st);

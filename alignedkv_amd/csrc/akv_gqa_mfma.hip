@@ -162,63 +162,13 @@ __device__ __forceinline__ void kt_compute(f32x4 *acc, const KTaskTile<SL> &t, i
 // query head j of the group at the channels 16 kg + 4 r + kq and leaves, for the K-pass lane of the same index,
 // 2 KG words of q (packed fp16 pairs r = 0,1 / 2,3 per channel group) and 4 words of level bits (bit 4 kg + r):
 // this head's level is 1 / is 2, and -- OR-ed over the heads of the group -- the mid / last plane row of the
-// channel is fetched.  grid (B * Hkv), 64 threads.
+// channel is fetched.  One wave per (batch, KV head): mfma_k_prepare (akv_step.h), run by this
+// kernel (grid (B * Hkv), 64 threads) or, with per-sequence lengths, by extra workgroups of the step's first kernel.
 template <int D, bool REF>
 __global__ __launch_bounds__(64) void mfma_k_prepare_kernel(const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q,
                                                            const unsigned short *__restrict__ k_new, u32 *__restrict__ prep,
                                                            uint8_t *__restrict__ levels_out, StepGeom geo) {
-    constexpr int KG = D / 16;
-    static_assert(4 * KG <= 32, "the level masks are 32 bits wide");
-    const int lane = threadIdx.x;
-    const int bh_kv = blockIdx.x, b = bh_kv / geo.Hkv, hkv = bh_kv - b * geo.Hkv;
-    const int G = geo.G;
-    const int64_t bh0 = (int64_t)b * geo.Hq + hkv * G;
-    const int j = lane & 15, kq = lane >> 4;
-    const bool head = j < G;
-    u32 *out = prep + ((int64_t)bh_kv * 64 + lane) * (2 * KG + 4);
-    u32 lv1 = 0, lv2 = 0;
-    u32 esum[KG][4];
-    u32 mx = 0;
-#pragma unroll
-    for (int kg = 0; kg < KG; ++kg) {
-        u32 qb[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int c = 16 * kg + 4 * r + kq;
-            qb[r] = head ? (u32)q[(bh0 + j) * D + c] : 0u;
-            // column max including the token appended by this step
-            const u32 cm = max((u32)kcm[(int64_t)bh_kv * D + c], exp_field(k_new[(int64_t)bh_kv * D + c]));
-            esum[kg][r] = (exp_field(qb[r]) + cm) & 0xffu;
-            mx = max(mx, esum[kg][r]);
-        }
-        out[2 * kg] = qb[0] | (qb[1] << 16);
-        out[2 * kg + 1] = qb[2] | (qb[3] << 16);
-    }
-    mx = max(mx, (u32)__shfl_xor((int)mx, 16, 64));
-    mx = max(mx, (u32)__shfl_xor((int)mx, 32, 64));
-#pragma unroll
-    for (int kg = 0; kg < KG; ++kg)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)esum[kg][r]);
-            if (head) {
-                lv1 |= (lv == 1 ? 1u : 0u) << (4 * kg + r);
-                lv2 |= (lv == 2 ? 1u : 0u) << (4 * kg + r);
-                if (levels_out != nullptr) levels_out[(bh0 + j) * D + 16 * kg + 4 * r + kq] = (uint8_t)lv;
-            }
-        }
-    // a plane row is fetched if any head of the group reads it: OR over the 16 lanes that share kq
-    u32 need_mid = head ? ~lv2 : 0u;
-    u32 need_last = head ? ~(lv1 | lv2) : 0u;
-#pragma unroll
-    for (int m = 1; m < 16; m <<= 1) {
-        need_mid |= (u32)__shfl_xor((int)need_mid, m, 64);
-        need_last |= (u32)__shfl_xor((int)need_last, m, 64);
-    }
-    out[2 * KG] = lv1;
-    out[2 * KG + 1] = lv2;
-    out[2 * KG + 2] = need_mid;
-    out[2 * KG + 3] = need_last;
+    mfma_k_prepare<D, REF>(kcm, q, k_new, prep, levels_out, geo, (int)blockIdx.x);
 }
 
 // The same for a tile whose rows are all used at level 2 by every head (only the high bytes were fetched): the low
@@ -364,7 +314,7 @@ template <int D>
 int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *kcm,
                        const unsigned short *q, const unsigned short *k_new, unsigned short *scores,
                        uint8_t *levels_out, u32 *prep, const StepGeom &geo, int B, int n_blocks, bool ref, float scale,
-                       hipStream_t st, PassShape *shape_only) {
+                       hipStream_t st, PassShape *shape_only, bool prepared) {
     // Slots per lane.  K blocks of 256 tokens: 16, so that the 16 lanes of a token-set group read a channel's whole row
     // of a block (256 B of first_8, 128 B of a nibble plane); measured at batch 32, 32 over 8 heads, lengths 2048..8192:
     // 62.5 us, against 78 with 8 slots per lane (half rows) and 68.8 with blocks of 64 tokens and 8 slots.  Three tiles
@@ -385,12 +335,14 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
         set_error("decode_step: score rows of %lld bytes exceed the 2 GiB the grouped K pass addresses", (long long)scores_bytes);
         return AKV_ERR_INVALID;
     }
-    if (ref)
-        hipLaunchKernelGGL((mfma_k_prepare_kernel<D, true>), dim3(B * geo.Hkv), dim3(64), 0, st, kcm, q, k_new, prep, levels_out, geo);
-    else
-        hipLaunchKernelGGL((mfma_k_prepare_kernel<D, false>), dim3(B * geo.Hkv), dim3(64), 0, st, kcm, q, k_new, prep, levels_out, geo);
-    int rc = check_launch("decode_step(mfma k_prepare)");
-    if (rc != AKV_OK) return rc;
+    if (!prepared) {
+        if (ref)
+            hipLaunchKernelGGL((mfma_k_prepare_kernel<D, true>), dim3(B * geo.Hkv), dim3(64), 0, st, kcm, q, k_new, prep, levels_out, geo);
+        else
+            hipLaunchKernelGGL((mfma_k_prepare_kernel<D, false>), dim3(B * geo.Hkv), dim3(64), 0, st, kcm, q, k_new, prep, levels_out, geo);
+        int rc = check_launch("decode_step(mfma k_prepare)");
+        if (rc != AKV_OK) return rc;
+    }
     dim3 grid((n_tasks + 4 * tpw - 1) / (4 * tpw), geo.Hkv, B);
 #define AKV_MK(RF, SLL, AH, KSH)                                                                                     \
     hipLaunchKernelGGL((mfma_k_pass_kernel<D, RF, SLL, AH, KSH>), grid, dim3(256), 0, st, f8, m4, l4, prep, scores, geo, \
@@ -656,7 +608,7 @@ int launch_mfma_v_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
 #define AKV_INST_K(DD)                                                                                                \
     template int launch_mfma_k_pass<DD>(const uint8_t *, const uint8_t *, const uint8_t *, const uint8_t *,           \
                                         const unsigned short *, const unsigned short *, unsigned short *, uint8_t *, \
-                                        u32 *, const StepGeom &, int, int, bool, float, hipStream_t, PassShape *);
+                                        u32 *, const StepGeom &, int, int, bool, float, hipStream_t, PassShape *, bool);
 #define AKV_INST_V(DD)                                                                                                \
     template VPlan mfma_v_plan<DD>(int, int, int);                                                                    \
     template int launch_mfma_v_pass<DD>(const uint8_t *, const uint8_t *, const uint8_t *, const unsigned short *,    \

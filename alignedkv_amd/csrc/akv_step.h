@@ -89,7 +89,7 @@ template <int D>
 int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *kcm,
                        const unsigned short *q, const unsigned short *k_new, unsigned short *scores,
                        uint8_t *levels_out, u32 *prep, const StepGeom &geo, int B, int n_blocks, bool ref, float scale,
-                       hipStream_t st, PassShape *shape_only = nullptr);
+                       hipStream_t st, PassShape *shape_only = nullptr, bool prepared = false);
 template <int D>
 VPlan mfma_v_plan(int B, int Hkv, int n_tokens);
 template <int D>
@@ -98,5 +98,68 @@ int launch_mfma_v_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
                        const StepGeom &geo, int B, const VPlan &p, bool ref, hipStream_t st);
 // words of set-up data per (batch, KV head) that launch_mfma_k_pass needs in `prep`
 inline size_t mfma_k_prep_words(int D) { return (size_t)64 * (2 * (D / 16) + 4); }
+
+// Set-up of the matrix-core K pass for (batch, KV head) bh_kv, by one wave: lane (j, kq) = (l % 16, l / 16) takes query
+// head j of the group at the channels 16 kg + 4 r + kq and leaves, for the K-pass lane of the same index, 2 KG words
+// of q (packed fp16 pairs r = 0,1 / 2,3 per channel group) and 4 words of level bits (bit 4 kg + r): this head's
+// level is 1 / is 2, and -- OR-ed over the heads of the group -- the mid / last plane row of the channel is fetched.
+// kcm may or may not hold this step's token yet: its exponent is folded in here either way.
+template <int D, bool REF>
+__device__ __forceinline__ void mfma_k_prepare(const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q,
+                                               const unsigned short *__restrict__ k_new, u32 *__restrict__ prep,
+                                               uint8_t *__restrict__ levels_out, const StepGeom &geo, int bh_kv) {
+    constexpr int KG = D / 16;
+    static_assert(4 * KG <= 32, "the level masks are 32 bits wide");
+    const int lane = threadIdx.x & 63;
+    const int b = bh_kv / geo.Hkv, hkv = bh_kv - b * geo.Hkv;
+    const int G = geo.G;
+    const int64_t bh0 = (int64_t)b * geo.Hq + hkv * G;
+    const int j = lane & 15, kq = lane >> 4;
+    const bool head = j < G;
+    u32 *out = prep + ((int64_t)bh_kv * 64 + lane) * (2 * KG + 4);
+    u32 lv1 = 0, lv2 = 0;
+    u32 esum[KG][4];
+    u32 mx = 0;
+#pragma unroll
+    for (int kg = 0; kg < KG; ++kg) {
+        u32 qb[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int c = 16 * kg + 4 * r + kq;
+            qb[r] = head ? (u32)q[(bh0 + j) * D + c] : 0u;
+            // column max including the token appended by this step
+            const u32 cm = max((u32)kcm[(int64_t)bh_kv * D + c], exp_field(k_new[(int64_t)bh_kv * D + c]));
+            esum[kg][r] = (exp_field(qb[r]) + cm) & 0xffu;
+            mx = max(mx, esum[kg][r]);
+        }
+        out[2 * kg] = qb[0] | (qb[1] << 16);
+        out[2 * kg + 1] = qb[2] | (qb[3] << 16);
+    }
+    mx = max(mx, (u32)__shfl_xor((int)mx, 16, 64));
+    mx = max(mx, (u32)__shfl_xor((int)mx, 32, 64));
+#pragma unroll
+    for (int kg = 0; kg < KG; ++kg)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)esum[kg][r]);
+            if (head) {
+                lv1 |= (lv == 1 ? 1u : 0u) << (4 * kg + r);
+                lv2 |= (lv == 2 ? 1u : 0u) << (4 * kg + r);
+                if (levels_out != nullptr) levels_out[(bh0 + j) * D + 16 * kg + 4 * r + kq] = (uint8_t)lv;
+            }
+        }
+    // a plane row is fetched if any head of the group reads it: OR over the 16 lanes that share kq
+    u32 need_mid = head ? ~lv2 : 0u;
+    u32 need_last = head ? ~(lv1 | lv2) : 0u;
+#pragma unroll
+    for (int m = 1; m < 16; m <<= 1) {
+        need_mid |= (u32)__shfl_xor((int)need_mid, m, 64);
+        need_last |= (u32)__shfl_xor((int)need_last, m, 64);
+    }
+    out[2 * KG] = lv1;
+    out[2 * KG + 1] = lv2;
+    out[2 * KG + 2] = need_mid;
+    out[2 * KG + 3] = need_last;
+}
 
 }  // namespace akv
