@@ -409,39 +409,50 @@ __device__ __forceinline__ i16x2 wrap_diff16(u16x2 a, u32 b) {
     return d.s;
 }
 
+// a2: amin << 10 in both halves; lanes without a head pass 0x0800 and probabilities of zero (no token below level 2).
 template <bool REF>
-__device__ __forceinline__ void v_macro_ops(VMacroOps &o, const u32x2 *p, unsigned char amin, bool head) {
+__device__ __forceinline__ void v_macro_ops(VMacroOps &o, const u32x2 *p, u16x2 a2, bool head) {
     u32 mid = 0, last = 0;
-    o.lv1 = 0;
-    o.lv2 = head ? 0xffffu : 0u;
 #pragma unroll
-    for (int sidx = 0; sidx < 4; ++sidx) o.p[sidx] = head ? p[sidx] : (u32x2){0u, 0u};
+    for (int sidx = 0; sidx < 4; ++sidx) o.p[sidx] = p[sidx];
     if (REF) {
         mid = last = head ? 0xffffu : 0u;
-        o.lv2 = 0;
-    } else if (head) {
+    } else {
         // 16-bit differences of two tokens at a time (they wrap like the reference's `short` arithmetic,
         // extension/csrc/V_cache.cu:195-197,211); level < 2 <=> diff < 0x0800, level 0 <=> diff < 0x0400, read off the
         // sign of a saturating subtraction.  Word w = 2 s + (0: tokens 0,1 | 1: tokens 2,3 of step s) leaves the flag
         // of its first token in bit 2 w and of its second in bit 16 + 2 w.
-        const unsigned short a16 = (unsigned short)((unsigned)amin << 10);
-        const u16x2 a2 = {a16, a16};
         const i16x2 c8 = {0x0800, 0x0800}, c4 = {0x0400, 0x0400};
+        i16x2 d[8];
+        u32 t8[8], any8 = 0;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) {
+            d[w] = wrap_diff16(a2, (w & 1) ? p[w >> 1].y : p[w >> 1].x);
+            union { i16x2 v; u32 u; } t;
+            t.v = __builtin_elementwise_sub_sat(d[w], c8);
+            t8[w] = t.u;
+            any8 |= t.u;
+        }
+        // nearly always no lane of the wave has a token below level 2 in these 64 tokens: nothing else to work out
+        if (__builtin_amdgcn_ballot_w64((any8 & 0x80008000u) != 0u) == 0ull) {
+            o.lv1 = 0;
+            o.lv2 = 0xffffu;
+            o.need = 0;
+            return;
+        }
         u32 acc8 = 0, acc4 = 0;
 #pragma unroll
         for (int w = 0; w < 8; ++w) {
-            const i16x2 d = wrap_diff16(a2, (w & 1) ? p[w >> 1].y : p[w >> 1].x);
-            union { i16x2 v; u32 u; } t8, t4;
-            t8.v = __builtin_elementwise_sub_sat(d, c8);
-            t4.v = __builtin_elementwise_sub_sat(d, c4);
-            acc8 |= ((t8.u >> 15) & 0x00010001u) << (2 * w);
+            union { i16x2 v; u32 u; } t4;
+            t4.v = __builtin_elementwise_sub_sat(d[w], c4);
+            acc8 |= ((t8[w] >> 15) & 0x00010001u) << (2 * w);
             acc4 |= ((t4.u >> 15) & 0x00010001u) << (2 * w);
         }
         mid = (acc8 & 0xffffu) | ((acc8 >> 16) << 1);
         last = (acc4 & 0xffffu) | ((acc4 >> 16) << 1);
-        o.lv1 = mid & ~last;
-        o.lv2 = ~mid & 0xffffu;
     }
+    o.lv1 = mid & ~last;
+    o.lv2 = ~mid & 0xffffu;
     // union over the heads: OR over the 16 lanes of the lane group (one DPP row)
     u32 both = mid | (last << 16);
     both |= (u32)__builtin_amdgcn_update_dpp(0, (int)both, 0x128, 0xf, 0xf, false);   // row_ror:8
@@ -485,12 +496,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     const bool head = j < G;
     const unsigned char amin = (REF || !head) ? 0 : amin_u8[bh0 + j];
     if (!REF && head && amin_out != nullptr && chunk == 0 && wave == 0 && kq == 0) amin_out[bh0 + j] = amin;
+    // what the levels are measured against; lanes without a head read probabilities of zero, for which this value says level 2
+    const unsigned short a16 = head ? (unsigned short)((unsigned)amin << 10) : (unsigned short)0x0800;
+    const u16x2 a2 = {a16, a16};
     const int lane_p = (int)((bh0 + (head ? j : 0)) * geo.row_stride + 4 * kq) * 2;
     const int lane_h = (4 * kq) * D + (lane & 15) * CPP, lane_m = (4 * kq) * (D / 2) + (lane & 15) * (CPP / 2);
 
     // probabilities of the lane's head for a macro step: 4 steps x 4 tokens (base + 16 s + 4 kq + r)
     auto load_probs = [&](u32x2 *dst, int base) {
-        const int o = base < t_end ? lane_p + base * 2 : kSkip;
+        const int o = (base < t_end && head) ? lane_p + base * 2 : kSkip;
 #pragma unroll
         for (int sidx = 0; sidx < 4; ++sidx) dst[sidx] = __builtin_amdgcn_raw_buffer_load_b64(rP, o + 32 * sidx, 0, 0);
     };
@@ -514,7 +528,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
         u32x2 pc[4];
         load_probs(pc, t_begin);
         load_probs(pn, t_begin + MACRO);
-        v_macro_ops<REF>(oc, pc, amin, head);
+        v_macro_ops<REF>(oc, pc, a2, head);
     }
     KTaskTile<CPP> t[4];
 #pragma unroll
@@ -522,7 +536,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     __builtin_amdgcn_sched_barrier(0);
     for (int base = t_begin; base < t_end; base += MACRO) {
         load_probs(pnn, base + 2 * MACRO);
-        v_macro_ops<REF>(on, pn, amin, head);     // levels and fetch masks of the next macro step
+        v_macro_ops<REF>(on, pn, a2, head);     // levels and fetch masks of the next macro step
 #pragma unroll
         for (int si = 0; si < 4; ++si) {
             if (si == 0) issue(t[3], oc, base, 3);
