@@ -99,10 +99,22 @@ def test_gqa_reads_each_kv_chunk_for_all_query_heads_consistently():
     assert (out_g.float() - out_m.float()).abs().max().item() <= 1e-3
 
 
-def test_config3_full_size_against_c_oracle():
+def _as_64_token_blocks(plane, kb):
+    """K plane [1, H, NB, D, w * kb / 64 ...] laid out in blocks of kb tokens -> the same bytes in blocks of 64 tokens."""
+    if kb == 64:
+        return plane
+    one, H, NB, D, row = plane.shape
+    sub = kb // 64
+    return np.ascontiguousarray(plane.reshape(one, H, NB, D, sub, row // sub).transpose(0, 1, 2, 4, 3, 5)).reshape(
+        one, H, NB * sub, D, row // sub)
+
+
+@pytest.mark.parametrize("k_block", [64, 256])
+def test_config3_full_size_against_c_oracle(k_block):
     """C3: 32 query heads over 8 KV heads, head_dim 128, batch 32, lengths uniform in [2048, 8192], K with 4
     outlier channels per KV head x10, V ~ N(0, 0.5).  Every sequence is checked against the C restatement of
-    the ops run on its own planes with the KV heads repeated."""
+    the ops run on its own planes with the KV heads repeated (K planes in blocks of 256 tokens are first rearranged
+    into the blocks of 64 the restatement works on)."""
     from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
     from tests.common import oracle_decode_step_c
     B, Hq, Hkv, D, cb = 32, 32, 8, 128, 64
@@ -110,7 +122,7 @@ def test_config3_full_size_against_c_oracle():
     Lmax = 8192 + cb
     lens = np.random.default_rng(3).integers(2048, 8193, B)
     lens[:4] = [2048, 8191, 4159, 8192]          # block-aligned, two that complete a block with the append, the maximum
-    cache = RaggedGQACache(1, B, Lmax, Hq, Hkv, D)
+    cache = RaggedGQACache(1, B, Lmax, Hq, Hkv, D, k_block=k_block)
     cache.record_levels = True
     gen = torch.Generator(device="cuda").manual_seed(33)
     tails = []
@@ -141,7 +153,7 @@ def test_config3_full_size_against_c_oracle():
         R = L // cb * cb
         rk = np.concatenate([tails[b][0], knh[b:b + 1]], axis=1)
         rv = np.concatenate([tails[b][1], vnh[b:b + 1]], axis=1)
-        kpl = [p[b:b + 1, :, :R // cb].cpu().numpy() for p in cache.k_planes[0]]
+        kpl = [_as_64_token_blocks(p[b:b + 1].cpu().numpy(), k_block)[:, :, :R // cb] for p in cache.k_planes[0]]
         vpl = [p[b:b + 1, :, :R].cpu().numpy() for p in cache.v_planes[0]]
         if rk.shape[1] == cb:
             # the append completed a block: what the step wrote into the planes must be the NumPy split of it
