@@ -73,7 +73,8 @@ def test_gqa_ragged_step_matches_per_sequence_oracle(B, Hq, Hkv, lens, steps, D)
         assert np.array_equal(cache.k_colmax[0][b, 0].cpu().numpy(), oc.k_colmax[0, 0, ::G])
 
 
-def test_gqa_reads_each_kv_chunk_for_all_query_heads_consistently():
+@pytest.mark.parametrize("k_block", [64, 256])
+def test_gqa_reads_each_kv_chunk_for_all_query_heads_consistently(k_block):
     """Uniform lengths through the same entry point (seq_lens=None): grouped heads against the multi-head
     cache fed with repeated keys and values."""
     from types import SimpleNamespace
@@ -84,7 +85,7 @@ def test_gqa_reads_each_kv_chunk_for_all_query_heads_consistently():
     G = Hq // Hkv
     q, k, v = make_qkv(B, L + 1, Hkv, D, seed=5)
     q = np.random.default_rng(1).standard_normal((B, 1, Hq, D)).astype(np.float16)
-    g = RaggedGQACache(1, B, L + 64, Hq, Hkv, D)
+    g = RaggedGQACache(1, B, L + 64, Hq, Hkv, D, k_block=k_block)
     for b in range(B):
         g.prefill(0, b, dev(k[b:b + 1, :L]), dev(v[b:b + 1, :L]))
     out_g = g.decode(0, dev(q), dev(k[:, L:]), dev(v[:, L:]))
@@ -107,6 +108,37 @@ def _as_64_token_blocks(plane, kb):
     sub = kb // 64
     return np.ascontiguousarray(plane.reshape(one, H, NB, D, sub, row // sub).transpose(0, 1, 2, 4, 3, 5)).reshape(
         one, H, NB * sub, D, row // sub)
+
+
+@pytest.mark.parametrize("k_block", [64, 256])
+def test_grouped_heads_with_one_length_for_all_sequences_match_the_per_sequence_call(k_block):
+    """seq_lens = None (every sequence has cur_len tokens: the token is appended by the middle stage, a full rest buffer
+    flushed by the save kernels, no task maps) against the same steps with a length per sequence on the device."""
+    from alignedkv_amd.extension._plane_cache import column_block
+    from alignedkv_amd.extension.KV_cache_cpp_extention import cuda_module
+    from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
+    B, Hq, Hkv, D, L, steps = 2, 8, 2, 128, 700, 70
+    _, k, v = make_qkv(B, L + steps, Hkv, D, seed=11, n_outliers=4)
+    rng = np.random.default_rng(2)
+    caches = [RaggedGQACache(1, B, L + steps + 64, Hq, Hkv, D, k_block=k_block) for _ in range(2)]
+    for c in caches:
+        for b in range(B):
+            c.prefill(0, b, dev(k[b:b + 1, :L]), dev(v[b:b + 1, :L]))
+    u = caches[1]
+    for t in range(L, L + steps):
+        q = dev(rng.standard_normal((B, 1, Hq, D)).astype(np.float16))
+        kn, vn = dev(k[:, t:t + 1]), dev(v[:, t:t + 1])
+        want = caches[0].decode(0, q, kn, vn)
+        out = torch.empty_like(q)
+        cuda_module.decode_step_gqa(u.k_planes[0], u.v_planes[0], u.k_colmax[0], u.v_colmax[0], u.restk[0].view(torch.uint8),
+                                    u.restv[0].view(torch.uint8), q.view(torch.uint8), kn.view(torch.uint8),
+                                    vn.view(torch.uint8), None, out.view(torch.uint8), u.scores.view(torch.uint8),
+                                    u.probs.view(torch.uint8), B, Hq, Hkv, u.n_max_blocks, u.max_seq_len, D, column_block, 32,
+                                    t, None, False, None, None, None, k_block=k_block)
+        assert torch.equal(out, want), f"step at {t} tokens"
+    for a, b_ in zip(caches[0].k_planes[0] + caches[0].v_planes[0], u.k_planes[0] + u.v_planes[0]):
+        assert torch.equal(a, b_)
+    assert torch.equal(caches[0].restk[0], u.restk[0]) and torch.equal(caches[0].k_colmax[0], u.k_colmax[0])
 
 
 @pytest.mark.parametrize("k_block", [64, 256])
