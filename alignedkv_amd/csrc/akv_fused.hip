@@ -374,19 +374,19 @@ __global__ __launch_bounds__(256) void fused_k_pass256_kernel(
                          need_mid, need_last, scores + (int64_t)bh * geo.row_stride, R, scale);
 }
 
-// The same pass for short caches: one workgroup per 256-token block, its four waves take a quarter of the channels each
-// and add their partial scores through LDS.  With a whole block per wave a cache of 1024 tokens x 32 heads gives the
-// pass 128 waves of 48 KiB each (8.1 us per step at batch 1); split like this it has 512 waves of 12 KiB, all loads
-// of a wave in flight at once.  grid (n_kblocks, H, B), 256 threads.
-template <int D, bool REF>
-__global__ __launch_bounds__(256) void fused_k_pass256_split_kernel(
+// The same pass with one workgroup per 256-token block: its four waves take a quarter of the channels each, request all
+// their rows at once (12 KiB per wave, five waves per SIMD) and add their partial scores through LDS.  A cache of
+// 1024 tokens x 32 heads gives this kernel 512 waves where a block per wave gives 128 waves of 48 KiB each; long caches
+// gain from the bytes in flight (see run_step).  grid (n_kblocks, H, B), 256 threads.
+template <int D, bool REF, int NWV>
+__global__ __launch_bounds__(64 * NWV) void fused_k_pass256_split_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
     unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, StepGeom geo, float scale) {
     constexpr int KB = 256;
     constexpr int NG = D / 4;      // load groups of 4 channels
     constexpr int HG = 4;          // groups per half tile
-    constexpr int GW = NG / 4;     // groups per wave
+    constexpr int GW = NG / NWV;   // groups per wave
     constexpr int NT = GW / HG;    // half tiles per wave
     static_assert(GW % HG == 0 && NG <= 32, "head_dim 64 or 128");
     const int lane = threadIdx.x & 63, wave = wave_index();
@@ -407,8 +407,8 @@ __global__ __launch_bounds__(256) void fused_k_pass256_split_kernel(
     for (int i = 0; i < NT; ++i) k256_issue_h<D, HG>(t[i], rH, blk, g_first + HG * i);
     __builtin_amdgcn_sched_barrier(0);
     __shared__ u32 staged[D];      // [channel]: q bits | exponent sum << 16
-    __shared__ float part[4][KB];  // [wave][slot]: partial scores
-    for (int c = threadIdx.x; c < D; c += 256) {
+    __shared__ float part[NWV][KB];  // [wave][slot]: partial scores
+    for (int c = threadIdx.x; c < D; c += 64 * NWV) {
         const u32 qb = q[(int64_t)bh * D + c];
         // column max including the token appended by this step
         const u32 cm = max((u32)kcm[(int64_t)bh * D + c], exp_field(k_new[(int64_t)bh * D + c]));
@@ -447,11 +447,15 @@ __global__ __launch_bounds__(256) void fused_k_pass256_split_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) part[wave][slot + i] = acc[i];
     __syncthreads();
-    const int token = blk * KB + threadIdx.x;
-    if (token < R) {
-        const float sum = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
-        // device scope: the workgroup that runs the softmax for this (batch, head) may sit on another XCD
-        store_u16_device(make_rsrc(scores + (int64_t)bh * geo.row_stride, (u32)R * 2), token * 2, float_to_half_bits(sum * scale));
+    for (int sl = threadIdx.x; sl < KB; sl += 64 * NWV) {
+        const int token = blk * KB + sl;
+        if (token < R) {
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NWV; ++w) sum += part[w][sl];
+            // device scope: the workgroup that runs the softmax for this (batch, head) may sit on another XCD
+            store_u16_device(make_rsrc(scores + (int64_t)bh * geo.row_stride, (u32)R * 2), token * 2, float_to_half_bits(sum * scale));
+        }
     }
 }
 
@@ -1023,10 +1027,10 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         return AKV_ERR_INVALID;
     }
     const int n_kblocks = (R + kb - 1) / kb;    // K plane blocks that hold tokens (the last one may be partly filled)
-    // short caches: a block per workgroup instead of per wave while that still fits the machine at once (16 waves per
-    // compute unit)
-    bool k_split = kb == 256 && geo.G == 1 && D <= 128 && !ragged && compute_units() > 0 &&
-                   (int64_t)B * Hq * n_kblocks <= 4 * compute_units();
+    // 256-token K blocks, one query head per KV head: a block per workgroup, a quarter of the channels per wave (all of a
+    // wave's loads in flight at once).  Measured against a block per wave: batch 1 x 1024 tokens 5.2 vs 8.1 us, 8 x 4096
+    // 33.6 vs 33.9, 4 x 32768 146.7 vs 155.2 (0.85 instead of 0.80 of HBM peak).
+    bool k_split = kb == 256 && geo.G == 1 && D <= 128;
     { AKV_TUNE("AKV_TUNE_K_SPLIT", v); if (has_v) k_split = k_split && v != 0; }
     const int bpw = k_split ? 1 : (kb == 256 ? k256_blocks_per_wave(B, Hq, n_kblocks) : k_blocks_per_wave(B, Hq, n_blocks));
     bool matrix_v = matrix;
@@ -1119,10 +1123,10 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         dim3 grid(ks.grid_x, ks.grid_y, B);
         if constexpr (D <= 128) {
             if (ref)
-                hipLaunchKernelGGL((fused_k_pass256_split_kernel<D, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
+                hipLaunchKernelGGL((fused_k_pass256_split_kernel<D, true, 4>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
                                    k_levels_out, geo_k, scale);
             else
-                hipLaunchKernelGGL((fused_k_pass256_split_kernel<D, false>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
+                hipLaunchKernelGGL((fused_k_pass256_split_kernel<D, false, 4>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
                                    k_levels_out, geo_k, scale);
         }
         int rc = check_launch("decode_step(k_pass256 split)");

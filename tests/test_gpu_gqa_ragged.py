@@ -21,7 +21,7 @@ def dev(a):
                                                    (2, 40, 2, [200, 330], 2, 128),
                                                    # K plane blocks of 256 tokens (negative head_dim marks them)
                                                    (3, 8, 2, [130, 64, 7], 70, -128), (2, 16, 1, [700, 255], 66, -128),
-                                                   (2, 12, 4, [260, 900], 3, -64)])
+                                                   (2, 12, 4, [260, 900], 3, -64), (2, 4, 4, [200, 600], 70, -128)])
 def test_gqa_ragged_step_matches_per_sequence_oracle(B, Hq, Hkv, lens, steps, D):
     from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
     kb = 256 if D < 0 else 64
