@@ -132,6 +132,35 @@ __device__ __forceinline__ void k_score_blocks(KHalfTile<D / 32> &ta, const uint
     }
 }
 
+// One block with everything in flight at once: the caller has requested the high bytes of all its channels
+// (k_issue_half_h<D, D / 16>) before working out q and the levels; here the nibble rows follow, then the arithmetic.
+// 16 KiB per wave and no loop: for kernels that give every block a wave of its own.
+template <int D>
+__device__ __forceinline__ void k_score_block_whole(KHalfTile<D / 16> &t, const uint8_t *m4, const uint8_t *l4, int n_blocks,
+                                                    int blk, const float *qf, u32 need_mid, u32 need_last,
+                                                    unsigned short *s_row, float scale) {
+    constexpr int CB = 64;
+    constexpr int NG = D / 16;
+    const int lane = threadIdx.x & 63;
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_blocks * (D * CB / 2));
+    const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_blocks * (D * CB / 2));
+    const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)n_blocks * CB * 2);
+    const int slot = (lane & 3) * 16 + ((lane & 32) ? 8 : 0) + ((lane & 16) ? 4 : 0) + ((lane & 8) ? 2 : 0) +
+                     ((lane & 4) ? 1 : 0);
+    k_issue_half_ml<D, NG>(t, rM, rL, blk, 0, need_mid, need_last);
+    __builtin_amdgcn_sched_barrier(0);
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    k_compute_half<NG>(acc, t, 0, qf, need_mid, need_last);
+    reduce_scatter_step<16>(acc, 32);
+    reduce_scatter_step<8>(acc, 16);
+    reduce_scatter_step<4>(acc, 8);
+    reduce_scatter_step<2>(acc, 4);
+    // device scope: the workgroup that runs the softmax for this (batch, head) may sit on another XCD
+    store_u16_device(rS, (blk * CB + slot) * 2, float_to_half_bits(acc[0] * scale));
+}
+
 // ------------------------------------------------------------------------------------------------
 // V: one wave accumulates tokens [t_begin, t_end) of one (batch, head) into acc[16].
 //   f8/m4/l4 point at token 0 of this (batch, head); n_tokens bounds the buffer resources.
