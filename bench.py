@@ -429,7 +429,7 @@ def main():
         "k_block": a.k_block, "other_k_block_us": other,
         "dense_in_planes_us": round(sec_ref * 1e6, 2),
         "speedup_vs_dense_in_planes": round(sec_ref / sec, 3),
-        "roofline": {"kernel": "fused_k_pass_kernel<%d,false,true>" % D if a.k_block == 64 else "fused_k_pass256_split_kernel<%d,false,4>" % D, "bound": "hbm", "achieved": round(achieved, 1),
+        "roofline": {"kernel": ("fused_k_pass_kernel<%d,false,true>" % D if D <= 128 else "fused_k_pass_kernel<%d,false>" % D) if a.k_block == 64 else "fused_k_pass256_split_kernel<%d,false,4>" % D, "bound": "hbm", "achieved": round(achieved, 1),
                      "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_K_PASS_TRAFFIC.get((B, H, D, L, a.k_kind, a.k_block)), "algorithmic_bytes_per_launch": int(k_pass_bytes),
                      "avg_launch_us": round(ph[0], 2), "event_pair_overhead_us": round(event_pair_us, 2)},
