@@ -182,7 +182,9 @@ __global__ void k_save_token_kernel(uint8_t *__restrict__ first_8, uint8_t *__re
 // k_cache_compute, tuned: d_block == 64
 // grid (ceil(n_blocks / (4*blocks_per_wave)), H, B), 256 threads (4 waves).
 // ------------------------------------------------------------------------------------------------
-template <int D, bool REF>
+// WHOLE (head_dim 64 and 128, blocks_per_wave == 1): a wave requests all rows of its block at once instead of walking
+// it in double-buffered half tiles (k_score_block_whole).
+template <int D, bool REF, bool WHOLE = false>
 __global__ __launch_bounds__(256) void k_compute_cb64_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const uint8_t *__restrict__ sum_u8, const uint8_t *__restrict__ max_u8, const unsigned short *__restrict__ q,
@@ -198,8 +200,13 @@ __global__ __launch_bounds__(256) void k_compute_cb64_kernel(
     const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
 
     const int64_t plane_off = (int64_t)bh * n_max_blocks * (D * (CB / 2));
-    KHalfTile<D / 32> ta;
-    k_prefetch_first<D>(ta, first_8 + plane_off * 2, n_blocks, first_blk);
+    KHalfTile<WHOLE ? D / 16 : D / 32> ta;
+    if constexpr (WHOLE) {
+        k_issue_half_h<D, D / 16>(ta, make_rsrc(first_8 + plane_off * 2, (u32)n_blocks * (D * CB)), first_blk, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    } else {
+        k_prefetch_first<D>(ta, first_8 + plane_off * 2, n_blocks, first_blk);
+    }
     // per-lane channel data: channel of group g is g*16 + lane/4
     float qf[NG];
     u32 need_mid = 0, need_last = 0;
@@ -214,8 +221,13 @@ __global__ __launch_bounds__(256) void k_compute_cb64_kernel(
         if (levels_out != nullptr && blockIdx.x == 0 && wave == 0 && (lane & 3) == 0)
             levels_out[(int64_t)bh * D + c] = (uint8_t)lv;
     }
-    k_score_blocks<D>(ta, first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
-                      need_mid, need_last, s + (int64_t)bh * ((int64_t)(n_blocks + 1) * CB), scale);
+    if constexpr (WHOLE) {
+        k_score_block_whole<D>(ta, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, qf, need_mid, need_last,
+                               s + (int64_t)bh * ((int64_t)(n_blocks + 1) * CB), scale);
+    } else {
+        k_score_blocks<D>(ta, first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
+                          need_mid, need_last, s + (int64_t)bh * ((int64_t)(n_blocks + 1) * CB), scale);
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -294,11 +306,19 @@ template <int D, bool REF>
 static void launch_k_cb64(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, const uint8_t *sum_u8,
                           const uint8_t *max_u8, const uint8_t *q, uint8_t *s, uint8_t *levels, int B, int H,
                           int n_blocks, int n_max_blocks, float scale, hipStream_t st) {
-    const int bpw = k_blocks_per_wave(B, H, n_blocks);
-    dim3 grid((n_blocks + 4 * bpw - 1) / (4 * bpw), H, B);
-    hipLaunchKernelGGL((k_compute_cb64_kernel<D, REF>), grid, dim3(256), 0, st, f8, m4, l4, sum_u8, max_u8,
-                       reinterpret_cast<const unsigned short *>(q), reinterpret_cast<unsigned short *>(s), levels,
-                       n_blocks, n_max_blocks, H, bpw, scale);
+    if constexpr (D <= 128) {
+        // a block per wave, all its rows in flight at once (as in the fused step)
+        dim3 grid((n_blocks + 3) / 4, H, B);
+        hipLaunchKernelGGL((k_compute_cb64_kernel<D, REF, true>), grid, dim3(256), 0, st, f8, m4, l4, sum_u8, max_u8,
+                           reinterpret_cast<const unsigned short *>(q), reinterpret_cast<unsigned short *>(s), levels,
+                           n_blocks, n_max_blocks, H, 1, scale);
+    } else {
+        const int bpw = k_blocks_per_wave(B, H, n_blocks);
+        dim3 grid((n_blocks + 4 * bpw - 1) / (4 * bpw), H, B);
+        hipLaunchKernelGGL((k_compute_cb64_kernel<D, REF>), grid, dim3(256), 0, st, f8, m4, l4, sum_u8, max_u8,
+                           reinterpret_cast<const unsigned short *>(q), reinterpret_cast<unsigned short *>(s), levels,
+                           n_blocks, n_max_blocks, H, bpw, scale);
+    }
 }
 
 template <int D, bool REF>
