@@ -1161,23 +1161,20 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
     } else if (n_blocks > 0) {
         dim3 grid(ks.grid_x, ks.grid_y, B);
+#define AKV_KP(RF, WH)                                                                                                 \
+    hipLaunchKernelGGL((fused_k_pass_kernel<D, RF, WH>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,   \
+                       k_levels_out, geo_k, bpw, scale)
+        bool launched = false;
         if constexpr (D <= 128) {
             if (k_whole) {
-                if (ref)
-                    hipLaunchKernelGGL((fused_k_pass_kernel<D, true, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                                       k_levels_out, geo_k, bpw, scale);
-                else
-                    hipLaunchKernelGGL((fused_k_pass_kernel<D, false, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                                       k_levels_out, geo_k, bpw, scale);
+                if (ref) AKV_KP(true, true); else AKV_KP(false, true);
+                launched = true;
             }
         }
-        if (k_whole) {
-        } else if (ref)
-            hipLaunchKernelGGL((fused_k_pass_kernel<D, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                               k_levels_out, geo_k, bpw, scale);
-        else
-            hipLaunchKernelGGL((fused_k_pass_kernel<D, false>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                               k_levels_out, geo_k, bpw, scale);
+        if (!launched) {
+            if (ref) AKV_KP(true, false); else AKV_KP(false, false);
+        }
+#undef AKV_KP
         int rc = check_launch("decode_step(k_pass)");
         if (rc != AKV_OK) return rc;
     }
