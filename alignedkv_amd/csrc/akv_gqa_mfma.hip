@@ -205,6 +205,54 @@ __device__ __forceinline__ void kt_compute_coarse(f32x4 *acc, const KTaskTile<SL
     }
 }
 
+// The two correction products alone: acc += C2 x B2 + C1 x B1 (operands as in mfma_levels)
+__device__ __forceinline__ void mfma_corrections(f32x4 &acc, u32 a_lo, u32 a_hi, f16x4 b1, f16x4 b2, u32 put1, u32 put2) {
+    acc = __builtin_amdgcn_mfma_f32_16x16x16f16(
+        as_f16x4(low_bits_excess(a_lo, 0xFF00FF00u, put2), low_bits_excess(a_hi, 0xFF00FF00u, put2)), b2, acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x16f16(
+        as_f16x4(low_bits_excess(a_lo, 0xFFF0FFF0u, put1), low_bits_excess(a_hi, 0xFFF0FFF0u, put1)), b1, acc, 0, 0, 0);
+}
+
+// What a tile that was multiplied at level 2 throughout still lacks: with A the values at the union level,
+// value_at_level - value_at_level_2 = C2 (level 0) or C2 - C1 (level 1), hence acc += C2 x (x [level < 2]) +
+// C1 x (-x [level == 1]).  need_mid / need_last: bit r of the lane's row r (as in kt_compute with kg = 0).
+template <int SL>
+__device__ __forceinline__ void kt_correct(f32x4 *acc, const KTaskTile<SL> &t, u32 need_mid, u32 need_last, f16x4 b1, f16x4 b2,
+                                           const LevelPuts &lp) {
+    constexpr int NX = (SL + 7) / 8;
+    constexpr int NP = SL == 4 ? 2 : 4;
+#pragma unroll
+    for (int x = 0; x < NX; ++x) {
+        u32 w[4][4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const bool mid = (need_mid >> r) & 1u, last = (need_last >> r) & 1u;
+            const u32 cm = mid ? 0u : 0x88888888u;
+            const u32 cl = (mid && !last) ? 0x88888888u : 0u;
+            u32 E, O;
+            split_even_odd(t.m[r][x] | cm, t.l[r][x] | cl, E, O);
+            const u32 Ha = t.h[r][SL == 4 ? 0 : 2 * x];
+            w[r][0] = __builtin_amdgcn_perm(Ha, E, 0x06010400u);
+            w[r][1] = __builtin_amdgcn_perm(Ha, O, 0x07010500u);
+            if constexpr (SL != 4) {
+                const u32 Hb = t.h[r][2 * x + 1];
+                w[r][2] = __builtin_amdgcn_perm(Hb, E, 0x06030402u);
+                w[r][3] = __builtin_amdgcn_perm(Hb, O, 0x07030502u);
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < NP; ++p) {
+            const int s0 = 8 * x + (p & 1) + 4 * (p >> 1);
+            const u32 a01_s0 = __builtin_amdgcn_perm(w[1][p], w[0][p], 0x05040100u);
+            const u32 a23_s0 = __builtin_amdgcn_perm(w[3][p], w[2][p], 0x05040100u);
+            const u32 a01_s2 = __builtin_amdgcn_perm(w[1][p], w[0][p], 0x07060302u);
+            const u32 a23_s2 = __builtin_amdgcn_perm(w[3][p], w[2][p], 0x07060302u);
+            mfma_corrections(acc[s0], a01_s0, a23_s0, b1, b2, lp.put1, lp.put2);
+            mfma_corrections(acc[s0 + 2], a01_s2, a23_s2, b1, b2, lp.put1, lp.put2);
+        }
+    }
+}
+
 template <int D, bool REF, int SL, int AHEAD, int KSH>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && AHEAD == 3 ? 3 : 1))) void mfma_k_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
@@ -522,6 +570,134 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     LevelPuts puts;
     puts.pin();
 
+    // Few tokens of the wave below level 2 for any head of the group (the usual case: under 1 % of the (token, head)
+    // pairs at batch 32, 32 over 8 heads, but 39 % of the 16-token tiles hold one): every tile is multiplied at level 2
+    // from its high bytes alone, and the tokens below level 2 -- listed up front from the probabilities -- are
+    // gathered into tiles of their own, 16 tokens each, whose rows are fetched at the level the group needs and add
+    // value_at_level - value_at_level_2 (kt_correct).  The first such tile is requested before the loop and has
+    // arrived when the loop ends.  Many such tokens (flat attention): the loop below, which corrects tile by tile.
+    bool handled = false;
+    if constexpr (!REF) {
+        constexpr int LIST = 256, MAX_LISTED = 48;
+        __shared__ unsigned short fine_tok[4][LIST];    // per wave: token - t_begin | head << 8 | bit 15: read at level 0
+        if (tokens_per_wave <= LIST) {
+            auto issue_high = [&](KTaskTile<CPP> &tile, int tok) {      // tokens tok .. tok + 15
+                const int oh = tok < t_end ? lane_h + tok * D : kSkip;
+#pragma unroll
+                for (int u = 0; u < 4; ++u) load_bytes<CPP>(tile.h[u], rH, oh + u * D);
+            };
+            KTaskTile<CPP> t[4];
+#pragma unroll
+            for (int i = 0; i < 3; ++i) issue_high(t[i], t_begin + 16 * i);
+            __builtin_amdgcn_sched_barrier(0);
+            // ---- the list: (token, head) pairs below level 2; every lane notes those of its head ----
+            unsigned short *list = fine_tok[wave];
+            int n_fine = 0;
+            // all probabilities of the lane's head for the wave's tokens in one round trip (they are the operands of the
+            // loop below as well): macro step mi, step s, tokens 4 kq + 0..3 -> bit 16 mi + 4 s + u of the lane's mask
+            u32x2 pall[LIST / MACRO][4];
+#pragma unroll
+            for (int mi = 0; mi < LIST / MACRO; ++mi) load_probs(pall[mi], t_begin + mi * MACRO);
+            {
+                const i16x2 c8 = {0x0800, 0x0800};
+                unsigned long long mask = 0ull;
+#pragma unroll
+                for (int mi = 0; mi < LIST / MACRO; ++mi) {
+                    u32 m16 = 0;
+#pragma unroll
+                    for (int w = 0; w < 8; ++w) {
+                        // 16-bit differences of two tokens (wrapping like the reference's `short` arithmetic,
+                        // extension/csrc/V_cache.cu:195-197,211): below level 2 <=> diff < 0x0800
+                        union { i16x2 v; u32 u; } x;
+                        x.v = __builtin_elementwise_sub_sat(wrap_diff16(a2, (w & 1) ? pall[mi][w >> 1].y : pall[mi][w >> 1].x), c8);
+                        m16 |= (((x.u >> 15) & 1u) | ((x.u >> 30) & 2u)) << (2 * w);
+                    }
+                    mask |= (unsigned long long)m16 << (16 * mi);
+                }
+                while (__builtin_amdgcn_ballot_w64(mask != 0ull) != 0ull) {
+                    const bool on = mask != 0ull;
+                    const int bit = on ? __builtin_ctzll(mask) : 0;
+                    const int mi = bit >> 4, sidx = (bit >> 2) & 3, u = bit & 3;
+                    // the probability itself, for the flag "read at level 0"
+                    u32 pb = 0;
+#pragma unroll
+                    for (int a = 0; a < LIST / MACRO; ++a)
+#pragma unroll
+                        for (int c = 0; c < 4; ++c)
+                            if (a == mi && c == sidx) pb = (u & 2) ? pall[a][c].y : pall[a][c].x;
+                    pb = (u & 1) ? pb >> 16 : pb & 0xffffu;
+                    const u32 entry = (u32)(64 * mi + 16 * sidx + 4 * kq + u) | ((u32)j << 8) |
+                                      ((v_level(amin, (unsigned short)pb) == 0 ? 1u : 0u) << 15);
+                    const unsigned long long bm = __builtin_amdgcn_ballot_w64(on);
+                    const int at = n_fine + (int)__builtin_amdgcn_mbcnt_hi((u32)(bm >> 32), __builtin_amdgcn_mbcnt_lo((u32)bm, 0u));
+                    if (on && at < LIST) list[at] = (unsigned short)entry;
+                    n_fine += __builtin_popcountll(bm);
+                    mask &= mask - 1ull;
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // the list is read by other lanes of the wave
+            if (n_fine <= MAX_LISTED) {
+                handled = true;
+                // ---- a tile of listed pairs: lane group kq takes the entries e0 + 4 kq + u (their rows at the pair's
+                //      level; the probability only in the lane of the pair's head, zero for the other heads) ----
+                KTaskTile<CPP> ct;
+                u32 cp[4];              // probability bits of the lane's head for its group's 4 tokens
+                u32 c_mid = 0, c_last = 0;
+                auto request_listed = [&](int e0) {
+                    c_mid = c_last = 0;
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int e = e0 + 4 * kq + u;
+                        const bool on = e < n_fine;
+                        const u32 entry = on ? (u32)list[e] : 0u;
+                        const int tok = t_begin + (int)(entry & 0xffu);
+                        const bool mine = on && ((entry >> 8) & 15u) == (u32)j;     // the pair's head is this lane's
+                        const bool last = on && (entry >> 15) != 0u;
+                        load_bytes<CPP>(ct.h[u], rH, on ? tok * D + (lane & 15) * CPP : kSkip);
+                        load_bytes<CPP / 2>(ct.m[u], rM, on ? tok * (D / 2) + (lane & 15) * (CPP / 2) : kSkip);
+                        load_bytes<CPP / 2>(ct.l[u], rL, last ? tok * (D / 2) + (lane & 15) * (CPP / 2) : kSkip);
+                        cp[u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(
+                            rP, mine ? (int)((bh0 + j) * geo.row_stride + tok) * 2 : kSkip, 0, 0);
+                        c_mid |= (on ? 1u : 0u) << u;
+                        c_last |= (last ? 1u : 0u) << u;
+                    }
+                };
+                auto apply_listed = [&]() {
+                    u32 b2[4], b1[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        const int lv = v_level(amin, (unsigned short)cp[u]);
+                        b2[u] = lv < 2 ? cp[u] : 0u;
+                        b1[u] = lv == 1 ? (cp[u] ^ 0x8000u) : 0u;
+                    }
+                    kt_correct<CPP>(acc, ct, c_mid, c_last, as_f16x4(b1[0] | (b1[1] << 16), b1[2] | (b1[3] << 16)),
+                                    as_f16x4(b2[0] | (b2[1] << 16), b2[2] | (b2[3] << 16)), puts);
+                };
+                request_listed(0);
+                __builtin_amdgcn_sched_barrier(0);
+                // ---- every tile at level 2 ----
+#pragma unroll
+                for (int mi = 0; mi < LIST / MACRO; ++mi) {
+                    const int base = t_begin + mi * MACRO;
+                    if (base < t_end) {
+#pragma unroll
+                        for (int si = 0; si < 4; ++si) {
+                            issue_high(t[(si + 3) & 3], base + 16 * (si + 3));
+                            __builtin_amdgcn_sched_barrier(0);
+                            kt_compute_coarse<CPP>(acc, t[si], as_f16x4(pall[mi][si].x, pall[mi][si].y));
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                }
+                // ---- the listed tokens: what their levels add to level 2 ----
+                for (int e0 = 0; e0 < n_fine; e0 += 16) {
+                    if (e0 > 0) request_listed(e0);
+                    apply_listed();
+                }
+            }
+        }
+    }
+    if (!handled) {
     u32x2 pn[4], pnn[4];
     VMacroOps oc, on;
     {
@@ -559,6 +735,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
         oc = on;
 #pragma unroll
         for (int i = 0; i < 4; ++i) pn[i] = pnn[i];
+    }
     }
     // optional record of the levels, outside the pipeline
     if (levels_out != nullptr) {
