@@ -40,7 +40,8 @@ def test_gqa_ragged_step_matches_per_sequence_oracle(B, Hq, Hkv, lens, steps, D)
         oracles.append(oc)
     flips = total = 0
     for s in range(steps):
-        q = rng.standard_normal((B, 1, Hq, D)).astype(np.float16)
+        # sharper, flat and in-between attention in turn: few, all and some of the tokens below level 2
+        q = (rng.standard_normal((B, 1, Hq, D)) * (1.0, 0.0, 0.3, 0.05)[s % 4]).astype(np.float16)
         kn = np.stack([k[b, lens[b] + s] for b in range(B)])[:, None]
         vn = np.stack([v[b, lens[b] + s] for b in range(B)])[:, None]
         out = cache.decode(0, dev(q), dev(kn), dev(vn)).cpu().numpy()
