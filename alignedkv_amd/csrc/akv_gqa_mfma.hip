@@ -515,7 +515,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const unsigned short *__restrict__ probs, const uint8_t *__restrict__ amin_u8, float *__restrict__ partial,
     uint8_t *__restrict__ levels_out, int levels_stride, uint8_t *__restrict__ amin_out, StepGeom geo,
-    int tokens_per_wave, int n_chunks, u32 probs_bytes) {
+    int tokens_per_wave, int n_chunks, u32 probs_bytes, int max_listed) {
     constexpr int CPP = D / 16;        // channels per lane
     constexpr int MACRO = 64;          // tokens per macro step: 4 tiles of 16 tokens
     __shared__ float fold[4][4][D];    // [wave][head of the pass][channel]
@@ -578,7 +578,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     // arrived when the loop ends.  Many such tokens (flat attention): the loop below, which corrects tile by tile.
     bool handled = false;
     if constexpr (!REF) {
-        constexpr int LIST = 256, MAX_LISTED = 48;
+        constexpr int LIST = 256;      // room of a wave's list; max_listed <= LIST pairs take this path
         __shared__ unsigned short fine_tok[4][LIST];    // per wave: token - t_begin | head << 8 | bit 15: read at level 0
         if (tokens_per_wave <= LIST) {
             auto issue_high = [&](KTaskTile<CPP> &tile, int tok) {      // tokens tok .. tok + 15
@@ -636,7 +636,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
                 }
             }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // the list is read by other lanes of the wave
-            if (n_fine <= MAX_LISTED) {
+            if (n_fine <= max_listed) {
                 handled = true;
                 // ---- a tile of listed pairs: lane group kq takes the entries e0 + 4 kq + u (their rows at the pair's
                 //      level; the probability only in the lane of the pair's head, zero for the other heads) ----
@@ -787,12 +787,16 @@ int launch_mfma_v_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
         return AKV_ERR_INVALID;
     }
     dim3 grid(p.n_chunks, geo.Hkv, B);
+    // pairs below level 2 per wave up to which they are listed and corrected in tiles of their own (at most 256: the
+    // room of the list; negative: always the loop that corrects tile by tile)
+    int max_listed = 48;
+    { AKV_TUNE("AKV_TUNE_V_LISTED", v); if (has_v) max_listed = v < 0 ? -1 : (v > 256 ? 256 : v); }
     if (ref)
         hipLaunchKernelGGL((mfma_v_pass_kernel<D, true>), grid, dim3(256), 0, st, f8, m4, l4, probs, amin, partial, levels_out,
-                           levels_stride, amin_out, geo, p.tokens_per_wave, p.n_chunks, (u32)probs_bytes);
+                           levels_stride, amin_out, geo, p.tokens_per_wave, p.n_chunks, (u32)probs_bytes, max_listed);
     else
         hipLaunchKernelGGL((mfma_v_pass_kernel<D, false>), grid, dim3(256), 0, st, f8, m4, l4, probs, amin, partial, levels_out,
-                           levels_stride, amin_out, geo, p.tokens_per_wave, p.n_chunks, (u32)probs_bytes);
+                           levels_stride, amin_out, geo, p.tokens_per_wave, p.n_chunks, (u32)probs_bytes, max_listed);
     return check_launch("decode_step(mfma v_pass)");
 }
 

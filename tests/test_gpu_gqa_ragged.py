@@ -23,6 +23,27 @@ def dev(a):
                                                    (3, 8, 2, [130, 64, 7], 70, -128), (2, 16, 1, [700, 255], 66, -128),
                                                    (2, 12, 4, [260, 900], 3, -64), (2, 4, 4, [200, 600], 70, -128)])
 def test_gqa_ragged_step_matches_per_sequence_oracle(B, Hq, Hkv, lens, steps, D):
+    _ragged_case_against_oracle(B, Hq, Hkv, lens, steps, D)
+
+
+@pytest.mark.parametrize("listed", [256, -1])
+@pytest.mark.parametrize("B,Hq,Hkv,lens,steps,D", [(3, 8, 2, [530, 64, 257], 8, 128), (2, 16, 1, [700, 255], 8, -128),
+                                                   (2, 12, 4, [260, 900], 8, -64)])
+def test_grouped_v_pass_with_every_pair_listed_and_with_none(monkeypatch, listed, B, Hq, Hkv, lens, steps, D):
+    """AKV_TUNE_V_LISTED: up to how many (token, head) pairs below level 2 a wave lists and corrects in tiles of their
+    own (256: whatever fits its list, many tiles one after the other; -1: never, the loop that corrects tile by tile)."""
+    from alignedkv_amd import load_library
+    lib = load_library()
+    monkeypatch.setenv("AKV_TUNE_V_LISTED", str(listed))
+    lib.akv_reload_tuning()
+    try:
+        _ragged_case_against_oracle(B, Hq, Hkv, lens, steps, D)
+    finally:
+        monkeypatch.delenv("AKV_TUNE_V_LISTED")
+        lib.akv_reload_tuning()
+
+
+def _ragged_case_against_oracle(B, Hq, Hkv, lens, steps, D):
     from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
     kb = 256 if D < 0 else 64
     D = abs(D)
