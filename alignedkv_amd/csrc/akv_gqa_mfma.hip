@@ -10,9 +10,11 @@
 // Per-head fetch levels (K: extension/csrc/K_cache.cu:211,249-252; V: extension/csrc/V_cache.cu:195-197,250-253)
 // stay exact.  A plane row is fetched at the finest level any head of the group asks for ("union level"); the
 // operand A holds the values at that level.  A head with a coarser level needs the value with its low bits
-// replaced (0x8 / 0x80): value_at_level = A - C1 (level 1) or A - C2 (level 2) with C1 = A - sub1(A),
-// C2 = A - sub2(A).  Both differences are exact in fp16 (same sign, exponent and upper mantissa), so two more
-// MFMAs with the operands (C1, -q [level == 1]) and (C2, -q [level == 2]) give every head exactly its own levels.
+// replaced (0x8 / 0x80): sub1(A) or sub2(A), one and-or per register.  Three MFMAs -- A, sub1(A), sub2(A) against x where
+// the head's level is 0, 1, 2 and zero elsewhere -- give every head exactly its own levels (mfma_levels).  Where a
+// tile has already been multiplied at level 2 throughout, what is missing is A - sub2(A) (level 0) or
+// sub1(A) - sub2(A) (level 1): differences that are exact in fp16 (same sign, exponent and upper mantissa), two MFMAs
+// (kt_correct).
 #include "akv_step.h"
 
 namespace akv {
@@ -48,7 +50,8 @@ struct LevelPuts {
     __device__ __forceinline__ void pin() { asm volatile("" : "+v"(put1), "+v"(put2)); }
 };
 
-// acc += A x B0  (+ C1 x B1 + C2 x B2 unless every plane is read)
+// acc += A x B0 + sub1(A) x B1 + sub2(A) x B2: B0 / B1 / B2 hold x where the head reads the element at level 0 / 1 / 2
+// and zero elsewhere (every plane read: only A x B0)
 template <bool REF>
 __device__ __forceinline__ void mfma_levels(f32x4 &acc, u32 a_lo, u32 a_hi, f16x4 b0, f16x4 b1, f16x4 b2, u32 put1,
                                             u32 put2) {
@@ -56,10 +59,8 @@ __device__ __forceinline__ void mfma_levels(f32x4 &acc, u32 a_lo, u32 a_hi, f16x
     // (an instruction takes one literal constant)
     acc = __builtin_amdgcn_mfma_f32_16x16x16f16(as_f16x4(a_lo, a_hi), b0, acc, 0, 0, 0);
     if (!REF) {
-        acc = __builtin_amdgcn_mfma_f32_16x16x16f16(
-            as_f16x4(low_bits_excess(a_lo, 0xFFF0FFF0u, put1), low_bits_excess(a_hi, 0xFFF0FFF0u, put1)), b1, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x16f16(
-            as_f16x4(low_bits_excess(a_lo, 0xFF00FF00u, put2), low_bits_excess(a_hi, 0xFF00FF00u, put2)), b2, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x16f16(as_f16x4((a_lo & 0xFFF0FFF0u) | put1, (a_hi & 0xFFF0FFF0u) | put1), b1, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x16f16(as_f16x4((a_lo & 0xFF00FF00u) | put2, (a_hi & 0xFF00FF00u) | put2), b2, acc, 0, 0, 0);
     }
 }
 
@@ -328,9 +329,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && 
             const u32 m1b = ((lv1 >> (4 * kg + 2)) & 1u ? 0xFFFFu : 0u) | ((lv1 >> (4 * kg + 3)) & 1u ? 0xFFFF0000u : 0u);
             const u32 m2a = ((lv2 >> (4 * kg)) & 1u ? 0xFFFFu : 0u) | ((lv2 >> (4 * kg + 1)) & 1u ? 0xFFFF0000u : 0u);
             const u32 m2b = ((lv2 >> (4 * kg + 2)) & 1u ? 0xFFFFu : 0u) | ((lv2 >> (4 * kg + 3)) & 1u ? 0xFFFF0000u : 0u);
-            const u32 na = qp[kg][0] ^ 0x80008000u, nb = qp[kg][1] ^ 0x80008000u;     // -q
-            kt_compute<REF, SL>(acc, t[kg % (AHEAD + 1)], kg, need_mid, need_last, as_f16x4(qp[kg][0], qp[kg][1]),
-                                as_f16x4(na & m1a, nb & m1b), as_f16x4(na & m2a, nb & m2b), puts);
+            const u32 qa = qp[kg][0], qb = qp[kg][1];
+            kt_compute<REF, SL>(acc, t[kg % (AHEAD + 1)], kg, need_mid, need_last, as_f16x4(qa & ~(m1a | m2a), qb & ~(m1b | m2b)),
+                                as_f16x4(qa & m1a, qb & m1b), as_f16x4(qa & m2a, qb & m2b), puts);
             __builtin_amdgcn_sched_barrier(0);
         }
         // lane (j, ig): acc[s][r] = score of slot s of token set 4 ig + r for query head j
@@ -720,13 +721,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
             __builtin_amdgcn_sched_barrier(0);
             if (fine(oc, si)) {
                 const u32 l1 = (oc.lv1 >> (4 * si)) & 0xfu, l2 = (oc.lv2 >> (4 * si)) & 0xfu;
-                const u32 na = oc.p[si].x ^ 0x80008000u, nb = oc.p[si].y ^ 0x80008000u;     // -p
-                const u32 n1a = na & ((l1 & 1u ? 0xFFFFu : 0u) | (l1 & 2u ? 0xFFFF0000u : 0u));
-                const u32 n1b = nb & ((l1 & 4u ? 0xFFFFu : 0u) | (l1 & 8u ? 0xFFFF0000u : 0u));
-                const u32 n2a = na & ((l2 & 1u ? 0xFFFFu : 0u) | (l2 & 2u ? 0xFFFF0000u : 0u));
-                const u32 n2b = nb & ((l2 & 4u ? 0xFFFFu : 0u) | (l2 & 8u ? 0xFFFF0000u : 0u));
+                const u32 pa = oc.p[si].x, pb = oc.p[si].y;
+                const u32 m1a = (l1 & 1u ? 0xFFFFu : 0u) | (l1 & 2u ? 0xFFFF0000u : 0u), m1b = (l1 & 4u ? 0xFFFFu : 0u) | (l1 & 8u ? 0xFFFF0000u : 0u);
+                const u32 m2a = (l2 & 1u ? 0xFFFFu : 0u) | (l2 & 2u ? 0xFFFF0000u : 0u), m2b = (l2 & 4u ? 0xFFFFu : 0u) | (l2 & 8u ? 0xFFFF0000u : 0u);
                 kt_compute<REF, CPP>(acc, t[si], 0, (oc.need >> (4 * si)) & 0xfu, (oc.need >> (16 + 4 * si)) & 0xfu,
-                                     as_f16x4(oc.p[si].x, oc.p[si].y), as_f16x4(n1a, n1b), as_f16x4(n2a, n2b), puts);
+                                     as_f16x4(pa & ~(m1a | m2a), pb & ~(m1b | m2b)), as_f16x4(pa & m1a, pb & m1b),
+                                     as_f16x4(pa & m2a, pb & m2b), puts);
             } else {
                 kt_compute_coarse<CPP>(acc, t[si], as_f16x4(oc.p[si].x, oc.p[si].y));
             }
