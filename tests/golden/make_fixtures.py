@@ -1,5 +1,6 @@
 """Writes tests/golden/akv_small_cases.npz: small seeded decode cases with everything the NumPy oracle derives
-from them (planes, fetch levels, threshold, probabilities, outputs).
+from them (planes, fetch levels, threshold, probabilities, outputs), and tests/golden/akv_gqa_cases.npz: grouped-query
+heads with a length per sequence (outputs, K levels and thresholds of every sequence run on its own with repeated KV heads).
 
 The reference ships no tests, golden vectors or fixtures, and its kernels are CUDA (nothing of it can run in this
 image), so these vectors come from this repository's own oracle (oracle/akv_oracle.py), whose functions are pinned
@@ -24,6 +25,50 @@ CASES = {   # name: (B, H, D, prefill, steps, k_block, literal_broadcast)
     "mha_kblock256": (1, 1, 64, 200, 2, 256, False),
     "mha_literal_broadcast": (2, 2, 64, 64, 1, 64, True),
 }
+
+
+GQA_CASES = {   # name: (Hq, Hkv, D, lengths per sequence, steps, k_block)
+    "gqa_g4_kblock256": (4, 1, 128, (270, 130), 2, 256),    # the first sequence has a block of 256 and a tile of the next
+    "gqa_g3_d64": (6, 2, 64, (130, 63), 2, 64),             # the second fills its rest buffer with the first step
+}
+
+
+def replay_gqa(Hq, Hkv, D, lens, steps, kb, k, v, q):
+    """Grouped-query heads with a length per sequence, as the reference's algorithm defines them: every sequence on its
+    own, the KV heads repeated for the query heads of their group.  Returns outputs [steps, B, 1, Hq, D] and, after
+    the last step, K levels [B, Hq, D] and thresholds [B, Hq]."""
+    G = Hq // Hkv
+    B = len(lens)
+    outs = np.zeros((steps, B, 1, Hq, D), np.float16)
+    klv = np.zeros((B, Hq, D), np.uint8)
+    amin = np.zeros((B, Hq), np.uint8)
+    for b in range(B):
+        oc = O.OracleCache(1, max(lens) + steps + 64, Hq, D, k_block=kb)
+        rep = lambda a: np.repeat(a, G, axis=2)
+        oc.save(rep(k[b:b + 1, :lens[b]]), rep(v[b:b + 1, :lens[b]]), 0, lens[b])
+        for s in range(steps):
+            t = lens[b] + s
+            outs[s, b] = oc.decode(q[s, b:b + 1], rep(k[b:b + 1, t:t + 1]), rep(v[b:b + 1, t:t + 1]))[0]
+        klv[b] = oc.last["k_levels"][0]
+        amin[b] = np.asarray(oc.last["amin"]).reshape(-1)
+    return outs, klv, amin
+
+
+def main_gqa():
+    out = {}
+    for name, (Hq, Hkv, D, lens, steps, kb) in GQA_CASES.items():
+        B = len(lens)
+        _, k, v = make_qkv(B, max(lens) + steps, Hkv, D, seed=len(name) + sum(lens), n_outliers=4)
+        q = np.random.default_rng(sum(lens)).standard_normal((steps, B, 1, Hq, D)).astype(np.float16)
+        outs, klv, amin = replay_gqa(Hq, Hkv, D, lens, steps, kb, k, v, q)
+        out[name + "/shape"] = np.array([Hq, Hkv, D, steps, kb], np.int32)
+        out[name + "/lens"] = np.array(lens, np.int32)
+        out[name + "/k"], out[name + "/v"], out[name + "/q"] = O.as_bits(k), O.as_bits(v), O.as_bits(q)
+        out[name + "/out"] = O.as_bits(outs)
+        out[name + "/k_levels"], out[name + "/amin"] = klv, amin
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "akv_gqa_cases.npz")
+    np.savez_compressed(path, **out)
+    print(path, os.path.getsize(path), "bytes")
 
 
 def main():
@@ -58,3 +103,4 @@ def main():
 
 if __name__ == "__main__":
     main()
+    main_gqa()

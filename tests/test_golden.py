@@ -98,3 +98,47 @@ def test_hip_path_reproduces_the_fixture(name, fused):
         assert np.array_equal(kc.last_levels.cpu().numpy(), c.g("k_levels"))
         # V levels depend on the probabilities: a level can flip where one sits on a rounding boundary
         assert (vc.last_levels.cpu().numpy() != c.g("v_levels")).mean() <= 0.01
+
+
+# ---- grouped-query heads with a length per sequence ---------------------------------------------------------------
+GQA = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "akv_gqa_cases.npz"))
+GQA_NAMES = sorted({k.split("/")[0] for k in GQA.files})
+
+
+def gqa_case(name):
+    Hq, Hkv, D, steps, kb = (int(x) for x in GQA[name + "/shape"])
+    g = lambda key: GQA[name + "/" + key]
+    return SimpleNamespace(Hq=Hq, Hkv=Hkv, D=D, steps=steps, kb=kb, lens=[int(x) for x in g("lens")], k=O.as_half(g("k")),
+                           v=O.as_half(g("v")), q=O.as_half(g("q")), out=O.as_half(g("out")), g=g)
+
+
+@pytest.mark.parametrize("name", GQA_NAMES)
+def test_numpy_oracle_reproduces_the_grouped_fixture(name):
+    from tests.golden.make_fixtures import replay_gqa
+    c = gqa_case(name)
+    outs, klv, amin = replay_gqa(c.Hq, c.Hkv, c.D, c.lens, c.steps, c.kb, c.k, c.v, c.q)
+    assert np.array_equal(O.as_bits(outs), c.g("out"))
+    assert np.array_equal(klv, c.g("k_levels")) and np.array_equal(amin, c.g("amin"))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", GQA_NAMES)
+def test_hip_path_reproduces_the_grouped_fixture(name):
+    import torch
+    from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
+    c = gqa_case(name)
+    B = len(c.lens)
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    cache = RaggedGQACache(1, B, max(c.lens) + c.steps + 64, c.Hq, c.Hkv, c.D, k_block=c.kb)
+    cache.record_levels = True
+    for b in range(B):
+        cache.prefill(0, b, dev(c.k[b:b + 1, :c.lens[b]]), dev(c.v[b:b + 1, :c.lens[b]]))
+    for s in range(c.steps):
+        kn = np.stack([c.k[b, c.lens[b] + s] for b in range(B)])[:, None]
+        vn = np.stack([c.v[b, c.lens[b] + s] for b in range(B)])[:, None]
+        out = cache.decode(0, dev(c.q[s]), dev(kn), dev(vn)).cpu().numpy()
+        assert np.max(np.abs(out.astype(np.float32) - c.out[s].astype(np.float32))) <= 2e-3
+    for b in range(B):
+        if (c.lens[b] + c.steps) // 64:
+            assert np.array_equal(cache.last_k_levels[b].cpu().numpy(), c.g("k_levels")[b])
+            assert np.array_equal(cache.last_alignment_min[b].cpu().numpy(), c.g("amin")[b])
