@@ -30,6 +30,7 @@ class V_Cache_Class(PlaneCacheBase):
         # (extension/v_cache_file.py:156-160, extension/csrc/V_cache.cu:195,337).
         self.literal_broadcast = literal_broadcast
         self.last_levels = None
+        self.last_probs = None
         self.last_alignment_min = None
         self.record_levels = False
 
@@ -112,6 +113,8 @@ class V_Cache_Class(PlaneCacheBase):
                                         self.max_seq_len, self.head_dim, s_cut.stride()[-2], flushed, reference,
                                         levels_out=levels)
         self.last_levels, self.last_alignment_min = levels, amin
+        if self.record_levels:
+            self.last_probs = s      # the probabilities the levels above were derived from (debug record)
         o = o.view(torch.half)
         o += torch.matmul(s[:, :, :, flushed:start_pos + seqlen], self._rest.transpose(1, 2)[:, :, :self._restlen, :])
         return o

@@ -70,9 +70,24 @@ class QuantizedCache_AlignedKV(_HFCache):
         self.fused = self.head_dim in (64, 128, 256)
         self.literal_broadcast = literal_broadcast
         self._device = device
-        self._scores = None
-        self._probs = None
+        # fp16 scratch rows of the fused step, one pair per stream: steps issued on different streams may overlap
+        # (all layers of one stream share a pair, their steps are ordered)
+        self._score_buffers = {}
         self._prepared = {}
+
+    def _buffers(self, device=None):
+        device = self._device if device is None else device
+        return self._score_buffers.get(_stream_ptr(device), (None, None))
+
+    @property
+    def _scores(self):
+        """fp16 scores [B, H, width] the fused step last wrote on the current stream (debug output)."""
+        return self._buffers()[0]
+
+    @property
+    def _probs(self):
+        """fp16 probabilities [B, H, width] the fused step last wrote on the current stream (debug output)."""
+        return self._buffers()[1]
 
     def update(self, key_states, value_states, layer_idx, cache_kwargs=None):
         raise Exception("This function is not used in AlignedKV")
@@ -132,15 +147,17 @@ class QuantizedCache_AlignedKV(_HFCache):
         st = self._prepared.get(layer_id)
         if st is None or st.key != key:
             B, H = self.max_batch_size, self.num_key_value_heads
-            if self._scores is None:
+            scores, probs = self._buffers(device)
+            if scores is None:
                 width = (kc.n_max_blocks + 1) * column_block
-                self._scores = torch.empty((B, H, width), dtype=torch.half, device=device)
-                self._probs = torch.empty((B, H, width), dtype=torch.half, device=device)
+                scores = torch.empty((B, H, width), dtype=torch.half, device=device)
+                probs = torch.empty((B, H, width), dtype=torch.half, device=device)
+                self._score_buffers[_stream_ptr(device)] = (scores, probs)
             st = cuda_module.prepare_decode_step(
                 (kc.k_cache_first_8, kc.k_cache_mid_4, kc.k_cache_last_4),
                 (vc.v_cache_first_8, vc.v_cache_mid_4, vc.v_cache_last_4),
                 kc._colmax, vc._colmax, kc._rest.view(torch.uint8), vc._rest.view(torch.uint8),
-                self._scores.view(torch.uint8), self._probs.view(torch.uint8), B, H, kc.k_n_max_blocks,
+                scores.view(torch.uint8), probs.view(torch.uint8), B, H, kc.k_n_max_blocks,
                 self.max_cache_len, self.head_dim, column_block, kc.k_block, vc.top_max_k, key=key)
             self._prepared[layer_id] = st
         return st

@@ -18,6 +18,11 @@ What pins each function (tests/test_oracle_*.py):
                                 original fp16 values; substituted levels == matmul on values
                                 truncated by closed form; cross-check with the C restatement
   bucket_max / amin / colmax    brute force on tiny inputs, closed forms
+  k_sum_and_max                 nested scalar loops on a tiny shape, known answers (tests/test_oracle_helpers.py)
+  softmax_fp32_to_half          torch.softmax(x.float()).half() on rows with -inf tails (<= 1 fp16 ulp, >= 99.9 % bit
+                                equal), float64 closed form, known answers
+  dense_attention               torch's fp16 matmul / fp32 softmax restatement of model/Llama_AlignedKV.py:130-139,
+                                float64 attention, a one-hot known answer
 fp16 tensors are carried as np.uint16 bit patterns unless stated otherwise.
 """
 from __future__ import annotations

@@ -19,6 +19,28 @@ def make_qkv(B, L, H, D, seed=0, k_kind="outlier", n_outliers=4):
     return q.astype(np.float16), k.astype(np.float16), v.astype(np.float16)
 
 
+# Worst end-to-end output error seen per comparison site, printed at the end of a test run (tests/conftest.py):
+# the slack the limits below leave is measured, not assumed.
+WORST_STEP_ERR = {}
+
+STEP_TOL = 1e-3          # max-abs bound on attention outputs against the oracle (fp32 accumulate)
+STEP_TOL_ROUNDED = 2e-3  # allowed only where the step's fp16 probabilities differ from the oracle's in some bit
+
+
+def assert_step_output(got, want, label, probs_equal=None):
+    """|got - want| <= 1e-3 for one decode step's output.  probs_equal=False (the fp16 probabilities the kernels produced
+    differ from the oracle's somewhere: a score rounded to the neighbouring fp16 value under another summation order,
+    which moves a sharp softmax row by up to ~0.4 %) widens the bound to 2e-3; probs_equal=True or None holds 1e-3."""
+    g = np.asarray(got).astype(np.float32)
+    w = np.asarray(want).astype(np.float32)
+    err = float(np.max(np.abs(g - w))) if g.size else 0.0
+    key = label + ("" if probs_equal is not False else " [probabilities differ]")
+    WORST_STEP_ERR[key] = max(WORST_STEP_ERR.get(key, 0.0), err)
+    limit = STEP_TOL_ROUNDED if probs_equal is False else STEP_TOL
+    assert err <= limit, f"{label}: max abs err {err:.3e} > {limit:g} (probabilities equal: {probs_equal})"
+    return err
+
+
 def ulp_diff_fp16(a, b):
     """Distance in units of fp16 representable values between two float16 arrays (finite)."""
     def key(x):

@@ -17,3 +17,11 @@ def oracle_c():
     from oracle import akv_oracle_c
     akv_oracle_c.build()
     return akv_oracle_c
+
+
+def pytest_terminal_summary(terminalreporter):
+    from tests.common import WORST_STEP_ERR
+    if WORST_STEP_ERR:
+        terminalreporter.write_line("worst max-abs error of attention outputs against the oracle, per comparison site:")
+        for k in sorted(WORST_STEP_ERR):
+            terminalreporter.write_line(f"  {WORST_STEP_ERR[k]:.3e}  {k}")

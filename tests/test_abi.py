@@ -55,3 +55,24 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(RuntimeError, match="no CPU or PyTorch fallback"):
         _lib.load_library()
+
+
+def test_reference_import_paths_resolve_to_this_library():
+    """The import lines of the reference's callers (extension/k_cache_file.py:3, extension/v_cache_file.py:5,
+    model/KVCache_AlignedKV.py:10-11, model/Llama_AlignedKV.py:14, example.py:4) work unchanged and give the same objects."""
+    from extension.KV_cache_cpp_extention import cuda_module
+    from extension.k_cache_file import K_Cache_Class
+    from extension.v_cache_file import V_Cache_Class
+    from model.KVCache_AlignedKV import QuantizedCache_AlignedKV
+    import alignedkv_amd.extension.KV_cache_cpp_extention as impl
+    import alignedkv_amd.extension.k_cache_file as kimpl
+    import alignedkv_amd.extension.v_cache_file as vimpl
+    import alignedkv_amd.model.KVCache_AlignedKV as cimpl
+    assert cuda_module is impl.cuda_module
+    assert K_Cache_Class is kimpl.K_Cache_Class and V_Cache_Class is vimpl.V_Cache_Class
+    assert QuantizedCache_AlignedKV is cimpl.QuantizedCache_AlignedKV
+    # the five ops of the reference's binding (extension/csrc/KV_cache_ops.cpp:69-75)
+    for op in ("k_cache_save", "k_cache_compute", "v_cache_save", "v_cache_test_compute", "v_cache_compute"):
+        assert callable(getattr(cuda_module, op))
+    import extension.k_cache_file as kf
+    assert kf.column_block == 64 and kf.cdiv(65, 64) == 2

@@ -10,6 +10,7 @@ import numpy as np
 import pytest
 
 from oracle import akv_oracle as O
+from tests.common import assert_step_output
 
 FIX = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "akv_small_cases.npz"))
 NAMES = sorted({k.split("/")[0] for k in FIX.files})
@@ -84,7 +85,7 @@ def test_hip_path_reproduces_the_fixture(name, fused):
     for s in range(c.steps):
         t = c.prefill + s
         out = cache.auto_compute(dev(c.q[s]), dev(c.k[:, t:t + 1]), dev(c.v[:, t:t + 1]), 0, None)
-        assert np.max(np.abs(out.cpu().numpy().astype(np.float32) - c.out[s].astype(np.float32))) <= 2e-3
+        assert_step_output(out.cpu().numpy(), c.out[s], f"golden fixture {name} (fused={fused})")
     R = kc.reststartpos
     nkb = O.cdiv(R, c.kb)
     got_k = [kc.k_cache_first_8, kc.k_cache_mid_4, kc.k_cache_last_4]
@@ -137,7 +138,7 @@ def test_hip_path_reproduces_the_grouped_fixture(name):
         kn = np.stack([c.k[b, c.lens[b] + s] for b in range(B)])[:, None]
         vn = np.stack([c.v[b, c.lens[b] + s] for b in range(B)])[:, None]
         out = cache.decode(0, dev(c.q[s]), dev(kn), dev(vn)).cpu().numpy()
-        assert np.max(np.abs(out.astype(np.float32) - c.out[s].astype(np.float32))) <= 2e-3
+        assert_step_output(out, c.out[s], f"golden grouped fixture {name}")
     for b in range(B):
         if (c.lens[b] + c.steps) // 64:
             assert np.array_equal(cache.last_k_levels[b].cpu().numpy(), c.g("k_levels")[b])

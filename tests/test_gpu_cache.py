@@ -9,7 +9,7 @@ import torch
 import torch.nn.functional as F
 
 from oracle import akv_oracle as O
-from tests.common import make_qkv
+from tests.common import assert_step_output, make_qkv
 
 pytestmark = pytest.mark.gpu
 
@@ -61,6 +61,11 @@ def test_cache_matches_oracle_step_by_step(prefill, steps, literal_broadcast, k_
         qt = rng.standard_normal((B, 1, H, D)).astype(np.float16)
         out = cache.auto_compute(dev(qt), dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None)
         want = oc.decode(qt, k[:, t:t + 1], v[:, t:t + 1])
+        probs_equal = None
+        if not fused:
+            # the op sequence: the probabilities are torch's softmax on the GPU, recorded by the V host class
+            probs_equal = bool(np.array_equal(O.as_bits(vc.last_probs[:, :, 0, :t + 1].cpu().numpy()),
+                                              O.as_bits(np.ascontiguousarray(oc.last["probs"][:, :, 0, :t + 1]))))
         assert cache.get_seq_length(0) == t + 1 and kc.reststartpos == oc.rest_start and kc.restklen == oc.rest_len
         assert planes_equal(cache, oc), f"planes differ after token {t}"
         assert np.array_equal(kc.k_cache_exp_column_max.cpu().numpy(), oc.k_colmax)
@@ -71,6 +76,8 @@ def test_cache_matches_oracle_step_by_step(prefill, steps, literal_broadcast, k_
             flips += int((got_lv != oc.last["v_levels"]).sum())
             total += got_lv.size
             if fused:
+                probs_equal = bool(np.array_equal(O.as_bits(cache._probs[:, :, :t + 1].cpu().numpy()),
+                                                  O.as_bits(np.ascontiguousarray(oc.last["probs"][:, :, 0, :t + 1]))))
                 # bit exact for the probabilities and the threshold the kernels themselves produced
                 R = oc.rest_start
                 pk = cache._probs[:, :, :R].cpu().numpy()
@@ -83,10 +90,9 @@ def test_cache_matches_oracle_step_by_step(prefill, steps, literal_broadcast, k_
                 pd = np.abs(cache._probs[:, :, :t + 1].cpu().numpy().astype(np.float32)
                             - oc.last["probs"][:, :, 0, :t + 1].astype(np.float32)).max()
                 assert pd <= 2e-3
-        err = np.max(np.abs(out.cpu().numpy().astype(np.float32) - want.astype(np.float32)))
-        # end to end a score may round to the neighbouring fp16 value (different summation order), which
-        # moves a sharp softmax by ~0.4 %: 2e-3 here; with identical op inputs the ops hold 1e-3 (test_gpu_ops.py)
-        assert err <= 2e-3, f"token {t}: max abs err {err}"
+        # 1e-3; only where the kernels' fp16 probabilities differ from the oracle's in some bit (a score rounded to the
+        # neighbouring fp16 value under another summation order) 2e-3.  The worst error seen is printed at the end of the run.
+        assert_step_output(out.cpu().numpy(), want, f"cache step by step (fused={fused}, k_block={k_block})", probs_equal)
     # probabilities are produced by two different softmax implementations: a V level can only flip
     # where a probability or the probe sits on a rounding boundary
     assert flips <= max(2, 0.002 * total), f"{flips} of {total} V levels differ"
