@@ -16,6 +16,8 @@
 // run first, exactly as the reference flushes before it computes.
 #include "akv_step.h"
 
+#include <mutex>
+
 namespace akv {
 
 // defined in akv_k.hip / akv_v.hip
@@ -1383,4 +1385,62 @@ extern "C" int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_
                                row_stride, workspace, workspace_bytes, k_levels_out, v_levels_out, amin_out, bsz,
                                n_kv_heads, n_kv_heads, n_max_blocks, max_seq_len, head_dim, d_block, d_block, top_max_k,
                                cur_len, nullptr, reference, literal_broadcast, stream);
+}
+
+// ------------------------------------------------------------------------------------------------
+// The step for callers that cannot allocate: its workspace (probe exponents, thresholds, tail outputs, partial sums
+// of the V pass, set-up words and task maps) lives in a file-scope device array instead of a buffer the caller
+// brings.  Every GPU the library runs on holds its own copy of the array at its own address; the address is looked
+// up once per device and only that pointer is ever handed to kernels.
+// ------------------------------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = AKV_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices];   // per device: address of that device's copy of `scratch`
+
+// address of the current device's copy of the scratch array (null + error set on failure)
+void *static_scratch() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error("decode_step_static: no current device (or more than %d devices)", kMaxDevices);
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *p = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || p == nullptr) {
+            set_error("decode_step_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+}  // namespace
+
+extern "C" int akv_decode_step_static(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,
+                                      uint8_t *v_mid_4, uint8_t *v_last_4, uint8_t *k_exp_column_max,
+                                      uint8_t *v_exp_column_max, uint8_t *restk, uint8_t *restv, const uint8_t *q,
+                                      const uint8_t *k_new, const uint8_t *v_new, const uint8_t *mask, int mask_stride,
+                                      uint8_t *out, uint8_t *scores, uint8_t *probs, int row_stride,
+                                      uint8_t *k_levels_out, uint8_t *v_levels_out, uint8_t *amin_out, int bsz,
+                                      int n_kv_heads, int n_max_blocks, int max_seq_len, int head_dim, int d_block,
+                                      int top_max_k, int cur_len, int rest_start, int rest_len, int reference,
+                                      int literal_broadcast, akv_stream_t stream) {
+    const size_t need = akv_decode_step_workspace_bytes(bsz, n_kv_heads, head_dim, max_seq_len);
+    AKV_REQUIRE(need > 0, "decode_step_static: non-positive dimension");
+    AKV_REQUIRE(need <= kStaticScratchBytes,
+                "decode_step_static: this shape needs %zu bytes of workspace, the built-in scratch array holds %zu; use "
+                "akv_decode_step with a workspace of your own", need, kStaticScratchBytes);
+    void *ws = static_scratch();
+    if (ws == nullptr) return AKV_ERR_LAUNCH;
+    return akv_decode_step(k_first_8, k_mid_4, k_last_4, v_first_8, v_mid_4, v_last_4, k_exp_column_max, v_exp_column_max,
+                           restk, restv, q, k_new, v_new, mask, mask_stride, out, scores, probs, row_stride, ws,
+                           kStaticScratchBytes, k_levels_out, v_levels_out, amin_out, bsz, n_kv_heads, n_max_blocks,
+                           max_seq_len, head_dim, d_block, top_max_k, cur_len, rest_start, rest_len, reference,
+                           literal_broadcast, stream);
 }

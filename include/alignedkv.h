@@ -157,6 +157,27 @@ AKV_API int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_las
                             int literal_broadcast, akv_stream_t stream);
 
 /*
+ * akv_decode_step for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as akv_decode_step
+ * without `workspace` / `workspace_bytes`: the step's scratch (probe exponents, thresholds, tail outputs, partial sums of
+ * the V pass) lives in an array of AKV_STATIC_SCRATCH_BYTES bytes inside the library's device code, one copy per GPU,
+ * held until the process ends.  The call allocates and frees nothing.  Shapes for which
+ * akv_decode_step_workspace_bytes(bsz, n_kv_heads, head_dim, max_seq_len) exceeds AKV_STATIC_SCRATCH_BYTES are rejected
+ * (AKV_ERR_INVALID).  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams,
+ * two host threads) race on it and must be serialised by the caller; nothing in the array has to survive between calls.
+ */
+#define AKV_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+AKV_API int akv_decode_step_static(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,
+                                   uint8_t *v_mid_4, uint8_t *v_last_4, uint8_t *k_exp_column_max,
+                                   uint8_t *v_exp_column_max, uint8_t *restk, uint8_t *restv, const uint8_t *q,
+                                   const uint8_t *k_new, const uint8_t *v_new, const uint8_t *mask, int mask_stride,
+                                   uint8_t *out, uint8_t *scores, uint8_t *probs, int row_stride,
+                                   uint8_t *k_levels_out, uint8_t *v_levels_out, uint8_t *amin_out,
+                                   int bsz, int n_kv_heads, int n_max_blocks, int max_seq_len, int head_dim, int d_block,
+                                   int top_max_k, int cur_len, int rest_start, int rest_len, int reference,
+                                   int literal_broadcast, akv_stream_t stream);
+
+/*
  * The fused decode step for grouped-query attention and per-sequence lengths; beyond the reference, which
  * asserts multi-head attention and keeps one scalar length per layer (model/KVCache_AlignedKV.py:32,
  * extension/k_cache_file.py:133, extension/v_cache_file.py:146).  Per query head the algorithm is the
