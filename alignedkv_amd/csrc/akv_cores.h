@@ -453,7 +453,8 @@ struct VListed {
     }
 };
 
-template <int D, bool REF, int NIT>
+// PAUX: cache policy of the probability loads (kDeviceScope when another workgroup of the same launch wrote them)
+template <int D, bool REF, int NIT, int PAUX = 0>
 __device__ __forceinline__ void v_accumulate(VFirstTile<D> &ft, const uint8_t *f8, const uint8_t *m4, const uint8_t *l4,
                                              int n_tokens, const unsigned short *s_row, unsigned char amin, int t_begin,
                                              int t_end, float *acc, uint8_t *levels_row) {
@@ -476,7 +477,7 @@ __device__ __forceinline__ void v_accumulate(VFirstTile<D> &ft, const uint8_t *f
 #pragma unroll
         for (int u = 0; u < HV; ++u) {
             const int t = t_begin + (hf * HV + u) * TPL + tl;
-            sb[hf][u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < t_end ? t * 2 : kSkip, 0, 0);
+            sb[hf][u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < t_end ? t * 2 : kSkip, 0, PAUX);
         }
     __builtin_amdgcn_sched_barrier(0);
     // Software pipeline over half tiles (see k_score_blocks): one half tile is in flight while the other is
@@ -679,41 +680,59 @@ __device__ __forceinline__ int v_stream_count_fine(const unsigned short *s_row, 
 // (v_stream_apply_list).  For rows where they are rare: a listed token costs a second fetch of its high bytes and a
 // share of a memory round trip of its own (at one token in nine the pass takes 52 instead of 30 us).
 // list: LDS, room for every token of the wave (n_per_wave * HT entries); count: its length.
-template <int D, int NR, int PF, int NRING>
+// PRE > 0: the wave's first PRE half tiles of high bytes were requested long before (`pre`, in registers since before
+// the caller's own set-up: whatever of the row travels while the caller cannot stream yet is time HBM would otherwise
+// idle); they are multiplied first, while the ring's first requests are on their way.
+template <int D, int NR, int PF, int NRING, int PRE = 0>
 __device__ __forceinline__ void v_stream_run_deferred(VRing<D, NRING> &ring, const uint8_t *f8, int n_tokens,
-                                                     const unsigned short *s_row, unsigned char amin, const VSeq &seq,
-                                                     float *acc, u32 *list, int &count) {
+                                                     const unsigned short *s_row, unsigned char amin, const VSeq &seq_in,
+                                                     float *acc, u32 *list, int &count,
+                                                     const VHighPart<VStream<D>::HV> *pre = nullptr) {
     using S = VStream<D>;
     static_assert(NR >= 2 && NR <= NRING, "one slot is multiplied while the others travel");
+    static_assert(PRE == 0 || PF == 0, "either the ring's first slots or the separate tiles are requested early");
     constexpr int HV = S::HV;
     const int lane = threadIdx.x & 63, tl = lane / S::LPR, cl = lane % S::LPR;
     const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
     const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)n_tokens * 2);
+    // tokens of a half tile below level 2 (one lane per token notes it: the first of its row), then the half tile at level 2
+    auto multiply = [&](const VHighPart<HV> &hi, const u32 *sb, int half) {
+        bool fine[HV];
+        bool any = false;
+#pragma unroll
+        for (int u = 0; u < HV; ++u) {
+            fine[u] = cl == 0 && v_level(amin, (unsigned short)sb[u]) < 2 && sb[u] != 0u;
+            any = any || fine[u];
+        }
+        if (__builtin_amdgcn_ballot_w64(any) != 0ull) {
+            const int base = half * S::HT + tl;
+#pragma unroll
+            for (int u = 0; u < HV; ++u) VListed<D>::append(list, count, fine[u], base + u * S::TPL, sb[u]);
+        }
+        v_compute_half_coarse<HV>(acc, hi, sb);
+        pin_accumulators(acc);
+    };
+    u32 psb[PRE > 0 ? PRE : 1][HV];
+#pragma unroll
+    for (int j = 0; j < PRE; ++j) v_stream_issue_probs<D>(psb[j], rS, seq_in.half(j));
+    VSeq seq = seq_in;
+    seq.first += PRE;
 #pragma unroll
     for (int k = PF; k < NR - 1; ++k) v_stream_issue_high<D>(ring.hi[k], rH, seq.half(k));
 #pragma unroll
     for (int k = 0; k < NR - 1; ++k) v_stream_issue_probs<D>(ring.sb[k], rS, seq.half(k));
     __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < PRE; ++j) {
+        multiply(pre[j], psb[j], seq_in.half(j));
+        __builtin_amdgcn_sched_barrier(0);
+    }
     auto round = [&](int i0) {
 #pragma unroll
         for (int k = 0; k < NR; ++k) {
             v_stream_issue<D, NRING>(ring, (k + NR - 1) % NR, rH, rS, seq.half(i0 + k + NR - 1));
             __builtin_amdgcn_sched_barrier(0);
-            // tokens of this half tile below level 2 (one lane per token notes it: the first of its row)
-            bool fine[HV];
-            bool any = false;
-#pragma unroll
-            for (int u = 0; u < HV; ++u) {
-                fine[u] = cl == 0 && v_level(amin, (unsigned short)ring.sb[k][u]) < 2 && ring.sb[k][u] != 0u;
-                any = any || fine[u];
-            }
-            if (__builtin_amdgcn_ballot_w64(any) != 0ull) {
-                const int base = seq.half(i0 + k) * S::HT + tl;
-#pragma unroll
-                for (int u = 0; u < HV; ++u) VListed<D>::append(list, count, fine[u], base + u * S::TPL, ring.sb[k][u]);
-            }
-            v_compute_half_coarse<HV>(acc, ring.hi[k], ring.sb[k]);
-            pin_accumulators(acc);
+            multiply(ring.hi[k], ring.sb[k], seq.half(i0 + k));
             __builtin_amdgcn_sched_barrier(0);
         }
     };

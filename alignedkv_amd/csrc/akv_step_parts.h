@@ -1,0 +1,546 @@
+// Device-side building blocks of the fused decode step, shared by its multi-launch form (akv_fused.hip) and its
+// one-launch form (akv_onelaunch.hip): the K pass over one 256-token stretch of a (batch, head) row, the middle stage
+// of a row (append, tail scores, softmax, probe, threshold, tail output) and the pieces of the V pass.
+#pragma once
+
+#include "akv_step.h"
+
+namespace akv {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
+    return v;
+}
+
+// K pass over the 256-token stretch `chunk` of a row of planes with 64-token blocks, by a workgroup of four waves: a wave
+// takes one block and requests all its rows at once (16 KiB in flight for head_dim 128, no loop).  bh_kv / bh: row of
+// the planes (KV head) and of q / the scores (query head).  Scores are stored at device scope.
+template <int D, bool REF>
+__device__ __forceinline__ void k_pass64_whole_blocks(
+    const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
+    const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
+    unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, const StepGeom &geo, float scale, int chunk, int bh_kv,
+    int bh, int R) {
+    constexpr int CB = 64;
+    constexpr int NG = D / 16;
+    static_assert(D <= 128, "a wave holds every channel of a block: head_dim 64 or 128");
+    const int lane = threadIdx.x & 63, wave = wave_index();
+    const int n_blocks = R / CB;
+    const int blk = chunk * 4 + wave;    // may lie past the end: the wave then only helps staging
+    const int64_t plane_off = (int64_t)bh_kv * geo.n_max_blocks * (D * (CB / 2));
+    KHalfTile<NG> ta;
+    k_issue_half_h<D, NG>(ta, make_rsrc(first_8 + plane_off * 2, (u32)n_blocks * (D * CB)), blk, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    // q and the exponent sums of all channels, staged once per workgroup (three scattered global loads per
+    // channel and wave otherwise: half as many load instructions again as the planes themselves need)
+    __shared__ u32 staged[D];      // [channel]: q bits | exponent sum << 16
+    for (int c = threadIdx.x; c < D; c += 256) {
+        const u32 qb = q[(int64_t)bh * D + c];
+        // column max including the token appended by this step
+        const u32 cm = max((u32)kcm[(int64_t)bh_kv * D + c], exp_field(k_new[(int64_t)bh_kv * D + c]));
+        staged[c] = qb | (((exp_field(qb) + cm) & 0xffu) << 16);
+    }
+    __syncthreads();
+    float qf[NG];
+    u32 esum[NG];
+    u32 mx = 0;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+        const u32 w = staged[g * 16 + (lane >> 2)];
+        qf[g] = lo_half_to_float(w);
+        esum[g] = w >> 16;
+        mx = max(mx, esum[g]);
+    }
+#pragma unroll
+    for (int m = 4; m <= 32; m <<= 1) mx = max(mx, (u32)__shfl_xor((int)mx, m, 64));
+    u32 need_mid = 0, need_last = 0;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+        const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)esum[g]);
+        need_mid |= (lv < 2 ? 1u : 0u) << g;
+        need_last |= (lv == 0 ? 1u : 0u) << g;
+        if (levels_out != nullptr && chunk == 0 && wave == 0 && (lane & 3) == 0)
+            levels_out[(int64_t)bh * D + g * 16 + (lane >> 2)] = (uint8_t)lv;
+    }
+    if (blk < n_blocks)
+        k_score_block_whole<D>(ta, mid_4 + plane_off, last_4 + plane_off, n_blocks, blk, qf, need_mid, need_last,
+                               scores + (int64_t)bh * geo.row_stride, scale);
+}
+
+// K pass over one 256-token block `blk` of the (batch, head) row `bh` of planes with 256-token blocks, by a workgroup of
+// NWV waves: each wave takes 1/NWV of the channels, requests all its rows at once (12 KiB per wave with four waves and
+// head_dim 128) and the partial scores are added through LDS.  R: flushed tokens of the row (the last block may be
+// partly filled).  Scores are stored at device scope.
+template <int D, bool REF, int NWV>
+__device__ __forceinline__ void k_pass256_split_block(
+    const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
+    const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
+    unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, const StepGeom &geo, float scale, int blk, int bh,
+    int R) {
+    constexpr int KB = 256;
+    constexpr int NG = D / 4;      // load groups of 4 channels
+    constexpr int HG = 4;          // groups per half tile
+    constexpr int GW = NG / NWV;   // groups per wave
+    constexpr int NT = GW / HG;    // half tiles per wave
+    static_assert(GW % HG == 0 && NG <= 32, "head_dim 64 or 128");
+    const int lane = threadIdx.x & 63, wave = wave_index();
+    const int n_blocks = (R + KB - 1) / KB;     // the last one may be partly filled
+    const int64_t plane_off = (int64_t)bh * geo.n_max_blocks * (D * (KB / 2));
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(first_8 + plane_off * 2, (u32)n_blocks * (D * KB));
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(mid_4 + plane_off, (u32)n_blocks * (D * KB / 2));
+    const __amdgpu_buffer_rsrc_t rL = make_rsrc(last_4 + plane_off, (u32)n_blocks * (D * KB / 2));
+    const int g_first = wave * GW;
+    KHalfTile<HG> t[NT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) k256_issue_h<D, HG>(t[i], rH, blk, g_first + HG * i);
+    __builtin_amdgcn_sched_barrier(0);
+    __shared__ u32 staged[D];      // [channel]: q bits | exponent sum << 16
+    __shared__ float part[NWV][KB];  // [wave][slot]: partial scores
+    for (int c = threadIdx.x; c < D; c += 64 * NWV) {
+        const u32 qb = q[(int64_t)bh * D + c];
+        // column max including the token appended by this step
+        const u32 cm = max((u32)kcm[(int64_t)bh * D + c], exp_field(k_new[(int64_t)bh * D + c]));
+        staged[c] = qb | (((exp_field(qb) + cm) & 0xffu) << 16);
+    }
+    __syncthreads();
+    u32 mx = 0;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) mx = max(mx, staged[4 * g + (lane >> 4)] >> 16);
+    mx = max(mx, (u32)__shfl_xor((int)mx, 16, 64));
+    mx = max(mx, (u32)__shfl_xor((int)mx, 32, 64));
+    float qf[GW];
+    u32 need_mid = 0, need_last = 0;   // bit g: of the wave's group g
+#pragma unroll
+    for (int g = 0; g < GW; ++g) {
+        const u32 w = staged[4 * (g_first + g) + (lane >> 4)];
+        qf[g] = lo_half_to_float(w);
+        const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)(w >> 16));
+        need_mid |= (lv < 2 ? 1u : 0u) << g;
+        need_last |= (lv == 0 ? 1u : 0u) << g;
+        if (levels_out != nullptr && blk == 0 && (lane & 15) == 0)
+            levels_out[(int64_t)bh * D + 4 * (g_first + g) + (lane >> 4)] = (uint8_t)lv;
+    }
+#pragma unroll
+    for (int i = 0; i < NT; ++i)
+        k256_issue_ml<D, HG>(t[i], rM, rL, blk, g_first + HG * i, need_mid << g_first, need_last << g_first);
+    __builtin_amdgcn_sched_barrier(0);
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NT; ++i) k_compute_half<HG>(acc, t[i], HG * i, qf, need_mid, need_last);
+    reduce_scatter_step<16>(acc, 32);
+    reduce_scatter_step<8>(acc, 16);
+    const int slot = (lane & 15) * 16 + ((lane & 32) ? 8 : 0) + ((lane & 16) ? 4 : 0);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part[wave][slot + i] = acc[i];
+    __syncthreads();
+    for (int sl = threadIdx.x; sl < KB; sl += 64 * NWV) {
+        const int token = blk * KB + sl;
+        if (token < R) {
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NWV; ++w) sum += part[w][sl];
+            // device scope: the workgroup that runs the softmax for this (batch, head) may sit on another XCD
+            store_u16_device(make_rsrc(scores + (int64_t)bh * geo.row_stride, (u32)R * 2), token * 2, float_to_half_bits(sum * scale));
+        }
+    }
+}
+
+struct MiddleArgs {
+    const unsigned short *q, *k_new, *v_new, *mask;
+    unsigned short *restk, *restv, *scores, *probs, *otail;
+    uint8_t *kcm, *vcm, *toe, *amin;
+    const uint8_t *v_first_8;
+    StepGeom g;
+    int mask_stride;
+    int top_k;
+    int persist;  // this kernel appends the token (it is not in the rest buffers / planes yet)
+};
+
+struct NoHook {
+    __device__ __forceinline__ void operator()() const {}
+};
+// hook: called once the loads that depend on nothing have been requested (a caller that goes on in the same
+// workgroup requests its own data there: loads return in order, so these come back first)
+// DEV: what later stages read (probabilities, threshold, tail output) is stored at device scope, for a launch whose
+// other workgroups -- on other XCDs, with L2 caches of their own -- go on with the row
+template <int D, int NT, typename Hook = NoHook, bool DEV = false>
+__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u32 *amin_lds = nullptr, Hook hook = Hook());
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
+// global store of the wave (here: 8 KiB of probabilities on their way to memory), which nobody inside the
+// middle stage reads back; the stage ends with a full barrier.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+template <int NW>
+__device__ __forceinline__ float block_reduce(float v, bool is_max, float *red) {
+    v = is_max ? wave_max(v) : wave_sum(v);
+    lds_barrier();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    lds_barrier();
+    float r = red[0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) r = is_max ? fmaxf(r, red[w]) : r + red[w];
+    return r;
+}
+
+// Decodes 8 fp16 scores (one 16-byte vector) into floats, adding the fp16 mask in fp16 if there is one.
+__device__ __forceinline__ void decode_scores8(const u32x4 w, const unsigned short *mrow, int t0, float *x) {
+    const u32 ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const u32 lo = ww[j] & 0xffffu, hi = ww[j] >> 16;
+        if (mrow == nullptr) {
+            x[2 * j] = half_bits_to_float(lo);
+            x[2 * j + 1] = half_bits_to_float(hi);
+        } else {
+            x[2 * j] = half_bits_to_float(float_to_half_bits(half_bits_to_float(lo) + half_bits_to_float(mrow[t0 + 2 * j])));
+            x[2 * j + 1] = half_bits_to_float(float_to_half_bits(half_bits_to_float(hi) + half_bits_to_float(mrow[t0 + 2 * j + 1])));
+        }
+    }
+}
+
+// NT threads (a multiple of 256) of one workgroup run the stage for one (batch, head).
+template <int D, int NT, typename Hook, bool DEV>
+__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u32 *amin_lds, Hook hook) {
+    constexpr int VPT = 4;                    // 16-byte score vectors a thread keeps in registers
+    constexpr int NW = NT / 64;               // waves
+    __shared__ float red[NW];
+    __shared__ unsigned short tail_s[64];     // fp16 scores of the tail (mask not yet added)
+    __shared__ float tail_p[64];              // probabilities of the tail
+    __shared__ u32 cand_key[NW][32];
+    __shared__ float probe_p[32];
+    __shared__ int probe_t[32];
+    __shared__ u32 red_min[NW];
+    __shared__ float tail_o[NW][D];           // per-wave sums of the tail's share of the output
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // bh indexes (batch, query head); the keys, values, column maxima and rest buffers belong to its KV head
+    const int b = bh / a.g.Hq, hq = bh - b * a.g.Hq, h = hq / a.g.G;
+    const int bh_kv = b * a.g.Hkv + h;
+    const int Hkv = a.g.Hkv, cb = a.g.cb;
+    const bool owner = hq % a.g.G == 0;       // one query head of the group writes the shared state
+    int R, nrest;
+    seq_state(a.g, b, R, nrest);
+    const int newest = nrest - 1;
+    const unsigned short *qrow = a.q + (int64_t)bh * D;
+    const unsigned short *knew = a.k_new + (int64_t)bh_kv * D;
+    const unsigned short *vnew = a.v_new + (int64_t)bh_kv * D;
+    unsigned short *srow = a.scores + (int64_t)bh * a.g.row_stride;
+    unsigned short *prow = a.probs + (int64_t)bh * a.g.row_stride;
+    const unsigned short *mrow = a.mask ? a.mask + (int64_t)b * a.mask_stride : nullptr;
+    const int nvec = R >> 3;
+    const bool in_regs = nvec <= NT * VPT;
+    // scores of the flushed part are read at device scope: other workgroups of the same launch wrote them
+    const __amdgpu_buffer_rsrc_t rScores = make_rsrc(srow, (u32)R * 2);
+    const __amdgpu_buffer_rsrc_t rProbs = make_rsrc(prow, (u32)(R + nrest) * 2);
+    auto store_probs8 = [&](int i, const u32x4 o) {
+        if constexpr (DEV) __builtin_amdgcn_raw_buffer_store_b128(o, rProbs, i * 16, 0, kDeviceScope);
+        else *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
+    };
+    auto store_prob1 = [&](int t, unsigned short p) {
+        if constexpr (DEV) store_u16_device(rProbs, t * 2, p);
+        else prow[t] = p;
+    };
+
+    // Everything that does not depend on anything else is requested first: the score vectors of the
+    // flushed part, the new token and the column maxima.
+    u32x4 sv[VPT];
+    if (in_regs) {
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int i = tid + NT * v;
+            sv[v] = load_b128_device(rScores, i < nvec ? i * 16 : kSkip);
+        }
+    }
+    // the tail's key rows and q: LPT lanes per tail token, 8 channels per 16-byte load, all rows in flight at once
+    // (a real decode step has 32 tail tokens on average)
+    constexpr int LPT = NT / 64;              // lanes per token (the rest buffer holds at most 64 tokens)
+    constexpr int NKV = (D / 8 + LPT - 1) / LPT;
+    const int tr = tid / LPT, tj = tid % LPT;
+    u32x4 tkw[NKV], tqw[NKV];
+    {
+        const unsigned short *krow = (tr == newest && a.persist) ? knew : a.restk + (((int64_t)b * cb + tr) * Hkv + h) * D;
+#pragma unroll
+        for (int i = 0; i < NKV; ++i) {
+            const int v8 = tj + i * LPT;
+            const bool on = tr < nrest && v8 < D / 8;
+            tkw[i] = on ? *reinterpret_cast<const u32x4 *>(krow + v8 * 8) : (u32x4){0u, 0u, 0u, 0u};
+            tqw[i] = on ? *reinterpret_cast<const u32x4 *>(qrow + v8 * 8) : (u32x4){0u, 0u, 0u, 0u};
+        }
+    }
+    // (a) append the token: rest buffers and column maxima (extension/k_cache_file.py:98-101).
+    //     vcm_mine: this thread's channel of the V column maxima after the update (threads < D).
+    static_assert(D <= NT, "one channel per thread");
+    u32 vcm_mine = 0;
+    {
+        const bool on = tid < D;
+        const int d = on ? tid : 0;
+        u32 kc = a.kcm[(int64_t)bh_kv * D + d], vc = a.vcm[(int64_t)bh_kv * D + d];
+        const u32 kb = knew[d], vb = vnew[d];
+        __builtin_amdgcn_sched_barrier(0);
+        hook();
+        __builtin_amdgcn_sched_barrier(0);
+        if (a.persist) {
+            // every query head of the group derives the updated maxima itself (max is idempotent, so it does
+            // not matter whether it reads them before or after the owner's store); only the owner stores
+            kc = max(kc, exp_field(kb));
+            vc = max(vc, exp_field(vb));
+            if (owner && on) {
+                const int64_t at = (((int64_t)b * cb + newest) * Hkv + h) * D + d;
+                a.restk[at] = (unsigned short)kb;
+                a.restv[at] = (unsigned short)vb;
+                a.kcm[(int64_t)bh_kv * D + d] = (uint8_t)kc;
+                a.vcm[(int64_t)bh_kv * D + d] = (uint8_t)vc;
+            }
+        }
+        vcm_mine = vc;
+    }
+    // (b) scores of the tail: fp16(fp16(q.k) / sqrt(D)), the two roundings of an fp16 matmul followed by
+    //     an fp16 division (extension/k_cache_file.py:156)
+    const float sqrt_d = sqrtf((float)D);
+    {
+        float part = 0.f;
+#pragma unroll
+        for (int i = 0; i < NKV; ++i) {
+            const u32 kk[4] = {tkw[i].x, tkw[i].y, tkw[i].z, tkw[i].w}, qq[4] = {tqw[i].x, tqw[i].y, tqw[i].z, tqw[i].w};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                part = fmaf(lo_half_to_float(kk[c]), lo_half_to_float(qq[c]), part);
+                part = fmaf(hi_half_to_float(kk[c]), hi_half_to_float(qq[c]), part);
+            }
+        }
+#pragma unroll
+        for (int mk = 1; mk < LPT; mk <<= 1) part += __shfl_xor(part, mk, 64);
+        if (tr < nrest && tj == 0) {
+            const float dot16 = half_bits_to_float(float_to_half_bits(part));
+            const unsigned short sc = float_to_half_bits(dot16 / sqrt_d);
+            tail_s[tr] = sc;
+            srow[R + tr] = sc;
+        }
+    }
+    lds_barrier();
+
+    // (c) softmax over [0, R + nrest): scores + mask in fp16, softmax in fp32, probabilities in fp16
+    //     (model/KVCache_AlignedKV.py:119-121), and the running arg-max of the residue classes mod 32:
+    //     vector i holds tokens 8i..8i+7, a thread's vectors are 256 apart, so its j-th token always has
+    //     residue (8*(tid&3) + j) mod 32.
+    auto masked1 = [&](u32 sbits, int t) -> float {
+        if (mrow == nullptr) return half_bits_to_float(sbits);
+        return half_bits_to_float(float_to_half_bits(half_bits_to_float(sbits) + half_bits_to_float(mrow[t])));
+    };
+    // arg-max key of a token: probability bits (fp16 of a non-negative number: ordered like an integer)
+    // in the high half, 0xFFFF - (token / 32) in the low half: the largest key is the largest probability
+    // and, among equals, the smallest token (first maximal index, as torch.max returns it)
+    u32 best[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) best[j] = 0u;
+    const float xt = tid < nrest ? masked1(tail_s[tid], R + tid) : -INFINITY;
+    float m = xt, sum = 0.f;
+    if (in_regs) {
+        float x[VPT][8];
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int i = tid + NT * v;
+            if (i < nvec) {
+                decode_scores8(sv[v], mrow, i * 8, x[v]);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) m = fmaxf(m, x[v][j]);
+            }
+        }
+        m = block_reduce<NW>(m, true, red);
+#pragma unroll
+        for (int v = 0; v < VPT; ++v)
+            if (tid + NT * v < nvec) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    x[v][j] = expf(x[v][j] - m);
+                    sum += x[v][j];
+                }
+            }
+        const float et = tid < nrest ? expf(xt - m) : 0.f;
+        sum = block_reduce<NW>(sum + et, false, red);
+        const float rsum = 1.0f / sum;
+#pragma unroll
+        for (int v = 0; v < VPT; ++v) {
+            const int i = tid + NT * v;
+            if (i < nvec) {
+                u32 out[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const u32 p0 = float_to_half_bits(div_by(x[v][2 * j], sum, rsum)), p1 = float_to_half_bits(div_by(x[v][2 * j + 1], sum, rsum));
+                    out[j] = p0 | (p1 << 16);
+                    const u32 grp = 0xffffu - (u32)(i >> 2);     // token / 32 = vector index / 4
+                    best[2 * j] = max(best[2 * j], (p0 << 16) | grp);
+                    best[2 * j + 1] = max(best[2 * j + 1], (p1 << 16) | grp);
+                }
+                const u32x4 o = {out[0], out[1], out[2], out[3]};
+                store_probs8(i, o);
+            }
+        }
+        if (tid < nrest) {
+            const unsigned short p = float_to_half_bits(div_by(et, sum, rsum));
+            store_prob1(R + tid, p);
+            tail_p[tid] = half_bits_to_float(p);
+        }
+    } else {
+        // long rows: three passes over the scores (they stay in the L2 of this workgroup's XCD)
+        float x[8];
+        for (int i = tid; i < nvec; i += NT) {
+            decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) m = fmaxf(m, x[j]);
+        }
+        m = block_reduce<NW>(m, true, red);
+        for (int i = tid; i < nvec; i += NT) {
+            decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) sum += expf(x[j] - m);
+        }
+        const float et = tid < nrest ? expf(xt - m) : 0.f;
+        sum = block_reduce<NW>(sum + et, false, red);
+        const float rsum = 1.0f / sum;
+        for (int i = tid; i < nvec; i += NT) {
+            decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
+            u32 out[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const u32 p0 = float_to_half_bits(div_by(expf(x[2 * j] - m), sum, rsum)), p1 = float_to_half_bits(div_by(expf(x[2 * j + 1] - m), sum, rsum));
+                out[j] = p0 | (p1 << 16);
+                const u32 grp = 0xffffu - (u32)(i >> 2);
+                best[2 * j] = max(best[2 * j], (p0 << 16) | grp);
+                best[2 * j + 1] = max(best[2 * j + 1], (p1 << 16) | grp);
+            }
+            const u32x4 o = {out[0], out[1], out[2], out[3]};
+            store_probs8(i, o);
+        }
+        if (tid < nrest) {
+            const unsigned short p = float_to_half_bits(div_by(et, sum, rsum));
+            store_prob1(R + tid, p);
+            tail_p[tid] = half_bits_to_float(p);
+        }
+    }
+
+    // value rows of the tail, used by (f): requested here so that they travel while the probe runs
+    constexpr int VPR = D / 8;                // 16-byte vectors per row
+    constexpr int NRG = NT / VPR;             // row groups
+    constexpr int MAXR = (64 + NRG - 1) / NRG;
+    static_assert(VPR <= 32, "head_dim above 256 needs another tail mapping");
+    const int c8 = tid % VPR, rg = tid / VPR;
+    u32x4 tvw[MAXR];
+#pragma unroll
+    for (int k = 0; k < MAXR; ++k) {
+        const int r = rg + k * NRG;
+        const unsigned short *vrow = (r == newest && a.persist) ? vnew : a.restv + (((int64_t)b * cb + r) * Hkv + h) * D;
+        tvw[k] = r < nrest ? *reinterpret_cast<const u32x4 *>(vrow + c8 * 8) : (u32x4){0u, 0u, 0u, 0u};
+    }
+
+    // (d)+(e) probe over the flushed part (extension/v_cache_file.py:119-143) and the alignment threshold
+    //     of this (batch, head) (extension/v_cache_file.py:156-160)
+    if (R > 0) {
+        // thread tid saw residues 8*(tid&3)+j.  Lanes of a wave that share (tid&3): two row rotations (DPP)
+        // inside a 16-lane row, two shuffles across rows; then one LDS row per wave and a last scan.
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            best[j] = max(best[j], (u32)__builtin_amdgcn_update_dpp(0, (int)best[j], 0x124, 0xf, 0xf, false));   // row_ror:4
+            best[j] = max(best[j], (u32)__builtin_amdgcn_update_dpp(0, (int)best[j], 0x128, 0xf, 0xf, false));   // row_ror:8
+            best[j] = max(best[j], (u32)__shfl_xor((int)best[j], 16, 64));
+            best[j] = max(best[j], (u32)__shfl_xor((int)best[j], 32, 64));
+        }
+        if (lane < 4) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) cand_key[wave][8 * lane + j] = best[j];
+        }
+        lds_barrier();
+        if (tid < 32) {
+            u32 key = 0u;
+#pragma unroll
+            for (int k = 0; k < NW; ++k) key = max(key, cand_key[k][tid]);
+            probe_p[tid] = half_bits_to_float(key >> 16);
+            probe_t[tid] = (int)(0xffffu - (key & 0xffffu)) * 32 + tid;
+        }
+        lds_barrier();
+        u32 align = 0xffu;
+        for (int d = tid; d < D; d += NT) {
+            // the 32 gathered bytes first, then the sum: 32 independent loads in flight instead of a chain
+            u32 hi[32];
+#pragma unroll
+            for (int i = 0; i < 32; ++i) hi[i] = a.v_first_8[((int64_t)bh_kv * a.g.max_seq_len + probe_t[i]) * D + d];
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < 32; ++i)
+                acc = fmaf(half_bits_to_float(((hi[i] << 8) | 0x80u) & 0x7fffu), probe_p[i], acc);
+            // exponent with the lowest bit cleared (`& 0x1F - 1`, extension/v_cache_file.py:142)
+            const u32 e = exp_field(float_to_half_bits(acc)) & 0x1eu;
+            a.toe[(int64_t)bh * D + d] = (uint8_t)e;
+            align = min(align, (e + 15u - vcm_mine) & 0xffu);     // uint8 wrap, as the reference's tensor arithmetic
+        }
+#pragma unroll
+        for (int mk = 32; mk >= 1; mk >>= 1) align = min(align, (u32)__shfl_xor((int)align, mk, 64));
+        if (lane == 0) red_min[wave] = align;
+        lds_barrier();
+        if (tid == 0) {
+            u32 mn = red_min[0];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) mn = min(mn, red_min[w]);
+            if constexpr (DEV) __builtin_amdgcn_raw_buffer_store_b8((unsigned char)mn, make_rsrc(a.amin + bh, 1u), 0, 0, kDeviceScope);
+            else a.amin[bh] = (uint8_t)mn;
+            if (amin_lds != nullptr) *amin_lds = mn;   // for a caller that goes on in the same workgroup
+        }
+    } else {
+        lds_barrier();
+    }
+    // (f) the tail's share of the output, an fp16 matmul result (extension/v_cache_file.py:189): a thread takes 8
+    //     channels of every NRG-th tail token (requested before the probe), lanes of a wave that share the channels
+    //     fold by shuffles, waves by LDS
+    {
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int k = 0; k < MAXR; ++k) {
+            const int r = rg + k * NRG;
+            const u32 vv[4] = {tvw[k].x, tvw[k].y, tvw[k].z, tvw[k].w};
+            const float pr = r < nrest ? tail_p[r] : 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[2 * i] = fmaf(lo_half_to_float(vv[i]), pr, acc[2 * i]);
+                acc[2 * i + 1] = fmaf(hi_half_to_float(vv[i]), pr, acc[2 * i + 1]);
+            }
+        }
+#pragma unroll
+        for (int mk = VPR; mk < 64; mk <<= 1)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] += __shfl_xor(acc[i], mk, 64);
+        if (lane < VPR) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) tail_o[wave][c8 * 8 + i] = acc[i];
+        }
+        lds_barrier();
+        for (int d = tid; d < D; d += NT) {
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) sum += tail_o[w][d];
+            if constexpr (DEV) store_u16_device(make_rsrc(a.otail + (int64_t)bh * D, (u32)D * 2), d * 2, float_to_half_bits(sum));
+            else a.otail[(int64_t)bh * D + d] = float_to_half_bits(sum);
+        }
+    }
+}
+
+// The step as one launch (akv_onelaunch.hip).
+bool one_launch_covers(int D, int kb, int rows, int R);
+template <int D>
+int launch_one_launch_step(const uint8_t *kf8, const uint8_t *km4, const uint8_t *kl4, const uint8_t *vf8, const uint8_t *vm4,
+                           const uint8_t *vl4, const MiddleArgs &ma, float *partial, unsigned short *out, uint8_t *k_levels_out,
+                           uint8_t *v_levels_out, uint8_t *amin_out, int rows, int R, int kb, bool ref, float scale,
+                           hipStream_t st, bool *launched);
+
+}  // namespace akv
