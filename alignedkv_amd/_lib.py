@@ -35,7 +35,6 @@ SIGNATURES = {
     "akv_profile_read_empty": (c_int, [_P]),
     "akv_decode_step_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "akv_decode_step": (c_int, [_P] * 14 + [_I] + [_P] * 3 + [_I, _P, c_size_t] + [_P] * 3 + [_I] * 12 + [_P]),
-    "akv_decode_step_timeouts": (c_int, [_P, _P]),
     "akv_decode_step_static": (c_int, [_P] * 14 + [_I] + [_P] * 3 + [_I] + [_P] * 3 + [_I] * 12 + [_P]),
 }
 

@@ -394,7 +394,7 @@ __device__ unsigned long long *g_tail_trace = nullptr;
 // compute units (or a multiple of them) every unit streams one row of V planes from start to end: no partial sums,
 // no combine launch, and the first high-byte tiles of every wave travel while the middle stage runs.
 // grid (B*H), 512 threads.
-template <int D, bool REF, int NR, int PF, int NT, int PRE = 0>
+template <int D, bool REF, int NR, int PF, int NT>
 __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict__ v_first_8,
                                                         const uint8_t *__restrict__ v_mid_4,
                                                         const uint8_t *__restrict__ v_last_4, MiddleArgs ma,
@@ -424,19 +424,7 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     seq.n_halves = (R + VStream<D>::HT - 1) / VStream<D>::HT;
     seq.n_per_wave = (seq.n_halves + NW - 1) / NW;
     VRing<D, NR> ring;
-    // PRE > 0: every wave requests its first PRE half tiles of high bytes before the middle stage (they depend on nothing)
-    // and keeps them in registers: PRE * 4 KiB per wave travel while the softmax and the probe run and HBM would idle
-    VHighPart<VStream<D>::HV> pre[PRE > 0 ? PRE : 1];
-    middle_body<D, NT>(ma, bh, &row_amin, [&]() {
-        if constexpr (PRE > 0) {
-            const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)R * D);
-#pragma unroll
-            for (int j = 0; j < PRE; ++j) v_stream_issue_high<D>(pre[j], rH, seq.half(j));
-            __builtin_amdgcn_sched_barrier(0);
-        } else {
-            v_stream_prefetch<D, NR, PF>(ring, f8, R, seq);
-        }
-    });
+    middle_body<D, NT>(ma, bh, &row_amin, [&]() { v_stream_prefetch<D, NR, PF>(ring, f8, R, seq); });
     AKV_TAIL_MARK(1);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
@@ -459,13 +447,12 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
         AKV_TAIL_MARK(3);
         if (n_fine * 16 <= seq.n_per_wave * VStream<D>::HT) {
             int count = 0;
-            v_stream_run_deferred<D, 2, (PRE > 0 ? 0 : PF), NR, PRE>(ring, f8, R, prow, amin, seq, acc, fine_list[wave], count, pre);
+            v_stream_run_deferred<D, 2, PF, NR>(ring, f8, R, prow, amin, seq, acc, fine_list[wave], count);
             AKV_TAIL_MARK(4);
             v_stream_apply_list<D>(f8, m4, l4, R, amin, acc, fine_list[wave], count);
             AKV_TAIL_MARK(5);
         } else {
-            // (the tiles requested early are not used here: this loop takes the nibble rows along from the start)
-            v_stream_run<D, REF, NR, (PRE > 0 ? 0 : PF)>(ring, f8, m4, l4, R, prow, amin, seq, acc);
+            v_stream_run<D, REF, NR, PF>(ring, f8, m4, l4, R, prow, amin, seq, acc);
         }
     }
     if (v_levels_out != nullptr)
@@ -711,22 +698,6 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     ma.kcm = kcm; ma.vcm = vcm; ma.toe = toe; ma.amin = amin; ma.v_first_8 = vf8;
     ma.g = geo; ma.mask_stride = mask_stride; ma.top_k = top_k; ma.persist = persist;
     mark(0, st);
-    // The whole step as one launch of resident workgroups (akv_onelaunch.hip) where it applies: one query head per KV
-    // head, one length for all sequences, head_dim 64 or 128.
-    if constexpr (D <= 128) {
-        bool one = geo.G == 1 && !ragged && !(literal_broadcast && !ref) && n_blocks > 0 && one_launch_covers(D, kb, B * Hq, R);
-        { AKV_TUNE("AKV_TUNE_ONE_LAUNCH", v); one = one && has_v && v != 0; }
-        if (one) {
-            bool launched = false;
-            const int rc = launch_one_launch_step<D>(kf8, km4, kl4, vf8, vm4, vl4, ma, partial, reinterpret_cast<unsigned short *>(out),
-                                                     k_levels_out, v_levels_out, amin_out, B * Hq, R, kb, ref, scale, st, &launched);
-            if (rc != AKV_OK) return rc;
-            if (launched) {
-                for (int i = 1; i <= 6; ++i) mark(i, st);
-                return AKV_OK;
-            }
-        }
-    }
     if (n_blocks > 0 && matrix) {
         int rc = AKV_OK;
         if constexpr (D <= 128)
@@ -804,19 +775,9 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (ref)
             hipLaunchKernelGGL((tail_step_kernel<D, true, 4, 3, 512>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
                                reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out);
-        else {
-            int pre = 0;
-            { AKV_TUNE("AKV_TUNE_TAIL_PRE", v); if (has_v) pre = v; }
-#define AKV_TAIL(PRE) hipLaunchKernelGGL((tail_step_kernel<D, false, 4, 1, 512, PRE>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma, \
-                                         reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out)
-            if (pre == 2) AKV_TAIL(2);
-            else if (pre == 3) AKV_TAIL(3);
-            else if (pre == 4) AKV_TAIL(4);
-            else if (pre == 6) AKV_TAIL(6);
-            else if (pre == 8) AKV_TAIL(8);
-            else AKV_TAIL(0);
-#undef AKV_TAIL
-        }
+        else
+            hipLaunchKernelGGL((tail_step_kernel<D, false, 4, 1, 512>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
+                               reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out);
         mark(2, st);
         mark(3, st);
         mark(4, st);

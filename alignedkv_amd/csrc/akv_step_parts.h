@@ -1,6 +1,5 @@
-// Device-side building blocks of the fused decode step, shared by its multi-launch form (akv_fused.hip) and its
-// one-launch form (akv_onelaunch.hip): the K pass over one 256-token stretch of a (batch, head) row, the middle stage
-// of a row (append, tail scores, softmax, probe, threshold, tail output) and the pieces of the V pass.
+// Device-side building blocks of the fused decode step (akv_fused.hip): the K pass over one 256-token stretch of a
+// (batch, head) row and the middle stage of a row (append, tail scores, softmax, probe, threshold, tail output).
 #pragma once
 
 #include "akv_step.h"
@@ -534,13 +533,5 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
         }
     }
 }
-
-// The step as one launch (akv_onelaunch.hip).
-bool one_launch_covers(int D, int kb, int rows, int R);
-template <int D>
-int launch_one_launch_step(const uint8_t *kf8, const uint8_t *km4, const uint8_t *kl4, const uint8_t *vf8, const uint8_t *vm4,
-                           const uint8_t *vl4, const MiddleArgs &ma, float *partial, unsigned short *out, uint8_t *k_levels_out,
-                           uint8_t *v_levels_out, uint8_t *amin_out, int rows, int R, int kb, bool ref, float scale,
-                           hipStream_t st, bool *launched);
 
 }  // namespace akv

@@ -178,15 +178,6 @@ AKV_API int akv_decode_step_static(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t
                                    int literal_broadcast, akv_stream_t stream);
 
 /*
- * No counterpart in the reference.  Where it applies (one query head per KV head, one length for all sequences,
- * head_dim 64 or 128) akv_decode_step runs as one launch whose workgroups hand work on to each other through counters in
- * device memory; a workgroup that waits for a row polls a bounded number of times, then gives up and counts that here.
- * Waits for `stream` and returns the number of such give-ups since the process started (0 in normal operation; a
- * non-zero count means some step on this stream left part of its output unwritten).
- */
-AKV_API int akv_decode_step_timeouts(akv_stream_t stream, unsigned int *timeouts);
-
-/*
  * The fused decode step for grouped-query attention and per-sequence lengths; beyond the reference, which
  * asserts multi-head attention and keeps one scalar length per layer (model/KVCache_AlignedKV.py:32,
  * extension/k_cache_file.py:133, extension/v_cache_file.py:146).  Per query head the algorithm is the
