@@ -26,11 +26,60 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0   # MI355X published HBM3E bandwidth
 
-# HBM bytes per launch of the K pass at the default workload, from the rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs summarised in profiles/decode_step_c2_hbm_traffic.txt (256-token K blocks) and decode_step_c2_k_block64_hbm_traffic.txt (FETCH_SIZE scaled x2.0 by the
-# known-size copy kernel, WRITE_SIZE x1.0): 222.4 MiB read + 2.0 MiB written.
-MEASURED_K_PASS_TRAFFIC = {(8, 32, 128, 4096, "outlier", 64): int((222.4 + 2.0) * (1 << 20)),
-                           (8, 32, 128, 4096, "outlier", 256): int((198.5 + 2.0) * (1 << 20))}
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def profile_figures(name):
+    """Per-kernel figures of a tracked rocprofv3 summary under profiles/ (`<name>_kernel_stats.txt`: average duration in
+    us; `<name>_hbm_traffic.txt`: MiB fetched and written per dispatch, already scaled by the known-size copy kernel).
+    Returns {kernel: {"avg_us", "fetch_mib", "write_mib"}}; empty when the summaries are not there.  The benchmark
+    prints them beside what it measures itself, so a summary that no longer matches the kernels shows up as a mismatch."""
+    out = {}
+    try:
+        for line in open(os.path.join(PROFILES, name + "_kernel_stats.txt")):
+            f = line.split()
+            if len(f) >= 5 and (line.startswith("akv::") or line.startswith("copy_probe")):
+                kernel = line[:line.index(f[-4])].strip()
+                out.setdefault(kernel, {})["avg_us"] = float(f[-3])
+        for line in open(os.path.join(PROFILES, name + "_hbm_traffic.txt")):
+            f = line.split()
+            if len(f) >= 6 and (line.startswith("akv::") or line.startswith("copy_probe")):
+                kernel = line[:line.index(f[-5])].strip()
+                out.setdefault(kernel, {}).update(fetch_mib=float(f[-3]), write_mib=float(f[-1]))
+    except (OSError, ValueError):
+        pass
+    return out
+
+
+def roofline_entry(kernel, algorithmic_bytes, event_us, event_pair_us, prof):
+    """Roofline of one kernel: algorithmic bytes per launch over its average launch duration.  The duration is
+    measured live with HIP events on the step's stream (interval minus the interval of an empty event pair); when the
+    tracked rocprofv3 summary has this kernel, the longer of the two durations is used, so `frac` never exceeds what the
+    committed profile supports.  `traffic` = HBM bytes per launch from the tracked FETCH_SIZE / WRITE_SIZE summary."""
+    live = max(event_us - event_pair_us, 1e-3)
+    prof_us = prof.get("avg_us")
+    used = max(live, prof_us) if prof_us else live
+    achieved = algorithmic_bytes / (used * 1e-6) / 1e9
+    traffic = None
+    if "fetch_mib" in prof:
+        traffic = int((prof["fetch_mib"] + prof.get("write_mib", 0.0)) * (1 << 20))
+    return {"kernel": kernel, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+            "algorithmic_bytes_per_launch": int(algorithmic_bytes), "avg_launch_us": round(used, 2),
+            "duration_source": "rocprofv3 summary under profiles/ (longer than the live measurement)" if used != live
+            else "HIP events on the step's stream minus an empty event pair",
+            "hip_event_interval_us": round(event_us, 2), "event_pair_overhead_us": round(event_pair_us, 2),
+            "rocprof_avg_launch_us": prof_us}
 
 
 def parse():
@@ -125,6 +174,26 @@ def time_steps(torch, runners, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+def step_percentiles(torch, runners, steps, batch=20):
+    """us/step over batches of `batch` consecutive steps (events on the current stream between the batches, one
+    synchronisation at the end): p10 / median / p90 of the batch means."""
+    n = len(runners)
+    nb = max(steps // batch, 5)
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(nb + 1)]
+    ev[0].record()
+    k = 0
+    for b in range(nb):
+        for _ in range(batch):
+            runners[k % n]()
+            k += 1
+        ev[b + 1].record()
+    torch.cuda.synchronize()
+    us = sorted(ev[b].elapsed_time(ev[b + 1]) * 1e3 / batch for b in range(nb))
+    pick = lambda f: us[min(len(us) - 1, int(f * len(us)))]
+    return {"p10": round(pick(0.1), 2), "median": round(pick(0.5), 2), "p90": round(pick(0.9), 2),
+            "sample": "%d batches of %d consecutive steps, HIP events between batches" % (nb, batch)}
+
+
 def phase_times(torch, lib, runners, steps):
     """Average duration (us) of the four kernels of the step, HIP events on the step's stream."""
     import ctypes
@@ -144,8 +213,8 @@ def phase_times(torch, lib, runners, steps):
             acc[j] += buf[j] * 1e3
         acc[4] += empty.value * 1e3
     lib.akv_profile_enable(0)
-    # an event pair around nothing still measures a few microseconds: take that off every phase
-    return [max(a - acc[4], 0.0) / steps for a in acc[:4]], acc[4] / steps
+    # raw intervals, and what an event pair around nothing measures (a few microseconds)
+    return [a / steps for a in acc[:4]], acc[4] / steps
 
 
 def algorithmic_bytes(k_levels, v_levels, B, H, D, R, L, top_k=32):
@@ -288,6 +357,8 @@ def bench_c3(a):
     buf = (ctypes.c_float * 4)()
     empty = ctypes.c_float()
     acc = [0.0] * 4
+    acc_raw = [0.0] * 4
+    empty_us = 0.0
     n = min(a.steps, 100)
     for i in range(n + 4):
         layer = i % a.layers
@@ -299,7 +370,20 @@ def bench_c3(a):
         if i >= 4:
             for j in range(4):
                 acc[j] += max(buf[j] - empty.value, 0.0) * 1e3 / n
+                acc_raw[j] += buf[j] * 1e3 / n
+            empty_us += empty.value * 1e3 / n
     lib.akv_profile_enable(0)
+    # bytes of the K pass per launch: plane rows at the finest level any query head of the group asks for, q, column
+    # maxima, new keys, scores written
+    k_plane_bytes = 0.0
+    for b in range(B):
+        R = (int(lens[b]) + 1) // cb * cb
+        kl = klv[b].reshape(Hkv, Hq // Hkv, D).min(1)
+        k_plane_bytes += R * (kl.size + 0.5 * (kl < 2).sum() + 0.5 * (kl == 0).sum())
+    k_pass_bytes = k_plane_bytes + B * Hq * D * 2 + B * Hkv * D * 3 + sum((int(l) + 1) // cb * cb for l in lens) * Hq * 2
+    prof = profile_figures("decode_step_c3_gqa") if (a.c3_q_heads == 32 and not a.c3_len and a.k_block == 256) else {}
+    k_kernel = "akv::mfma_k_pass_kernel<%d, false" % D
+    k_prof = next((v for k, v in prof.items() if k.startswith(k_kernel)), {})
     res = {"metric": "decode-attn us/step, grouped-query 32 over 8 heads x 128, batch 32, lengths U[2048,8192]",
            "value": round(sec * 1e6, 2), "unit": "us/step", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
            "ms_per_step": round(sec * 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
@@ -311,8 +395,64 @@ def bench_c3(a):
            "effective_hbm_gbps": round(kv_bytes / sec / 1e9, 1), "pct_hbm_peak": round(100 * kv_bytes / sec / 1e9 / HBM_PEAK_GBPS, 1),
            "kernel_us": {"k_pass": round(acc[0], 2), "middle": round(acc[1], 2), "v_pass": round(acc[2], 2),
                          "combine": round(acc[3], 2)},
-           "dense_in_planes_us": round(sec_ref * 1e6, 2), "speedup_vs_dense_in_planes": round(sec_ref / sec, 3)}
+           "dense_in_planes_us": round(sec_ref * 1e6, 2), "speedup_vs_dense_in_planes": round(sec_ref / sec, 3),
+           "roofline": roofline_entry(k_kernel, k_pass_bytes, acc_raw[0], empty_us, k_prof),
+           "roofline_step": {"bound": "hbm", "achieved": round(kv_bytes / sec / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                             "frac": round(kv_bytes / sec / 1e9 / HBM_PEAK_GBPS, 4), "algorithmic_bytes_per_step": int(kv_bytes),
+                             "us_per_step": round(sec * 1e6, 2), "duration_source": "wall clock around the timed steps"}}
+    if not a.no_cpu:
+        res.update(cpu_baseline_c3(torch, cache, lens, q, k_new, v_new, lens0, bound))
     print(json.dumps(res))
+
+
+def cpu_baseline_c3(torch, cache, lens, q, k_new, v_new, lens0, bound):
+    """The C restatement of the ops (OpenMP) + the NumPy host logic on the host cores for the grouped-query workload: every
+    sequence on its own planes with the KV heads repeated per query head, one full-size step of layer 0 (what the
+    reference's multi-head algorithm does for each query head).  Also the parity of the GPU step against it."""
+    import numpy as np
+    from oracle import akv_oracle_c as OC
+    from tests.common import oracle_decode_step_c
+    B, Hq, Hkv, D, cb, kb = cache.bsz, cache.n_q_heads, cache.n_kv_heads, cache.head_dim, 64, cache.k_block
+    G = Hq // Hkv
+    cache.record_levels = True
+    cache.seq_lens[0].copy_(lens0)
+    cache.len_bound[0] = bound
+    out = cache.decode(0, q, k_new, v_new).cpu().numpy()
+    klv_gpu = cache.last_k_levels.cpu().numpy()
+    cache.record_levels = False
+    OC.lib()
+    rep = lambda x, ax: np.ascontiguousarray(np.repeat(x, G, axis=ax))
+
+    def as_64(plane):      # K plane in blocks of kb tokens -> the same bytes in blocks of 64 tokens
+        if kb == 64:
+            return plane
+        one, H, NB, D_, row = plane.shape
+        sub = kb // 64
+        return np.ascontiguousarray(plane.reshape(one, H, NB, D_, sub, row // sub).transpose(0, 1, 2, 4, 3, 5)).reshape(
+            one, H, NB * sub, D_, row // sub)
+
+    qh, knh, vnh = q.cpu().numpy(), k_new.cpu().numpy(), v_new.cpu().numpy()
+    kcm, vcm = cache.k_colmax[0].cpu().numpy(), cache.v_colmax[0].cpu().numpy()
+    restk, restv = cache.restk[0].cpu().numpy(), cache.restv[0].cpu().numpy()
+    seconds, worst, k_equal = 0.0, 0.0, True
+    for b in range(B):
+        Lb = int(lens[b]) + 1
+        R = Lb // cb * cb
+        n_rest = Lb - R
+        kpl = [rep(as_64(p[b:b + 1].cpu().numpy())[:, :, :R // cb], 1) for p in cache.k_planes[0]]
+        vpl = [rep(p[b:b + 1, :, :R].cpu().numpy(), 1) for p in cache.v_planes[0]]
+        args = (kpl, vpl, rep(kcm[b:b + 1], 2), rep(vcm[b:b + 1], 2), qh[b:b + 1], rep(knh[b:b + 1], 2), rep(vnh[b:b + 1], 2), R)
+        rk, rv = rep(restk[b:b + 1, :n_rest], 2), rep(restv[b:b + 1, :n_rest], 2)
+        t0 = time.perf_counter()
+        want, klv, vlv, amin, p = oracle_decode_step_c(*args, rest_k=rk, rest_v=rv)
+        seconds += time.perf_counter() - t0
+        worst = max(worst, float(np.max(np.abs(out[b:b + 1].astype(np.float32) - want.astype(np.float32)))))
+        k_equal = k_equal and bool(np.array_equal(klv_gpu[b], klv[0]))
+    return {"cpu_baseline": {"value": round(seconds * 1e6, 1), "unit": "us/step", "cores": OC.num_threads(), "kind": "port",
+                             "cpu_model": cpu_model(), "host_cores": os.cpu_count(),
+                             "sample": "one full-size step of layer 0, sequence by sequence (C restatement with OpenMP + NumPy "
+                                       "host logic, KV heads repeated per query head; copies to the host not timed)"},
+            "parity": {"max_abs_err_vs_oracle": worst, "k_levels_equal": k_equal}}
 
 
 def main():
@@ -366,7 +506,10 @@ def main():
     runners = [StepRunner(torch, lib, cache, i, q, k_new, v_new, out, False, i == 0) for i in range(a.layers)]
     sec = time_steps(torch, runners, a.steps, a.warmup)
     us = sec * 1e6
-    out_aligned = out.clone()
+    pct = step_percentiles(torch, runners, a.steps)
+    runners[0]()
+    torch.cuda.synchronize()
+    out_aligned = out.clone()            # layer 0's output
     k_levels = runners[0].k_levels.cpu().numpy()
     v_levels = runners[0].v_levels.cpu().numpy()
 
@@ -375,11 +518,13 @@ def main():
     by = algorithmic_bytes(k_levels, v_levels, B, H, D, R, L + 1)
     eff_gbps = by["total"] / sec / 1e9
 
-    # per-kernel durations (HIP events on the stream) -> roofline of the dominant kernel, the K pass
-    ph, event_pair_us = phase_times(torch, lib, runners, min(a.steps, 200))
+    # per-kernel durations (HIP events on the stream) -> roofline of the step's kernels
+    ph_raw, event_pair_us = phase_times(torch, lib, runners, min(a.steps, 200))
+    ph = [max(x - event_pair_us, 0.0) for x in ph_raw]
     k_pass_bytes = by["k_plane"] + B * H * D * (2 + 1 + 2) + B * H * R * 2     # planes + q, column max, new key + scores
     v_pass_bytes = by["v_plane"] + B * H * R * 2 + B * H * D * 2 + B * H * (R // 256) * D * 4
-    achieved = k_pass_bytes / (ph[0] * 1e-6) / 1e9
+    # everything after the K pass: scores and probabilities, probe rows, V planes, the token's fp16 rows, the output
+    tail_bytes = by["total"] - k_pass_bytes
     # With one row of (batch, head) pairs per compute unit the library runs everything after the K pass as one
     # launch: the second interval then covers it and the last two are empty
     one_launch_tail = ph[2] < 0.5 and ph[3] < 0.5
@@ -407,11 +552,21 @@ def main():
         out2 = torch.empty_like(q)
         runners2 = [StepRunner(torch, lib, cache2, i, q, k_new, v_new, out2, False, False) for i in range(a.layers)]
         sec_other = time_steps(torch, runners2, max(a.steps // 2, 20), 10)
-        # summation order differs, levels do not
+        runners2[0]()
+        torch.cuda.synchronize()
+        # summation order differs, levels do not (both: layer 0)
         other = {"k_block": other_kb, "us_per_step": round(sec_other * 1e6, 2),
                  "max_abs_diff_of_outputs": float((out2.float() - out_aligned.float()).abs().max())}
         del cache2, runners2
 
+    # figures of the tracked rocprofv3 summaries for this exact workload (none for other shapes)
+    default_workload = (B, H, D, L, a.k_kind) == (8, 32, 128, 4096, "outlier")
+    prof = profile_figures("decode_step_c2" + ("" if a.k_block == 256 else "_k_block64")) if default_workload else {}
+    if a.k_block == 64:
+        k_kernel = "akv::fused_k_pass_kernel<%d, false, true>" % D if D <= 128 else "akv::fused_k_pass_kernel<%d, false, false>" % D
+    else:
+        k_kernel = "akv::fused_k_pass256_split_kernel<%d, false, 4>" % D
+    tail_kernel = "akv::tail_step_kernel<%d, false, 4, 1, 512>" % D
     res = {
         "metric": "decode-attn us/step (+ effective HBM GB/s, %% of peak), B=%d L=%d %dx%d" % (B, L, H, D),
         "value": round(us, 2), "unit": "us/step", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -419,6 +574,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "C2: batch %d, %d heads x %d, cache %d + 1 appended token, K %s, %d layers rotated, K plane blocks of %d tokens"
                                % (B, H, D, L, a.k_kind, a.layers, a.k_block)},
+        "us_per_step_percentiles": pct,
         "effective_hbm_gbps": round(eff_gbps, 1), "pct_hbm_peak": round(100 * eff_gbps / HBM_PEAK_GBPS, 1),
         "algorithmic_bytes": int(by["total"]), "dense_fp16_bytes": int(by["dense"]),
         "bytes_vs_dense": round(by["total"] / by["dense"], 4),
@@ -429,11 +585,14 @@ def main():
         "k_block": a.k_block, "other_k_block_us": other,
         "dense_in_planes_us": round(sec_ref * 1e6, 2),
         "speedup_vs_dense_in_planes": round(sec_ref / sec, 3),
-        "roofline": {"kernel": ("fused_k_pass_kernel<%d,false,true>" % D if D <= 128 else "fused_k_pass_kernel<%d,false>" % D) if a.k_block == 64 else "fused_k_pass256_split_kernel<%d,false,4>" % D, "bound": "hbm", "achieved": round(achieved, 1),
-                     "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_K_PASS_TRAFFIC.get((B, H, D, L, a.k_kind, a.k_block)), "algorithmic_bytes_per_launch": int(k_pass_bytes),
-                     "avg_launch_us": round(ph[0], 2), "event_pair_overhead_us": round(event_pair_us, 2)},
+        # the dominant kernel (the K pass), the step's other kernel, and the step as a whole
+        "roofline": roofline_entry(k_kernel, k_pass_bytes, ph_raw[0], event_pair_us, prof.get(k_kernel, {})),
+        "roofline_step": {"bound": "hbm", "achieved": round(eff_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                          "frac": round(eff_gbps / HBM_PEAK_GBPS, 4), "algorithmic_bytes_per_step": int(by["total"]),
+                          "us_per_step": round(us, 2), "duration_source": "wall clock around the timed steps"},
     }
+    if one_launch_tail:
+        res["roofline_tail"] = roofline_entry(tail_kernel, tail_bytes, ph_raw[1], event_pair_us, prof.get(tail_kernel, {}))
     if copy_gbps is not None:
         res["copy_probe_gbps_read_plus_write"] = round(copy_gbps, 1)
     try:
@@ -447,6 +606,7 @@ def main():
         torch.cuda.synchronize()
         err = float(np.max(np.abs(out.cpu().numpy().astype(np.float32) - cpu_out.astype(np.float32))))
         res["cpu_baseline"] = {"value": round(cpu_sec * 1e6, 1), "unit": "us/step", "cores": threads, "kind": "port",
+                               "cpu_model": cpu_model(), "host_cores": os.cpu_count(),
                                "sample": "%d full-size steps of layer 0 (min), C restatement with OpenMP + NumPy host logic"
                                          % a.cpu_steps}
         dsec, dthreads = cpu_dense_torch(torch, B, H, D, L + 1)
