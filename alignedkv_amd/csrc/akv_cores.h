@@ -642,7 +642,8 @@ __device__ __forceinline__ void v_stream_run(VRing<D, NR> &ring, const uint8_t *
 
 // Number of the wave's tokens below level 2: the probabilities of the wave's half tiles, 16 bytes per lane and load;
 // for rows of at most 64 * 16 * 8 / 2 tokens per wave.
-template <int D>
+// LDSP: s_row is a copy of the row's probabilities in LDS (a caller that produced them in the same workgroup).
+template <int D, bool LDSP = false>
 __device__ __forceinline__ int v_stream_count_fine(const unsigned short *s_row, int n_tokens, unsigned char amin, const VSeq &seq) {
     using S = VStream<D>;
     constexpr int UPH = S::HT * 2 / 16;    // 16-byte units of probabilities per half tile
@@ -657,9 +658,11 @@ __device__ __forceinline__ int v_stream_count_fine(const unsigned short *s_row, 
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int f = lane + 64 * j, i = f / UPH, part = f % UPH;
-        const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(rS, (seq.half(i) * S::HT + part * 8) * 2, 0, 0);
-        const u32 ww[4] = {w.x, w.y, w.z, w.w};
         const bool on = seq.half(i) < seq.n_halves;
+        u32x4 w;
+        if constexpr (LDSP) w = on ? *reinterpret_cast<const u32x4 *>(s_row + seq.half(i) * S::HT + part * 8) : (u32x4){0u, 0u, 0u, 0u};
+        else w = __builtin_amdgcn_raw_buffer_load_b128(rS, (seq.half(i) * S::HT + part * 8) * 2, 0, 0);
+        const u32 ww[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
             union { u32 u; u16x2_t v; } x;
@@ -680,59 +683,56 @@ __device__ __forceinline__ int v_stream_count_fine(const unsigned short *s_row, 
 // (v_stream_apply_list).  For rows where they are rare: a listed token costs a second fetch of its high bytes and a
 // share of a memory round trip of its own (at one token in nine the pass takes 52 instead of 30 us).
 // list: LDS, room for every token of the wave (n_per_wave * HT entries); count: its length.
-// PRE > 0: the wave's first PRE half tiles of high bytes were requested long before (`pre`, in registers since before
-// the caller's own set-up: whatever of the row travels while the caller cannot stream yet is time HBM would otherwise
-// idle); they are multiplied first, while the ring's first requests are on their way.
-template <int D, int NR, int PF, int NRING, int PRE = 0>
+// LDSP: s_row is a copy of the row's probabilities in LDS; a half tile's probabilities are then read when it is
+// multiplied instead of travelling with its high bytes (four fewer memory instructions per half tile).
+template <int D, int NR, int PF, int NRING, bool LDSP = false>
 __device__ __forceinline__ void v_stream_run_deferred(VRing<D, NRING> &ring, const uint8_t *f8, int n_tokens,
-                                                     const unsigned short *s_row, unsigned char amin, const VSeq &seq_in,
-                                                     float *acc, u32 *list, int &count,
-                                                     const VHighPart<VStream<D>::HV> *pre = nullptr) {
+                                                     const unsigned short *s_row, unsigned char amin, const VSeq &seq,
+                                                     float *acc, u32 *list, int &count) {
     using S = VStream<D>;
     static_assert(NR >= 2 && NR <= NRING, "one slot is multiplied while the others travel");
-    static_assert(PRE == 0 || PF == 0, "either the ring's first slots or the separate tiles are requested early");
     constexpr int HV = S::HV;
     const int lane = threadIdx.x & 63, tl = lane / S::LPR, cl = lane % S::LPR;
     const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
     const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)n_tokens * 2);
-    // tokens of a half tile below level 2 (one lane per token notes it: the first of its row), then the half tile at level 2
-    auto multiply = [&](const VHighPart<HV> &hi, const u32 *sb, int half) {
-        bool fine[HV];
-        bool any = false;
-#pragma unroll
-        for (int u = 0; u < HV; ++u) {
-            fine[u] = cl == 0 && v_level(amin, (unsigned short)sb[u]) < 2 && sb[u] != 0u;
-            any = any || fine[u];
-        }
-        if (__builtin_amdgcn_ballot_w64(any) != 0ull) {
-            const int base = half * S::HT + tl;
-#pragma unroll
-            for (int u = 0; u < HV; ++u) VListed<D>::append(list, count, fine[u], base + u * S::TPL, sb[u]);
-        }
-        v_compute_half_coarse<HV>(acc, hi, sb);
-        pin_accumulators(acc);
+    auto issue = [&](int k, int half) {
+        if constexpr (LDSP) v_stream_issue_high<D>(ring.hi[k], rH, half);
+        else v_stream_issue<D, NRING>(ring, k, rH, rS, half);
     };
-    u32 psb[PRE > 0 ? PRE : 1][HV];
-#pragma unroll
-    for (int j = 0; j < PRE; ++j) v_stream_issue_probs<D>(psb[j], rS, seq_in.half(j));
-    VSeq seq = seq_in;
-    seq.first += PRE;
 #pragma unroll
     for (int k = PF; k < NR - 1; ++k) v_stream_issue_high<D>(ring.hi[k], rH, seq.half(k));
+    if constexpr (!LDSP) {
 #pragma unroll
-    for (int k = 0; k < NR - 1; ++k) v_stream_issue_probs<D>(ring.sb[k], rS, seq.half(k));
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int j = 0; j < PRE; ++j) {
-        multiply(pre[j], psb[j], seq_in.half(j));
-        __builtin_amdgcn_sched_barrier(0);
+        for (int k = 0; k < NR - 1; ++k) v_stream_issue_probs<D>(ring.sb[k], rS, seq.half(k));
     }
+    __builtin_amdgcn_sched_barrier(0);
     auto round = [&](int i0) {
 #pragma unroll
         for (int k = 0; k < NR; ++k) {
-            v_stream_issue<D, NRING>(ring, (k + NR - 1) % NR, rH, rS, seq.half(i0 + k + NR - 1));
+            issue((k + NR - 1) % NR, seq.half(i0 + k + NR - 1));
             __builtin_amdgcn_sched_barrier(0);
-            multiply(ring.hi[k], ring.sb[k], seq.half(i0 + k));
+            const int half = seq.half(i0 + k);
+            if constexpr (LDSP) {
+                // (a half tile past the wave's share: its high bytes came back as zeros, its probabilities count as zeros)
+                const bool on = half < seq.n_halves;
+#pragma unroll
+                for (int u = 0; u < HV; ++u) ring.sb[k][u] = on ? (u32)s_row[half * S::HT + tl + u * S::TPL] : 0u;
+            }
+            // tokens of this half tile below level 2 (one lane per token notes it: the first of its row)
+            bool fine[HV];
+            bool any = false;
+#pragma unroll
+            for (int u = 0; u < HV; ++u) {
+                fine[u] = cl == 0 && v_level(amin, (unsigned short)ring.sb[k][u]) < 2 && ring.sb[k][u] != 0u;
+                any = any || fine[u];
+            }
+            if (__builtin_amdgcn_ballot_w64(any) != 0ull) {
+                const int base = half * S::HT + tl;
+#pragma unroll
+                for (int u = 0; u < HV; ++u) VListed<D>::append(list, count, fine[u], base + u * S::TPL, ring.sb[k][u]);
+            }
+            v_compute_half_coarse<HV>(acc, ring.hi[k], ring.sb[k]);
+            pin_accumulators(acc);
             __builtin_amdgcn_sched_barrier(0);
         }
     };

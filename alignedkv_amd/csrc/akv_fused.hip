@@ -381,13 +381,6 @@ __global__ __launch_bounds__(NT) void fused_middle_kernel(MiddleArgs a) {
 
 constexpr int tail_rows_per_cu = 2, tail_max_tokens = 8192;
 
-#ifdef AKV_TRACE
-// Development aid (not compiled into the library): per workgroup, timestamps of the phases of tail_step_kernel.
-__device__ unsigned long long *g_tail_trace = nullptr;
-#define AKV_TAIL_MARK(i) do { if (g_tail_trace != nullptr && threadIdx.x == 0) g_tail_trace[(size_t)blockIdx.x * 16 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
-#else
-#define AKV_TAIL_MARK(i) do { } while (0)
-#endif
 
 // Second half of a step in one launch: the middle stage, the V pass and the final sum for one (batch, head) per
 // workgroup of 8 waves, after a K pass that ran as a launch of its own.  With about as many (batch, head) pairs as
@@ -411,7 +404,7 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     if (g_tail_trace != nullptr && threadIdx.x == 0) {
         unsigned xcc;
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        g_tail_trace[(size_t)blockIdx.x * 16 + 8] = xcc;
+        g_tail_trace[(size_t)blockIdx.x * 24 + 8] = xcc;
     }
 #endif
     int R, nrest_unused;
@@ -424,7 +417,9 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     seq.n_halves = (R + VStream<D>::HT - 1) / VStream<D>::HT;
     seq.n_per_wave = (seq.n_halves + NW - 1) / NW;
     VRing<D, NR> ring;
-    middle_body<D, NT>(ma, bh, &row_amin, [&]() { v_stream_prefetch<D, NR, PF>(ring, f8, R, seq); });
+    // the row's probabilities stay in LDS for the V part (the copy in memory is the step's debug output)
+    __shared__ __attribute__((aligned(16))) unsigned short probs_lds[tail_max_tokens + 64];
+    middle_body<D, NT>(ma, bh, &row_amin, [&]() { v_stream_prefetch<D, NR, PF>(ring, f8, R, seq); }, probs_lds);
     AKV_TAIL_MARK(1);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
@@ -443,11 +438,11 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
         // heads x 4096 tokens).  More than one in 16 among the wave's tokens (flat attention): the loop that takes
         // their nibble rows along with the half tiles, ring of NR.  (A row has at most tail_max_tokens flushed tokens.)
         __shared__ u32 fine_list[NW][tail_max_tokens / NW];
-        const int n_fine = v_stream_count_fine<D>(prow, R, amin, seq);
+        const int n_fine = v_stream_count_fine<D, true>(probs_lds, R, amin, seq);
         AKV_TAIL_MARK(3);
         if (n_fine * 16 <= seq.n_per_wave * VStream<D>::HT) {
             int count = 0;
-            v_stream_run_deferred<D, 2, PF, NR>(ring, f8, R, prow, amin, seq, acc, fine_list[wave], count);
+            v_stream_run_deferred<D, 2, PF, NR, true>(ring, f8, R, probs_lds, amin, seq, acc, fine_list[wave], count);
             AKV_TAIL_MARK(4);
             v_stream_apply_list<D>(f8, m4, l4, R, amin, acc, fine_list[wave], count);
             AKV_TAIL_MARK(5);

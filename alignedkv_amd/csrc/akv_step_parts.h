@@ -6,6 +6,14 @@
 
 namespace akv {
 
+#ifdef AKV_TRACE
+// Development aid (not compiled into the library): per workgroup, timestamps of the phases of tail_step_kernel.
+__device__ unsigned long long *g_tail_trace = nullptr;
+#define AKV_TAIL_MARK(i) do { if (g_tail_trace != nullptr && threadIdx.x == 0) g_tail_trace[(size_t)blockIdx.x * 24 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
+#else
+#define AKV_TAIL_MARK(i) do { } while (0)
+#endif
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
@@ -170,8 +178,11 @@ struct NoHook {
 // workgroup requests its own data there: loads return in order, so these come back first)
 // DEV: what later stages read (probabilities, threshold, tail output) is stored at device scope, for a launch whose
 // other workgroups -- on other XCDs, with L2 caches of their own -- go on with the row
+// probs_lds (may be null): LDS copy of the row's probabilities, tokens 0 .. R + tail, for a caller that goes on in the
+// same workgroup
 template <int D, int NT, typename Hook = NoHook, bool DEV = false>
-__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u32 *amin_lds = nullptr, Hook hook = Hook());
+__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u32 *amin_lds = nullptr, Hook hook = Hook(),
+                                            unsigned short *probs_lds = nullptr);
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
 // global store of the wave (here: 8 KiB of probabilities on their way to memory), which nobody inside the
@@ -210,7 +221,7 @@ __device__ __forceinline__ void decode_scores8(const u32x4 w, const unsigned sho
 
 // NT threads (a multiple of 256) of one workgroup run the stage for one (batch, head).
 template <int D, int NT, typename Hook, bool DEV>
-__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u32 *amin_lds, Hook hook) {
+__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u32 *amin_lds, Hook hook, unsigned short *probs_lds) {
     constexpr int VPT = 4;                    // 16-byte score vectors a thread keeps in registers
     constexpr int NW = NT / 64;               // waves
     __shared__ float red[NW];
@@ -242,10 +253,12 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
     const __amdgpu_buffer_rsrc_t rScores = make_rsrc(srow, (u32)R * 2);
     const __amdgpu_buffer_rsrc_t rProbs = make_rsrc(prow, (u32)(R + nrest) * 2);
     auto store_probs8 = [&](int i, const u32x4 o) {
+        if (probs_lds != nullptr) *reinterpret_cast<u32x4 *>(probs_lds + i * 8) = o;
         if constexpr (DEV) __builtin_amdgcn_raw_buffer_store_b128(o, rProbs, i * 16, 0, kDeviceScope);
         else *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
     };
     auto store_prob1 = [&](int t, unsigned short p) {
+        if (probs_lds != nullptr) probs_lds[t] = p;
         if constexpr (DEV) store_u16_device(rProbs, t * 2, p);
         else prow[t] = p;
     };
@@ -327,6 +340,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
         }
     }
     lds_barrier();
+    AKV_TAIL_MARK(10);
 
     // (c) softmax over [0, R + nrest): scores + mask in fp16, softmax in fp32, probabilities in fp16
     //     (model/KVCache_AlignedKV.py:119-121), and the running arg-max of the residue classes mod 32:
@@ -356,6 +370,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
             }
         }
         m = block_reduce<NW>(m, true, red);
+        AKV_TAIL_MARK(11);
 #pragma unroll
         for (int v = 0; v < VPT; ++v)
             if (tid + NT * v < nvec) {
@@ -367,6 +382,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
             }
         const float et = tid < nrest ? expf(xt - m) : 0.f;
         sum = block_reduce<NW>(sum + et, false, red);
+        AKV_TAIL_MARK(12);
         const float rsum = 1.0f / sum;
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
@@ -428,6 +444,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
         }
     }
 
+    AKV_TAIL_MARK(13);
     // value rows of the tail, used by (f): requested here so that they travel while the probe runs
     constexpr int VPR = D / 8;                // 16-byte vectors per row
     constexpr int NRG = NT / VPR;             // row groups
@@ -467,6 +484,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
             probe_t[tid] = (int)(0xffffu - (key & 0xffffu)) * 32 + tid;
         }
         lds_barrier();
+        AKV_TAIL_MARK(14);
         u32 align = 0xffu;
         for (int d = tid; d < D; d += NT) {
             // the 32 gathered bytes first, then the sum: 32 independent loads in flight instead of a chain
@@ -484,6 +502,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
         }
 #pragma unroll
         for (int mk = 32; mk >= 1; mk >>= 1) align = min(align, (u32)__shfl_xor((int)align, mk, 64));
+        AKV_TAIL_MARK(15);
         if (lane == 0) red_min[wave] = align;
         lds_barrier();
         if (tid == 0) {
