@@ -820,7 +820,6 @@ inline VPlan v_plan(int B, int H, int D, int n_tokens) {
         const int iter_tokens = D == 256 ? 32 : 64;
         int k = 1;   // iterations per wave: 1, 2 or 4
         while (k < 4 && (int64_t)B * H * ((n_tokens + 4 * iter_tokens * k * 2 - 1) / (4 * iter_tokens * k * 2)) >= 2048) k *= 2;
-        { AKV_TUNE("AKV_TUNE_V_ITERS", v); if (has_v) k = v == 4 ? 4 : (v == 2 ? 2 : 1); }
         p.iters_per_wave = k;
         p.tokens_per_wave = iter_tokens * k;
         p.chunk_tokens = 4 * p.tokens_per_wave;
@@ -837,7 +836,6 @@ inline int k_blocks_per_wave(int B, int H, int n_blocks) {
     // enough waves to fill 256 CUs several times over, a few blocks per wave to amortise set-up
     int bpw = 1;
     while (bpw < 4 && (int64_t)B * H * ((n_blocks + bpw * 2 - 1) / (bpw * 2)) >= 8192) bpw *= 2;
-    { AKV_TUNE("AKV_TUNE_K_BPW", v); if (has_v && v > 0) bpw = v; }
     return bpw;
 }
 
@@ -846,7 +844,6 @@ inline int k256_blocks_per_wave(int B, int H, int n_blocks) {
     // a wave streams 64 KiB per 256-token block: one block per wave unless that makes more than ~16 k waves
     int bpw = 1;
     while (bpw < 4 && (int64_t)B * H * ((n_blocks + bpw * 2 - 1) / (bpw * 2)) >= 8192) bpw *= 2;
-    { AKV_TUNE("AKV_TUNE_K_BPW", v); if (has_v && v > 0) bpw = v; }
     return bpw;
 }
 

@@ -294,69 +294,10 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
                       need_mid, need_last, scores + (int64_t)bh * geo.row_stride, scale);
 }
 
-// K pass over planes with 256-token blocks (multi-head; see k256_score_blocks).
-// grid (ceil(n_kblocks / (4*blocks_per_wave)), H, B), 256 threads.
-template <int D, bool REF>
-__global__ __launch_bounds__(256) void fused_k_pass256_kernel(
-    const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
-    const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
-    unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, StepGeom geo, int blocks_per_wave,
-    float scale) {
-    constexpr int KB = 256;
-    constexpr int NG = D / 4;
-    const int lane = threadIdx.x & 63, wave = wave_index();
-    int chunk, h, b;
-    if (!step_block(geo, chunk, h, b)) return;
-    const int bh = b * geo.Hq + h;
-    int R, nrest;
-    seq_state(geo, b, R, nrest);
-    const int n_blocks = (R + KB - 1) / KB;     // the last one may be partly filled
-    const int first_blk = (chunk * 4 + wave) * blocks_per_wave;    // may lie past the end: the wave then only helps staging
-    const int end_blk = min(first_blk + blocks_per_wave, n_blocks);
-    const int64_t plane_off = (int64_t)bh * geo.n_max_blocks * (D * (KB / 2));
-    KHalfTile<4> ta;
-    k256_prefetch_first<D>(ta, first_8 + plane_off * 2, n_blocks, first_blk);
-    // q and the exponent sums of all channels, staged once per workgroup: every lane needs 32 of them (channels
-    // 4 g + lane/16), and 96 scattered global loads per wave would double the pass's load instructions
-    __shared__ u32 staged[D];      // [channel]: q bits | exponent sum << 16
-    for (int c = threadIdx.x; c < D; c += 256) {
-        const u32 qb = q[(int64_t)bh * D + c];
-        // column max including the token appended by this step
-        const u32 cm = max((u32)kcm[(int64_t)bh * D + c], exp_field(k_new[(int64_t)bh * D + c]));
-        staged[c] = qb | (((exp_field(qb) + cm) & 0xffu) << 16);
-    }
-    __syncthreads();
-    u32 qh[NG / 2];
-    u32 esum[NG];
-    u32 mx = 0;
-#pragma unroll
-    for (int g = 0; g < NG; ++g) {
-        const u32 w = staged[4 * g + (lane >> 4)];
-        const u32 qb = w & 0xffffu;
-        if (g & 1) qh[g >> 1] |= qb << 16; else qh[g >> 1] = qb;
-        esum[g] = w >> 16;
-        mx = max(mx, esum[g]);
-    }
-    mx = max(mx, (u32)__shfl_xor((int)mx, 16, 64));
-    mx = max(mx, (u32)__shfl_xor((int)mx, 32, 64));
-    u32 need_mid = 0, need_last = 0;
-#pragma unroll
-    for (int g = 0; g < NG; ++g) {
-        const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)esum[g]);
-        need_mid |= (lv < 2 ? 1u : 0u) << g;
-        need_last |= (lv == 0 ? 1u : 0u) << g;
-        if (levels_out != nullptr && chunk == 0 && wave == 0 && (lane & 15) == 0)
-            levels_out[(int64_t)bh * D + 4 * g + (lane >> 4)] = (uint8_t)lv;
-    }
-    if (first_blk >= n_blocks) return;
-    k256_score_blocks<D>(ta, first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qh,
-                         need_mid, need_last, scores + (int64_t)bh * geo.row_stride, R, scale);
-}
-
-// The same pass with one workgroup per 256-token block: its four waves take a quarter of the channels each, request all
-// their rows at once (12 KiB per wave, five waves per SIMD) and add their partial scores through LDS.  A cache of
-// 1024 tokens x 32 heads gives this kernel 512 waves where a block per wave gives 128 waves of 48 KiB each; long caches
-// gain from the bytes in flight (see run_step).  grid (n_kblocks, H, B), 256 threads.
+// K pass over planes with 256-token blocks (multi-head): one workgroup per block, its four waves take a quarter of the
+// channels each, request all their rows at once (12 KiB per wave, five waves per SIMD) and add their partial scores
+// through LDS.  (A block per wave with double-buffered half tiles measured behind on every shape: 33.9 vs 33.6 us at
+// batch 8 x 4096 tokens, 155.2 vs 146.9 at 4 x 32768, 8.1 vs 5.2 at 1 x 1024.)  grid (n_kblocks, H, B), 256 threads.
 template <int D, bool REF, int NWV>
 __global__ __launch_bounds__(64 * NWV) void fused_k_pass256_split_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
@@ -599,25 +540,17 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     // grouped-query heads: one workgroup per plane chunk serves 2 or 4 query heads (AKV_TUNE_GROUP: see group_heads),
     // or up to 16 on the matrix cores (K pass)
     const bool grouped = group_heads(geo.G) > 1;
-    bool matrix = geo.G >= 2 && geo.G <= 16 && D <= 128;   // (the 32-bit level masks hold 128 channels)
-    { AKV_TUNE("AKV_TUNE_MFMA", v); if (has_v) matrix = matrix && v != 0; }
+    const bool matrix = geo.G >= 2 && geo.G <= 16 && D <= 128;   // (the 32-bit level masks hold 128 channels)
     if (kb != 64 && geo.G > 1 && !matrix) {
         set_error("decode_step: grouped-query heads over K plane blocks of %d tokens need the matrix-core K pass", kb);
         return AKV_ERR_INVALID;
     }
     const int n_kblocks = (R + kb - 1) / kb;    // K plane blocks that hold tokens (the last one may be partly filled)
-    // 256-token K blocks, one query head per KV head: a block per workgroup, a quarter of the channels per wave (all of a
-    // wave's loads in flight at once).  Measured against a block per wave: batch 1 x 1024 tokens 5.2 vs 8.1 us, 8 x 4096
-    // 33.6 vs 33.9, 4 x 32768 146.7 vs 155.2 (0.85 instead of 0.80 of HBM peak).
-    bool k_split = kb == 256 && geo.G == 1 && D <= 128;
-    { AKV_TUNE("AKV_TUNE_K_SPLIT", v); if (has_v) k_split = k_split && v != 0; }
     // 64-token K blocks (head_dim 64 and 128): a block per wave with all its rows requested at once; against two blocks
     // per wave in half tiles: 36.8 vs 37.3 us at batch 8 x 4096 tokens, 160.2 vs 163.6 at 4 x 32768
-    bool k_whole = kb == 64 && D <= 128 && !grouped && !matrix;
-    { AKV_TUNE("AKV_TUNE_K_WHOLE", v); if (has_v) k_whole = k_whole && v != 0; }
-    const int bpw = (k_split || k_whole) ? 1 : (kb == 256 ? k256_blocks_per_wave(B, Hq, n_kblocks) : k_blocks_per_wave(B, Hq, n_blocks));
-    bool matrix_v = matrix;
-    { AKV_TUNE("AKV_TUNE_MFMA_V", v); if (has_v) matrix_v = matrix_v && v != 0; }
+    const bool k_whole = kb == 64 && D <= 128 && !grouped && !matrix;
+    const int bpw = (kb == 256 || k_whole) ? 1 : k_blocks_per_wave(B, Hq, n_blocks);
+    const bool matrix_v = matrix;
     VPlan p = v_plan(B, grouped ? Hq / group_heads(geo.G) : Hq, D, R);
     if constexpr (D <= 128) {
         if (matrix_v) p = mfma_v_plan<D>(B, Hkv, R);
@@ -634,8 +567,8 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
             int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo, B, n_blocks, ref, scale, st, &ks);
             if (rc != AKV_OK) return rc;
         } else {
-            if (k_split) ks = PassShape{n_kblocks, Hkv, kb};
-            else ks = PassShape{group_grid_x((n_kblocks + 4 * bpw - 1) / (4 * bpw), geo.G), Hkv, 4 * bpw * kb};
+            if (kb == 256) ks = PassShape{n_kblocks, Hkv, kb};
+            else ks = PassShape{group_grid_x((n_blocks + 4 * bpw - 1) / (4 * bpw), geo.G), Hkv, 4 * bpw * kb};
         }
         if (matrix_v) vs = PassShape{p.n_chunks, Hkv, p.chunk_tokens};
         else vs = PassShape{grouped ? p.n_chunks : group_grid_x(p.n_chunks, geo.G), grouped ? Hkv * (geo.G / group_heads(geo.G)) : Hkv,
@@ -702,7 +635,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     } else if (n_blocks > 0 && grouped) {
         int rc = launch_group_k_pass<D>(kf8, km4, kl4, kcm, q16, k16, s16, k_levels_out, geo_k, B, n_blocks, ref, scale, st);
         if (rc != AKV_OK) return rc;
-    } else if (n_blocks > 0 && kb == 256 && k_split) {
+    } else if (n_blocks > 0 && kb == 256) {
         dim3 grid(ks.grid_x, ks.grid_y, B);
         if constexpr (D <= 128) {
             if (ref)
@@ -713,18 +646,6 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
                                    k_levels_out, geo_k, scale);
         }
         int rc = check_launch("decode_step(k_pass256 split)");
-        if (rc != AKV_OK) return rc;
-    } else if (n_blocks > 0 && kb == 256) {
-        dim3 grid(ks.grid_x, ks.grid_y, B);
-        if constexpr (D <= 128) {
-            if (ref)
-                hipLaunchKernelGGL((fused_k_pass256_kernel<D, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                                   k_levels_out, geo_k, bpw, scale);
-            else
-                hipLaunchKernelGGL((fused_k_pass256_kernel<D, false>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                                   k_levels_out, geo_k, bpw, scale);
-        }
-        int rc = check_launch("decode_step(k_pass256)");
         if (rc != AKV_OK) return rc;
     } else if (n_blocks > 0) {
         dim3 grid(ks.grid_x, ks.grid_y, B);
@@ -783,8 +704,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     {
         // threads per (batch, head) row: a thread keeps 32 scores in registers between the softmax passes, so
         // rows above 8192 / 16384 tokens get 512 / 1024 threads (512 and 1024 measure level with 256 at 4096 tokens)
-        int nt = R <= 8192 ? 256 : (R <= 16384 ? 512 : 1024);
-        { AKV_TUNE("AKV_TUNE_MIDDLE_NT", v); if (has_v) nt = v; }
+        const int nt = R <= 8192 ? 256 : (R <= 16384 ? 512 : 1024);
         if (nt == 1024) hipLaunchKernelGGL((fused_middle_kernel<D, 1024>), dim3(B * Hq), dim3(1024), 0, st, ma);
         else if (nt == 512) hipLaunchKernelGGL((fused_middle_kernel<D, 512>), dim3(B * Hq), dim3(512), 0, st, ma);
         else hipLaunchKernelGGL((fused_middle_kernel<D, 256>), dim3(B * Hq), dim3(256), 0, st, ma);

@@ -289,13 +289,7 @@ __global__ __launch_bounds__(256) void group_v_pass_kernel(
 
 // ---- host ------------------------------------------------------------------------------------------
 int group_heads(int G) {
-    int gh = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);
-    AKV_TUNE("AKV_TUNE_GROUP", v);
-    if (has_v) {   // 0 / 1: one query head per workgroup; 2: at most two
-        if (v <= 1) gh = 1;
-        else if (v == 2 && gh == 4) gh = 2;
-    }
-    return gh;
+    return G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);
 }
 
 template <int D>
@@ -307,7 +301,6 @@ int launch_group_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4,
     // a wave's set-up (q, levels and masks of GH heads) costs about half a block: several blocks per wave
     int bpw = 1;
     while (bpw < 8 && (int64_t)B * geo.Hkv * (geo.G / GH) * ((n_blocks + 8 * bpw - 1) / (8 * bpw)) * 4 >= 6144) bpw *= 2;
-    { AKV_TUNE("AKV_TUNE_K_BPW", v); if (has_v && v > 0) bpw = v; }
     dim3 grid((n_blocks + 4 * bpw - 1) / (4 * bpw), geo.Hkv * (geo.G / GH), B);
     if (shape_only != nullptr) {
         *shape_only = PassShape{(int)grid.x, (int)grid.y, 4 * bpw * 64};

@@ -368,13 +368,11 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
     // of a block (256 B of first_8, 128 B of a nibble plane); measured at batch 32, 32 over 8 heads, lengths 2048..8192:
     // 62.5 us, against 78 with 8 slots per lane (half rows) and 68.8 with blocks of 64 tokens and 8 slots.  Three tiles
     // ahead instead of one (one wave per SIMD instead of two) measured 75.7 us, two tasks per wave 69.1.
-    int sl = geo.kb == 256 ? 16 : 8;
-    { AKV_TUNE("AKV_TUNE_K_SL", v); if (has_v) sl = v == 16 ? 16 : (v == 4 && geo.kb != 256 ? 4 : 8); }
+    const int sl = geo.kb == 256 ? 16 : 8;
     const int nbt = sl / 4;
     const int n_tasks = (n_blocks + nbt - 1) / nbt;
     int tpw = 1;
     while (tpw < 8 && (int64_t)B * geo.Hkv * ((n_tasks + 8 * tpw - 1) / (8 * tpw)) * 4 >= 32768) tpw *= 2;
-    { AKV_TUNE("AKV_TUNE_K_TPW", v); if (has_v && v > 0) tpw = v; }
     if (shape_only != nullptr) {
         *shape_only = PassShape{(n_tasks + 4 * tpw - 1) / (4 * tpw), geo.Hkv, 4 * tpw * nbt * 64};
         return AKV_OK;
@@ -396,16 +394,9 @@ int launch_mfma_k_pass(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, 
 #define AKV_MK(RF, SLL, AH, KSH)                                                                                     \
     hipLaunchKernelGGL((mfma_k_pass_kernel<D, RF, SLL, AH, KSH>), grid, dim3(256), 0, st, f8, m4, l4, prep, scores, geo, \
                        tpw, scale, (u32)scores_bytes)
-    int ahead = 3;
-    { AKV_TUNE("AKV_TUNE_K_AHEAD", v); if (has_v) ahead = v; }
-    constexpr int DEEP = (D / 16) % 8 == 0 ? 7 : 3;
-    if (geo.kb == 256 && sl == 16) { if (ref) AKV_MK(true, 16, 1, 2); else AKV_MK(false, 16, 1, 2); }
-    else if (geo.kb == 256) { if (ref) AKV_MK(true, 8, 3, 2); else AKV_MK(false, 8, 3, 2); }
-    else if (sl == 16) { if (ref) AKV_MK(true, 16, 1, 0); else AKV_MK(false, 16, 1, 0); }
-    else if (sl == 8 && ahead == 7) { if (ref) AKV_MK(true, 8, DEEP, 0); else AKV_MK(false, 8, DEEP, 0); }
-    else if (sl == 8) { if (ref) AKV_MK(true, 8, 3, 0); else AKV_MK(false, 8, 3, 0); }
-    else if (ahead == 7) { if (ref) AKV_MK(true, 4, DEEP, 0); else AKV_MK(false, 4, DEEP, 0); }
-    else { if (ref) AKV_MK(true, 4, 3, 0); else AKV_MK(false, 4, 3, 0); }
+    // 256-token blocks: 16 slots per lane, one tile ahead; 64-token blocks: 8 slots per lane, three tiles ahead
+    if (geo.kb == 256) { if (ref) AKV_MK(true, 16, 1, 2); else AKV_MK(false, 16, 1, 2); }
+    else { if (ref) AKV_MK(true, 8, 3, 0); else AKV_MK(false, 8, 3, 0); }
 #undef AKV_MK
     return check_launch("decode_step(mfma k_pass)");
 }
@@ -769,7 +760,6 @@ VPlan mfma_v_plan(int B, int Hkv, int n_tokens) {
     p.tuned = true;
     int k = 1;   // macro steps of 64 tokens per wave
     while (k < 4 && (int64_t)B * Hkv * ((n_tokens + 512 * k - 1) / (512 * k)) >= 2048) k *= 2;
-    { AKV_TUNE("AKV_TUNE_V_ITERS", v); if (has_v && v > 0) k = v; }
     p.iters_per_wave = k;
     p.tokens_per_wave = 64 * k;
     p.chunk_tokens = 4 * p.tokens_per_wave;

@@ -321,12 +321,10 @@ def test_fused_step_rejects_bad_state():
 
 @pytest.mark.parametrize("reference", [False, True])
 @pytest.mark.parametrize("switch,D,k_block", [("AKV_TUNE_TAIL", 128, 64), ("AKV_TUNE_TAIL", 128, 256),
-                                              ("AKV_TUNE_TAIL", 64, 64), ("AKV_TUNE_TAIL", 256, 64),
-                                              ("AKV_TUNE_K_SPLIT", 128, 256), ("AKV_TUNE_K_SPLIT", 64, 256)])
+                                              ("AKV_TUNE_TAIL", 64, 64), ("AKV_TUNE_TAIL", 256, 64), ("AKV_TUNE_TAIL", 64, 256)])
 def test_two_launch_step_matches_the_four_launch_step(monkeypatch, reference, switch, D, k_block):
     """AKV_TUNE_TAIL=1 runs everything after the K pass as one kernel (one 8-wave workgroup per (batch, head)); it must
-    agree with the four-launch step: identical fetch levels and threshold, outputs within 1e-3.  Likewise
-    AKV_TUNE_K_SPLIT=0/1: the K pass of a short cache with a 256-token block per wave or per workgroup."""
+    agree with the four-launch step: identical fetch levels and threshold, outputs within 1e-3."""
     from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
     B, H, prefill, steps = 2, 8, 1100, 70
     q, k, v = make_qkv(B, prefill + steps, H, D, seed=123)
