@@ -340,14 +340,6 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     __shared__ u32 row_amin;
     const int wave = wave_index();
     const int bh = blockIdx.x;
-    AKV_TAIL_MARK(0);
-#ifdef AKV_TRACE
-    if (g_tail_trace != nullptr && threadIdx.x == 0) {
-        unsigned xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        g_tail_trace[(size_t)blockIdx.x * 24 + 8] = xcc;
-    }
-#endif
     int R, nrest_unused;
     seq_state(ma.g, bh / ma.g.Hq, R, nrest_unused);
     const int64_t row0 = (int64_t)bh * ma.g.max_seq_len;
@@ -361,10 +353,8 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     // the row's probabilities stay in LDS for the V part (the copy in memory is the step's debug output)
     __shared__ __attribute__((aligned(16))) unsigned short probs_lds[tail_max_tokens + 64];
     middle_body<D, NT>(ma, bh, &row_amin, [&]() { v_stream_prefetch<D, NR, PF>(ring, f8, R, seq); }, probs_lds);
-    AKV_TAIL_MARK(1);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
-    AKV_TAIL_MARK(2);
     const unsigned char amin = REF ? 0 : (unsigned char)row_amin;
     if (!REF && amin_out != nullptr && threadIdx.x == 0) amin_out[bh] = amin;
     float acc[16];
@@ -380,13 +370,10 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
         // their nibble rows along with the half tiles, ring of NR.  (A row has at most tail_max_tokens flushed tokens.)
         __shared__ u32 fine_list[NW][tail_max_tokens / NW];
         const int n_fine = v_stream_count_fine<D, true>(probs_lds, R, amin, seq);
-        AKV_TAIL_MARK(3);
         if (n_fine * 16 <= seq.n_per_wave * VStream<D>::HT) {
             int count = 0;
             v_stream_run_deferred<D, 2, PF, NR, true>(ring, f8, R, probs_lds, amin, seq, acc, fine_list[wave], count);
-            AKV_TAIL_MARK(4);
             v_stream_apply_list<D>(f8, m4, l4, R, amin, acc, fine_list[wave], count);
-            AKV_TAIL_MARK(5);
         } else {
             v_stream_run<D, REF, NR, PF>(ring, f8, m4, l4, R, prow, amin, seq, acc);
         }
@@ -395,7 +382,6 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
         for (int t = threadIdx.x; t < R; t += NT) v_levels_out[(int64_t)bh * R + t] = (uint8_t)(REF ? 0 : v_level(amin, prow[t]));
     v_fold_lanes<D, NW>(acc, wave_part);
     __syncthreads();
-    AKV_TAIL_MARK(6);
     for (int d = threadIdx.x; d < D; d += NT) {
         float sum = 0.f;
 #pragma unroll
@@ -403,7 +389,6 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
         const float o16 = half_bits_to_float(float_to_half_bits(sum));
         out[(int64_t)bh * D + d] = float_to_half_bits(o16 + half_bits_to_float(ma.otail[(int64_t)bh * D + d]));
     }
-    AKV_TAIL_MARK(7);
 }
 
 // Threshold indexing of the reference expression as written (extension/v_cache_file.py:157-160): entry b*H+h
@@ -930,8 +915,3 @@ extern "C" int akv_decode_step_static(uint8_t *k_first_8, uint8_t *k_mid_4, uint
                            literal_broadcast, stream);
 }
 
-#ifdef AKV_TRACE
-extern "C" __attribute__((visibility("default"))) int akv_debug_tail_trace_buffer(void *p) {
-    return (int)hipMemcpyToSymbol(HIP_SYMBOL(akv::g_tail_trace), &p, sizeof(p));
-}
-#endif

@@ -6,14 +6,6 @@
 
 namespace akv {
 
-#ifdef AKV_TRACE
-// Development aid (not compiled into the library): per workgroup, timestamps of the phases of tail_step_kernel.
-__device__ unsigned long long *g_tail_trace = nullptr;
-#define AKV_TAIL_MARK(i) do { if (g_tail_trace != nullptr && threadIdx.x == 0) g_tail_trace[(size_t)blockIdx.x * 24 + (i)] = __builtin_amdgcn_s_memrealtime(); } while (0)
-#else
-#define AKV_TAIL_MARK(i) do { } while (0)
-#endif
-
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
@@ -340,7 +332,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
         }
     }
     lds_barrier();
-    AKV_TAIL_MARK(10);
 
     // (c) softmax over [0, R + nrest): scores + mask in fp16, softmax in fp32, probabilities in fp16
     //     (model/KVCache_AlignedKV.py:119-121), and the running arg-max of the residue classes mod 32:
@@ -370,7 +361,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
             }
         }
         m = block_reduce<NW>(m, true, red);
-        AKV_TAIL_MARK(11);
 #pragma unroll
         for (int v = 0; v < VPT; ++v)
             if (tid + NT * v < nvec) {
@@ -382,7 +372,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
             }
         const float et = tid < nrest ? expf(xt - m) : 0.f;
         sum = block_reduce<NW>(sum + et, false, red);
-        AKV_TAIL_MARK(12);
         const float rsum = 1.0f / sum;
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
@@ -444,7 +433,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
         }
     }
 
-    AKV_TAIL_MARK(13);
     // value rows of the tail, used by (f): requested here so that they travel while the probe runs
     constexpr int VPR = D / 8;                // 16-byte vectors per row
     constexpr int NRG = NT / VPR;             // row groups
@@ -484,7 +472,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
             probe_t[tid] = (int)(0xffffu - (key & 0xffffu)) * 32 + tid;
         }
         lds_barrier();
-        AKV_TAIL_MARK(14);
         u32 align = 0xffu;
         for (int d = tid; d < D; d += NT) {
             // the 32 gathered bytes first, then the sum: 32 independent loads in flight instead of a chain
@@ -502,7 +489,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
         }
 #pragma unroll
         for (int mk = 32; mk >= 1; mk >>= 1) align = min(align, (u32)__shfl_xor((int)align, mk, 64));
-        AKV_TAIL_MARK(15);
         if (lane == 0) red_min[wave] = align;
         lds_barrier();
         if (tid == 0) {
