@@ -522,7 +522,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     const int n_blocks = R / cb;
     // the kernel multiplies by the fp16-rounded scale (extension/csrc/K_cache.cu:306)
     const float scale = __half2float(__float2half_rn(1.0f / sqrtf((float)D)));
-    // grouped-query heads: one workgroup per plane chunk serves 2 or 4 query heads (AKV_TUNE_GROUP: see group_heads),
+    // grouped-query heads: one workgroup per plane chunk serves 2 or 4 query heads (group_heads),
     // or up to 16 on the matrix cores (K pass)
     const bool grouped = group_heads(geo.G) > 1;
     const bool matrix = geo.G >= 2 && geo.G <= 16 && D <= 128;   // (the 32-bit level masks hold 128 channels)
