@@ -572,8 +572,9 @@ def main():
         "value": round(us, 2), "unit": "us/step", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(us / 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "C2: batch %d, %d heads x %d, cache %d + 1 appended token, K %s, %d layers rotated, K plane blocks of %d tokens"
-                               % (B, H, D, L, a.k_kind, a.layers, a.k_block)},
+        "config": {"workload": "%s: batch %d, %d heads x %d, cache %d + 1 appended token, K %s, %d layers rotated, K plane blocks of %d tokens"
+                               % ({(8, 32, 128, 4096): "C2", (1, 32, 128, 1024): "C1", (4, 32, 128, 32768): "C4"}.get((B, H, D, L), "other shape"),
+                                  B, H, D, L, a.k_kind, a.layers, a.k_block)},
         "us_per_step_percentiles": pct,
         "effective_hbm_gbps": round(eff_gbps, 1), "pct_hbm_peak": round(100 * eff_gbps / HBM_PEAK_GBPS, 1),
         "algorithmic_bytes": int(by["total"]), "dense_fp16_bytes": int(by["dense"]),
