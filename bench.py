@@ -104,6 +104,8 @@ def parse():
                          "lengths uniform in [2048, 8192] -- an extra line, not the headline metric")
     ap.add_argument("--c3-q-heads", type=int, default=32, help="c3 only: query heads over the 8 KV heads")
     ap.add_argument("--c3-len", type=int, default=0, help="c3 only: one length for every sequence instead of U[2048, 8192]")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the short runs of the other workloads (C1, C3, C4) that the headline line carries along")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a plain 256 MiB copy kernel (known size, for scaling hardware byte counters)")
     a = ap.parse_args()
@@ -455,6 +457,30 @@ def cpu_baseline_c3(torch, cache, lens, q, k_new, v_new, lens0, bound):
             "parity": {"max_abs_err_vs_oracle": worst, "k_levels_equal": k_equal}}
 
 
+def other_workloads(a):
+    """Short runs of the configurations that are not the headline (C1, C4: the multi-head step at other shapes; C3:
+    grouped-query heads with a length per sequence), each in a process of its own: us/step and per-kernel times for the
+    same line.  A run that fails is reported as such and does not touch the headline figure."""
+    import subprocess
+    runs = {"c1": ["--batch", "1", "--cache-len", "1024", "--k-block", "64", "--steps", "200", "--warmup", "20"],
+            "c3": ["--workload", "c3", "--steps", "100", "--warmup", "10"],
+            "c4": ["--batch", "4", "--cache-len", "32768", "--k-kind", "lognormal", "--steps", "100", "--warmup", "10"]}
+    out = {}
+    for name, extra in runs.items():
+        cmd = [sys.executable, os.path.abspath(__file__), "--no-cpu", "--no-extras", "--seed", str(a.seed)] + extra
+        try:
+            r = subprocess.run(cmd, capture_output=True, text=True, timeout=240)
+            d = json.loads(r.stdout.strip().splitlines()[-1])
+            out[name] = {"us_per_step": d["value"], "workload": d["config"]["workload"], "kernel_us": d.get("kernel_us"),
+                         "pct_hbm_peak": d.get("pct_hbm_peak"), "bytes_vs_dense": d.get("bytes_vs_dense"),
+                         "k_pass_roofline_frac": d["roofline"]["frac"], "steps": d["steps"],
+                         "dense_baseline_us": d.get("dense_fp16_hip_us", d.get("dense_in_planes_us")),
+                         "command": "python bench.py --no-cpu " + " ".join(extra)}
+        except Exception as e:      # noqa: BLE001 (reported in the line)
+            out[name] = {"error": "%s: %s" % (type(e).__name__, str(e)[:200])}
+    return out
+
+
 def main():
     a = parse()
     if a.gpus != 1:
@@ -626,6 +652,8 @@ def main():
                 r.at_length(L + sidx)()
         torch.cuda.synchronize()
         res["avg_us_over_64_growing_steps"] = round((time.perf_counter() - t0) / (64 * a.layers) * 1e6, 2)
+    if not a.no_extras and not a.no_cpu and (B, H, D, L) == (8, 32, 128, 4096):
+        res["other_workloads"] = other_workloads(a)
     print(json.dumps(res))
 
 
