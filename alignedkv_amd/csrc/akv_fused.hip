@@ -655,16 +655,17 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     // Second half of the step in one launch (see tail_step_kernel)
     // It is used when the (batch, head) pairs spread evenly over the compute units (every unit gets the same one or
     // two rows) and the rows are not long: measured on MI355X with 32 heads x 128, against the three launches it
-    // replaces: 30.2 vs 34.8 us per step at batch 8 x 1024 tokens, 76.0 vs 78.7 at 8 x 4096, 141.6 vs 145.9 at
-    // 16 x 4096; level at 32 x 4096 and behind at 8 x 16384 (one workgroup per unit streams at 4.5 TB/s, the V pass
-    // of many small workgroups at 6).
+    // replaces: 43.2 vs 46.3 us per step at batch 8 x 2048 tokens, 69.2 vs 74.7 at 8 x 4096, 99.4 vs 105.0 at 8 x 6144,
+    // 134.1 vs 133.0 at 8 x 8192, 130.4 vs 133.2 at 16 x 4096, 184.3 vs 188.4 at 16 x 6144, but 250.7 vs 241.5 at
+    // 16 x 8192 (two long rows per unit: one workgroup per row streams at 4.5 TB/s, the V pass of many small workgroups
+    // at 6): up to 12288 tokens per compute unit.
     // With fewer rows than compute units a row's workgroup streams alone at about 45 GB/s, while the V pass of many
     // small workgroups needs 4 us or the time of its bytes at 5 TB/s and then two more launches (2.5 us): measured
     // with 32 heads x 128 at batch 1 x 1024 tokens 21.7 vs 23.9 us per step, 2 x 2048: 25.5 vs 26.3, 4 x 4096: 43.7
     // vs 45.6, but 1 x 4096: 30.3 vs 27.0.
     const int cus = compute_units();
     const int rows = B * Hq;
-    bool tail = cus > 0 && rows % cus == 0 && rows / cus <= tail_rows_per_cu;
+    bool tail = cus > 0 && rows % cus == 0 && rows / cus <= tail_rows_per_cu && (rows / cus) * R <= 12288;
     if (cus > 0 && rows < cus) {
         const float row_us = (float)R * D / 45e3f, passes_us = fmaxf(4.f, (float)rows * R * D / 5e6f) + 2.5f;
         tail = row_us < passes_us;
