@@ -186,7 +186,7 @@ def test_v_cache_test_compute_parity(mod, B, H, D, L, K):
                                                  (2, 2, 128, 300, 257, 0), (2, 3, 64, 256, 192, 64),
                                                  (1, 2, 256, 128, 128, 64), (2, 3, 6, 50, 37, 3),
                                                  (1, 2, 128, 64, 0, 64), (1, 32, 128, 4096, 4096, 64)])
-def test_v_cache_compute_parity(mod, B, H, D, L, n_tok, extra, reference):
+def test_v_cache_compute_parity(mod, B, H, D, L, n_tok, extra, reference, require_all_levels=True):
     rng = np.random.default_rng(L + n_tok)
     _, _, v = make_qkv(B, L, H, D, 8)
     planes = O.v_planes_alloc(B, H, L + 5, D)
@@ -196,8 +196,8 @@ def test_v_cache_compute_parity(mod, B, H, D, L, n_tok, extra, reference):
     # thresholds around the typical probability exponent so that all three levels occur
     amin = rng.integers(6, 14, (B, H)).astype(np.uint8)
     want, want_lv = O.v_cache_compute(*planes, O.as_bits(p), amin, n_tok, reference, True)
-    if not reference and n_tok >= 128 and D >= 64:
-        assert len(np.unique(want_lv)) == 3
+    if require_all_levels and not reference and n_tok >= 128 and D >= 64:
+        assert len(np.unique(want_lv)) == 3      # (the hand-picked shapes exercise every level)
     pd = dev(p)
     s_cut = pd[:, :, :, :n_tok]                       # sliced view, row stride W (the reference passes this)
     lv = torch.full((B, H, max(n_tok, 1)), 255, dtype=torch.uint8, device="cuda")
