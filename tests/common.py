@@ -57,7 +57,7 @@ def assert_close_fp16(got, want, abs_floor):
     spacing = np.abs(np.spacing(np.asarray(want, np.float16))).astype(np.float64)
     err = np.abs(g - w)
     bad = err > spacing + abs_floor
-    assert not bad.any(), f"max err {err.max():.3e} (allowed {float((spacing + abs_floor)[err.argmax()]):.3e}) at {int(bad.sum())} entries"
+    assert not bad.any(), f"max err {err.max():.3e} (allowed {float((spacing + abs_floor).flat[err.argmax()]):.3e}) at {int(bad.sum())} entries"
 
 
 def oracle_decode_step_c(k_planes, v_planes, k_colmax, v_colmax, q, k_new, v_new, R, d_block=64, top_k=32,

@@ -360,20 +360,32 @@ def test_two_launch_step_matches_the_four_launch_step(monkeypatch, reference, sw
     lib.akv_reload_tuning()
 
 
-def test_sharp_attention_step_is_exact_stage_by_stage():
+def _stagewise_shapes(seed, n):
+    rng = np.random.default_rng(seed)
+    for _ in range(n):
+        B, H, D = int(rng.choice([1, 2, 3, 8])), int(rng.choice([4, 8, 32])), int(rng.choice([64, 128, 128, 256]))
+        kb = int(rng.choice([64, 256])) if D <= 128 else 64
+        prefill = int(rng.choice([1, 63, 64, 65, 200, 511, 512, 1000, 1500]))
+        steps = int(rng.choice([2, 5, 66]))
+        if B * H * (prefill + steps) * D > 20e6:
+            steps = 2
+        yield (B, H, D, kb, prefill, steps, float(rng.choice([1.0, 0.05, 0.3, 3.0])), int(rng.integers(0, 1000)))
+
+
+@pytest.mark.parametrize("B,H,D,kb,prefill,steps,qscale,seed", [(8, 4, 64, 256, 512, 66, 3.0, 35)] + list(_stagewise_shapes(21, 10)))
+def test_step_is_exact_stage_by_stage(B, H, D, kb, prefill, steps, qscale, seed):
     """Large scores (q scaled by 3: the leading token holds 70 % of a row) make the end-to-end output ill-conditioned: fp16
     scores near 15 are 2**-7 apart, so a score that lands on the neighbouring fp16 value under another fp32 summation order
     moves its probability by 0.8 % and the output by a few 1e-3 -- in the reference as much as here.  The step is therefore
     checked stage by stage: fetch levels and threshold bit for bit, every score within one fp16 value of the oracle's (3e-4
-    for scores near zero), the
+    per 128 channels for scores near zero), the
     probabilities equal to the oracle's softmax OF THE KERNEL'S OWN SCORES (within one fp16 value, nearly all bit for bit),
     and the output within 1e-3 of the oracle's V side applied to the kernel's own probabilities."""
     from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
-    from tests.common import assert_close_fp16, ulp_diff_fp16
-    B, H, D, kb, prefill, steps = 8, 4, 64, 256, 512, 66
-    Lmax = prefill + steps + 64
-    _, k, v = make_qkv(B, prefill + steps, H, D, seed=135)
-    rng = np.random.default_rng(35)
+    from tests.common import ulp_diff_fp16
+    Lmax = max(prefill + steps + 64, 128)
+    _, k, v = make_qkv(B, prefill + steps, H, D, seed=seed + 100)
+    rng = np.random.default_rng(seed)
     cache = QuantizedCache_AlignedKV(cfg(H, D), B, Lmax, "cuda", torch.half, k_block=kb)
     oc = O.OracleCache(B, Lmax, H, D, k_block=kb)
     kc, vc = cache.key_cache[0], cache.value_cache[0]
@@ -383,30 +395,44 @@ def test_sharp_attention_step_is_exact_stage_by_stage():
     oc.save(k[:, :prefill], v[:, :prefill], 0, prefill)
     worst_end_to_end = worst_v_side = 0.0
     for t in range(prefill, prefill + steps):
-        qt = (3.0 * rng.standard_normal((B, 1, H, D))).astype(np.float16)
+        qt = (qscale * rng.standard_normal((B, 1, H, D))).astype(np.float16)
         out = cache.auto_compute(dev(qt), dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None).cpu().numpy()
         want = oc.decode(qt, k[:, t:t + 1], v[:, t:t + 1])
         R, L = oc.rest_start, t + 1
-        assert np.array_equal(kc.last_levels.cpu().numpy(), oc.last["k_levels"])
+        if R:
+            assert np.array_equal(kc.last_levels.cpu().numpy(), oc.last["k_levels"])
         sg = cache._scores[:, :, :L].cpu().numpy()
-        # (one fp16 value, or 3e-4 where a dot product is much smaller than its terms)
-        assert_close_fp16(sg, oc.last["scores"][:, :, 0, :L], 3e-4)
+        # (one fp16 value, or 3e-4 per 128 channels where a dot product is much smaller than its terms; the tail's scores
+        # are rounded twice, fp16(fp16(q.k) / sqrt(D)) as in extension/k_cache_file.py:156: a dot product on the
+        # neighbouring fp16 value can end two values away)
+        floor = 3e-4 * max(1, D // 128)
+        so = oc.last["scores"][:, :, 0, :L]
+        values_off = ulp_diff_fp16(sg, so)
+        finite = np.isfinite(so)
+        beyond_floor = np.abs(np.where(finite, sg, 0).astype(np.float32) - np.where(finite, so, 0).astype(np.float32)) > floor
+        assert not ((values_off[:, :, :R] > 1) & beyond_floor[:, :, :R]).any(), f"a score is more than one fp16 value off at token {t}"
+        assert not ((values_off[:, :, R:] > 2) & beyond_floor[:, :, R:]).any(), f"a tail score is more than two fp16 values off at token {t}"
         pg = cache._probs[:, :, :L].cpu().numpy()
         p_of_own_scores = O.softmax_fp32_to_half(sg[:, :, None, :])[:, :, 0]
         du = ulp_diff_fp16(pg, p_of_own_scores)
-        assert du.max() <= 1 and (du == 0).mean() >= 0.999, f"softmax of the kernel's scores differs at token {t}"
-        amin = vc.last_alignment_min.cpu().numpy()
-        tv, ti = O.bucket_max(np.ascontiguousarray(pg[:, :, None, :R]), L)
-        to = O.v_cache_test_compute(oc.v_planes[0], O.as_bits(tv), ti)
-        assert np.array_equal(amin, O.alignment_min(O.test_o_exponent(to), oc.v_colmax, False)), f"threshold differs at token {t}"
-        assert np.array_equal(vc.last_levels.cpu().numpy(), O.v_levels(amin, O.as_bits(np.ascontiguousarray(pg[:, :, :R]))))
-        o_planes, _ = O.v_cache_compute(*oc.v_planes, O.as_bits(np.ascontiguousarray(pg[:, :, None, :R])), amin, R, False,
-                                        return_levels=True)
-        o_own = (o_planes + O.rest_output(np.ascontiguousarray(pg[:, :, None, R:L]), oc.restv, oc.rest_len)).astype(np.float16)
+        assert du.max() <= 1 and (du != 0).sum() <= max(4, 0.002 * du.size), f"softmax of the kernel's scores differs at token {t}"
+        if R:
+            amin = vc.last_alignment_min.cpu().numpy()
+            tv, ti = O.bucket_max(np.ascontiguousarray(pg[:, :, None, :R]), L)
+            to = O.v_cache_test_compute(oc.v_planes[0], O.as_bits(tv), ti)
+            assert np.array_equal(amin, O.alignment_min(O.test_o_exponent(to), oc.v_colmax, False)), f"threshold differs at token {t}"
+            assert np.array_equal(vc.last_levels.cpu().numpy(), O.v_levels(amin, O.as_bits(np.ascontiguousarray(pg[:, :, :R]))))
+            o_own, _ = O.v_cache_compute(*oc.v_planes, O.as_bits(np.ascontiguousarray(pg[:, :, None, :R])), amin, R, False,
+                                         return_levels=True)
+        else:
+            o_own = np.zeros((B, H, 1, D), np.float16)
+        if oc.rest_len:
+            o_own = (o_own + O.rest_output(np.ascontiguousarray(pg[:, :, None, R:L]), oc.restv, oc.rest_len)).astype(np.float16)
         v_side = float(np.abs(out.astype(np.float32) - o_own.reshape(B, 1, H, D).astype(np.float32)).max())
         worst_v_side = max(worst_v_side, v_side)
         worst_end_to_end = max(worst_end_to_end, float(np.abs(out.astype(np.float32) - want.astype(np.float32)).max()))
         assert v_side <= 1e-3, f"V side on the kernel's probabilities: {v_side:.3e} at token {t}"
     from tests.common import WORST_STEP_ERR
-    WORST_STEP_ERR["sharp attention, V side on the kernel's own probabilities"] = worst_v_side
-    WORST_STEP_ERR["sharp attention, end to end (ill-conditioned: not asserted)"] = worst_end_to_end
+    key = "stage by stage (q x %g)" % qscale
+    WORST_STEP_ERR[key + ", V side on the kernel's own probabilities"] = max(WORST_STEP_ERR.get(key + ", V side on the kernel's own probabilities", 0.0), worst_v_side)
+    WORST_STEP_ERR[key + ", end to end (not asserted)"] = max(WORST_STEP_ERR.get(key + ", end to end (not asserted)", 0.0), worst_end_to_end)
