@@ -28,7 +28,8 @@ int launch_v_save(uint8_t *first_8, uint8_t *mid_4, uint8_t *last_4, const uint8
                   int max_seq_len, int head_dim, int start_pos, int seq_len, int v_new_seq, hipStream_t st);
 
 // Optional per-phase timing of the fused step (benchmark aid): when enabled, events are recorded on the
-// step's stream around the K pass, the middle kernel, the V pass and the combine kernel.
+// step's stream around the K pass, the middle kernel, the V pass and the combine kernel.  Process-wide and
+// unsynchronised on purpose: for a single-threaded benchmark that runs one step at a time on one stream.
 static bool g_profile = false;
 static hipEvent_t g_ev[7];   // 0..4 around the four phases, 5 and 6 back to back (interval of an empty phase)
 static bool g_ev_ready = false;
@@ -670,6 +671,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         const float row_us = (float)R * D / 45e3f, passes_us = fmaxf(4.f, (float)rows * R * D / 5e6f) + 2.5f;
         tail = row_us < passes_us;
     }
+    // AKV_TUNE_TAIL=0/1 in the environment overrides the choice (the tests run both forms of the step on the same inputs)
     { AKV_TUNE("AKV_TUNE_TAIL", v); if (has_v) tail = v != 0; }
     tail = tail && n_blocks >= 1 && R <= tail_max_tokens && geo.G == 1 && !ragged && !(literal_broadcast && !ref);
     if (tail) {

@@ -168,11 +168,9 @@ struct NoHook {
 };
 // hook: called once the loads that depend on nothing have been requested (a caller that goes on in the same
 // workgroup requests its own data there: loads return in order, so these come back first)
-// DEV: what later stages read (probabilities, threshold, tail output) is stored at device scope, for a launch whose
-// other workgroups -- on other XCDs, with L2 caches of their own -- go on with the row
 // probs_lds (may be null): LDS copy of the row's probabilities, tokens 0 .. R + tail, for a caller that goes on in the
 // same workgroup
-template <int D, int NT, typename Hook = NoHook, bool DEV = false>
+template <int D, int NT, typename Hook = NoHook>
 __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u32 *amin_lds = nullptr, Hook hook = Hook(),
                                             unsigned short *probs_lds = nullptr);
 
@@ -212,7 +210,7 @@ __device__ __forceinline__ void decode_scores8(const u32x4 w, const unsigned sho
 }
 
 // NT threads (a multiple of 256) of one workgroup run the stage for one (batch, head).
-template <int D, int NT, typename Hook, bool DEV>
+template <int D, int NT, typename Hook>
 __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u32 *amin_lds, Hook hook, unsigned short *probs_lds) {
     constexpr int VPT = 4;                    // 16-byte score vectors a thread keeps in registers
     constexpr int NW = NT / 64;               // waves
@@ -243,16 +241,13 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
     const bool in_regs = nvec <= NT * VPT;
     // scores of the flushed part are read at device scope: other workgroups of the same launch wrote them
     const __amdgpu_buffer_rsrc_t rScores = make_rsrc(srow, (u32)R * 2);
-    const __amdgpu_buffer_rsrc_t rProbs = make_rsrc(prow, (u32)(R + nrest) * 2);
     auto store_probs8 = [&](int i, const u32x4 o) {
         if (probs_lds != nullptr) *reinterpret_cast<u32x4 *>(probs_lds + i * 8) = o;
-        if constexpr (DEV) __builtin_amdgcn_raw_buffer_store_b128(o, rProbs, i * 16, 0, kDeviceScope);
-        else *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
+        *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
     };
     auto store_prob1 = [&](int t, unsigned short p) {
         if (probs_lds != nullptr) probs_lds[t] = p;
-        if constexpr (DEV) store_u16_device(rProbs, t * 2, p);
-        else prow[t] = p;
+        prow[t] = p;
     };
 
     // Everything that does not depend on anything else is requested first: the score vectors of the
@@ -495,8 +490,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
             u32 mn = red_min[0];
 #pragma unroll
             for (int w = 1; w < NW; ++w) mn = min(mn, red_min[w]);
-            if constexpr (DEV) __builtin_amdgcn_raw_buffer_store_b8((unsigned char)mn, make_rsrc(a.amin + bh, 1u), 0, 0, kDeviceScope);
-            else a.amin[bh] = (uint8_t)mn;
+            a.amin[bh] = (uint8_t)mn;
             if (amin_lds != nullptr) *amin_lds = mn;   // for a caller that goes on in the same workgroup
         }
     } else {
@@ -533,8 +527,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
             float sum = 0.f;
 #pragma unroll
             for (int w = 0; w < NW; ++w) sum += tail_o[w][d];
-            if constexpr (DEV) store_u16_device(make_rsrc(a.otail + (int64_t)bh * D, (u32)D * 2), d * 2, float_to_half_bits(sum));
-            else a.otail[(int64_t)bh * D + d] = float_to_half_bits(sum);
+            a.otail[(int64_t)bh * D + d] = float_to_half_bits(sum);
         }
     }
 }

@@ -29,6 +29,7 @@ class K_Cache_Class(PlaneCacheBase):
                                           (bsz, n_local_kv_heads, nb, head_dim, k_block // 2), register_buffer)
         self._colmax = torch.zeros((bsz, 1, n_local_kv_heads, head_dim), dtype=torch.uint8, device=device)
         self.last_levels = None     # uint8 [bsz, heads, head_dim] of the last decoding_compute when record_levels
+        self.last_scores = None     # fp16 copy of the scores it returned (debug record, with record_levels)
         self.record_levels = False
 
     # names the reference exposes
@@ -96,4 +97,6 @@ class K_Cache_Class(PlaneCacheBase):
         s[:, :, :, self.reststartpos:self.reststartpos + self._restlen] = \
             torch.matmul(q.transpose(1, 2), rest) / math.sqrt(self.head_dim)
         s[:, :, :, start_pos + seqlen:] = float("-inf")
+        if self.record_levels:
+            self.last_scores = s.clone()     # the caller adds its mask in place
         return s

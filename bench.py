@@ -49,12 +49,12 @@ def profile_figures(name):
         for line in open(os.path.join(PROFILES, name + "_kernel_stats.txt")):
             f = line.split()
             if len(f) >= 5 and (line.startswith("akv::") or line.startswith("copy_probe")):
-                kernel = line[:line.index(f[-4])].strip()
+                kernel = line.rsplit(None, 4)[0].strip()     # (split from the right: the name's template arguments hold numbers too)
                 out.setdefault(kernel, {})["avg_us"] = float(f[-3])
         for line in open(os.path.join(PROFILES, name + "_hbm_traffic.txt")):
             f = line.split()
             if len(f) >= 6 and (line.startswith("akv::") or line.startswith("copy_probe")):
-                kernel = line[:line.index(f[-5])].strip()
+                kernel = line.rsplit(None, 5)[0].strip()
                 out.setdefault(kernel, {}).update(fetch_mib=float(f[-3]), write_mib=float(f[-1]))
     except (OSError, ValueError):
         pass

@@ -165,6 +165,10 @@ AKV_API int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_las
  * akv_decode_step_workspace_bytes(bsz, n_kv_heads, head_dim, max_seq_len) exceeds AKV_STATIC_SCRATCH_BYTES are rejected
  * (AKV_ERR_INVALID).  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (two streams,
  * two host threads) race on it and must be serialised by the caller; nothing in the array has to survive between calls.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress), which may load the library's device
+ * code on that device: make that one call outside stream capture; every later call only launches kernels.  The array
+ * is part of the device code of the fused step: a GPU on which the library runs any fused step holds these
+ * AKV_STATIC_SCRATCH_BYTES whether or not this entry point is ever called.
  */
 #define AKV_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
 AKV_API int akv_decode_step_static(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,
@@ -218,7 +222,9 @@ AKV_API int akv_dense_decode_step(uint8_t *k_cache, uint8_t *v_cache, const uint
 /*
  * Benchmark aid, no counterpart in the reference: with profiling enabled, akv_decode_step records HIP
  * events on its stream around its four phases; akv_profile_read waits for the last recorded step and
- * returns the elapsed milliseconds of {K pass, middle, V pass, combine}.  Process-wide, not thread safe.
+ * returns the elapsed milliseconds of {K pass, middle, V pass, combine}.  The switch and the events are process-wide
+ * and unsynchronised: single-threaded benchmark use only (one host thread, one stream at a time); leave profiling
+ * off in a program that runs steps from several threads or streams.
  */
 /* The AKV_TUNE_* environment switches are read when first used; call this after changing one in a running process. */
 AKV_API int akv_reload_tuning(void);

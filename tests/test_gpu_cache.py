@@ -9,7 +9,7 @@ import torch
 import torch.nn.functional as F
 
 from oracle import akv_oracle as O
-from tests.common import assert_step_output, make_qkv
+from tests.common import assert_outputs_agree, assert_step_output, assert_step_stagewise, make_qkv
 
 pytestmark = pytest.mark.gpu
 
@@ -87,12 +87,16 @@ def test_cache_matches_oracle_step_by_step(prefill, steps, literal_broadcast, k_
                 to = O.v_cache_test_compute(oc.v_planes[0], O.as_bits(tv), ti)
                 want_amin = O.alignment_min(O.test_o_exponent(to), oc.v_colmax, literal_broadcast)
                 assert np.array_equal(amin, want_amin), f"threshold differs at token {t}"
-                pd = np.abs(cache._probs[:, :, :t + 1].cpu().numpy().astype(np.float32)
-                            - oc.last["probs"][:, :, 0, :t + 1].astype(np.float32)).max()
-                assert pd <= 2e-3
-        # 1e-3; only where the kernels' fp16 probabilities differ from the oracle's in some bit (a score rounded to the
-        # neighbouring fp16 value under another summation order) 2e-3.  The worst error seen is printed at the end of the run.
-        assert_step_output(out.cpu().numpy(), want, f"cache step by step (fused={fused}, k_block={k_block})", probs_equal)
+        # 1e-3 end to end; where a score landed on the neighbouring fp16 value (the probabilities then differ from the
+        # oracle's in some bit) and that moved the output further, the step has to pass stage by stage instead
+        def stagewise():
+            if fused:
+                sc, pr = cache._scores.cpu().numpy(), cache._probs.cpu().numpy()
+            else:
+                sc, pr = kc.last_scores[:, :, 0].cpu().numpy(), vc.last_probs[:, :, 0].cpu().numpy()
+            return assert_step_stagewise(out.cpu().numpy(), sc, pr, oc, D, vc.last_alignment_min.cpu().numpy() if oc.rest_start else None,
+                                         vc.last_levels.cpu().numpy() if oc.rest_start else None, literal_broadcast, f"token {t}")
+        assert_step_output(out.cpu().numpy(), want, f"cache step by step (fused={fused}, k_block={k_block})", probs_equal, stagewise)
     # probabilities are produced by two different softmax implementations: a V level can only flip
     # where a probability or the probe sits on a rounding boundary
     assert flips <= max(2, 0.002 * total), f"{flips} of {total} V levels differ"
@@ -182,6 +186,7 @@ def test_fused_step_with_mask_and_reference_flag(monkeypatch, tail):
         for fused in (True, False):
             c = QuantizedCache_AlignedKV(cfg(H, D), B, 256, "cuda", torch.half)
             c.fused, c.reference = fused, reference
+            c.key_cache[0].record_levels = c.value_cache[0].record_levels = True
             c.auto_compute(dev(q[:, :1].repeat(prefill, axis=1)), dev(k[:, :prefill]), dev(v[:, :prefill]), 0, None)
             caches.append(c)
         for t in range(prefill, prefill + 4):
@@ -190,7 +195,9 @@ def test_fused_step_with_mask_and_reference_flag(monkeypatch, tail):
             mask[1, 0, 0, 3:40] = float("-inf")
             outs = [c.auto_compute(qt, dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, mask) for c in caches]
             assert torch.isfinite(outs[0]).all()
-            assert (outs[0].float() - outs[1].float()).abs().max().item() <= 2e-3
+            assert_outputs_agree(outs[0].cpu().numpy(), outs[1].cpu().numpy(), caches[0]._probs[:, :, :t + 1].cpu().numpy(),
+                                 caches[1].value_cache[0].last_probs[:, :, 0, :t + 1].cpu().numpy(), np.abs(v).max(),
+                                 "fused step against the op sequence, with a mask")
             assert caches[0]._probs[1, :, 3:40].abs().max().item() == 0.0
     monkeypatch.delenv("AKV_TUNE_TAIL")
     load_library().akv_reload_tuning()
@@ -252,7 +259,9 @@ def test_step_on_as_many_rows_as_compute_units_matches_the_op_sequence():
         caches.append(c)
     for t in range(prefill, prefill + steps):
         outs = [c.auto_compute(dev(q[:, t:t + 1]), dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None) for c in caches]
-        assert (outs[0].float() - outs[1].float()).abs().max().item() <= 2e-3
+        assert_outputs_agree(outs[0].cpu().numpy(), outs[1].cpu().numpy(), caches[0]._probs[:, :, :t + 1].cpu().numpy(),
+                             caches[1].value_cache[0].last_probs[:, :, 0, :t + 1].cpu().numpy(), np.abs(v).max(),
+                             "fused step against the op sequence, 256 rows")
         assert torch.equal(caches[0].key_cache[0].last_levels, caches[1].key_cache[0].last_levels)
         flips = (caches[0].value_cache[0].last_levels != caches[1].value_cache[0].last_levels).float().mean().item()
         assert flips <= 0.01
@@ -290,7 +299,9 @@ def test_fused_step_against_op_sequence_on_random_shapes(monkeypatch):
         for s in range(steps):
             t = prefill + s
             outs = [c.auto_compute(dev(q[:, s:s + 1]), dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None) for c in caches]
-            assert (outs[0].float() - outs[1].float()).abs().max().item() <= 2e-3, what
+            assert_outputs_agree(outs[0].cpu().numpy(), outs[1].cpu().numpy(), caches[0]._probs[:, :, :t + 1].cpu().numpy(),
+                                 caches[1].value_cache[0].last_probs[:, :, 0, :t + 1].cpu().numpy(), np.abs(v).max(),
+                                 "fused step against the op sequence, random shapes", what)
             if caches[1].key_cache[0].reststartpos:
                 assert torch.equal(caches[0].key_cache[0].last_levels, caches[1].key_cache[0].last_levels), what
                 a, b = caches[0].value_cache[0].last_levels, caches[1].value_cache[0].last_levels
@@ -372,7 +383,11 @@ def _stagewise_shapes(seed, n):
         yield (B, H, D, kb, prefill, steps, float(rng.choice([1.0, 0.05, 0.3, 3.0])), int(rng.integers(0, 1000)))
 
 
-@pytest.mark.parametrize("B,H,D,kb,prefill,steps,qscale,seed", [(8, 4, 64, 256, 512, 66, 3.0, 35)] + list(_stagewise_shapes(21, 10)))
+# The first four are cases a randomised run over shapes found with an end-to-end difference of 2.2e-3 to 3.4e-3, each traced
+# to one score on the neighbouring fp16 value: one with q scaled by 3 and three with unscaled q (head_dim 256 and 64).
+@pytest.mark.parametrize("B,H,D,kb,prefill,steps,qscale,seed", [(8, 4, 64, 256, 512, 66, 3.0, 35), (3, 32, 256, 64, 200, 66, 1.0, 16),
+                                                                (8, 32, 64, 256, 200, 66, 1.0, 6), (8, 32, 64, 256, 512, 66, 1.0, 40)]
+                         + list(_stagewise_shapes(21, 10)))
 def test_step_is_exact_stage_by_stage(B, H, D, kb, prefill, steps, qscale, seed):
     """Large scores (q scaled by 3: the leading token holds 70 % of a row) make the end-to-end output ill-conditioned: fp16
     scores near 15 are 2**-7 apart, so a score that lands on the neighbouring fp16 value under another fp32 summation order
@@ -382,7 +397,6 @@ def test_step_is_exact_stage_by_stage(B, H, D, kb, prefill, steps, qscale, seed)
     probabilities equal to the oracle's softmax OF THE KERNEL'S OWN SCORES (within one fp16 value, nearly all bit for bit),
     and the output within 1e-3 of the oracle's V side applied to the kernel's own probabilities."""
     from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
-    from tests.common import ulp_diff_fp16
     Lmax = max(prefill + steps + 64, 128)
     _, k, v = make_qkv(B, prefill + steps, H, D, seed=seed + 100)
     rng = np.random.default_rng(seed)
@@ -398,40 +412,14 @@ def test_step_is_exact_stage_by_stage(B, H, D, kb, prefill, steps, qscale, seed)
         qt = (qscale * rng.standard_normal((B, 1, H, D))).astype(np.float16)
         out = cache.auto_compute(dev(qt), dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None).cpu().numpy()
         want = oc.decode(qt, k[:, t:t + 1], v[:, t:t + 1])
-        R, L = oc.rest_start, t + 1
+        R = oc.rest_start
         if R:
             assert np.array_equal(kc.last_levels.cpu().numpy(), oc.last["k_levels"])
-        sg = cache._scores[:, :, :L].cpu().numpy()
-        # (one fp16 value, or 3e-4 per 128 channels where a dot product is much smaller than its terms; the tail's scores
-        # are rounded twice, fp16(fp16(q.k) / sqrt(D)) as in extension/k_cache_file.py:156: a dot product on the
-        # neighbouring fp16 value can end two values away)
-        floor = 3e-4 * max(1, D // 128)
-        so = oc.last["scores"][:, :, 0, :L]
-        values_off = ulp_diff_fp16(sg, so)
-        finite = np.isfinite(so)
-        beyond_floor = np.abs(np.where(finite, sg, 0).astype(np.float32) - np.where(finite, so, 0).astype(np.float32)) > floor
-        assert not ((values_off[:, :, :R] > 1) & beyond_floor[:, :, :R]).any(), f"a score is more than one fp16 value off at token {t}"
-        assert not ((values_off[:, :, R:] > 2) & beyond_floor[:, :, R:]).any(), f"a tail score is more than two fp16 values off at token {t}"
-        pg = cache._probs[:, :, :L].cpu().numpy()
-        p_of_own_scores = O.softmax_fp32_to_half(sg[:, :, None, :])[:, :, 0]
-        du = ulp_diff_fp16(pg, p_of_own_scores)
-        assert du.max() <= 1 and (du != 0).sum() <= max(4, 0.002 * du.size), f"softmax of the kernel's scores differs at token {t}"
-        if R:
-            amin = vc.last_alignment_min.cpu().numpy()
-            tv, ti = O.bucket_max(np.ascontiguousarray(pg[:, :, None, :R]), L)
-            to = O.v_cache_test_compute(oc.v_planes[0], O.as_bits(tv), ti)
-            assert np.array_equal(amin, O.alignment_min(O.test_o_exponent(to), oc.v_colmax, False)), f"threshold differs at token {t}"
-            assert np.array_equal(vc.last_levels.cpu().numpy(), O.v_levels(amin, O.as_bits(np.ascontiguousarray(pg[:, :, :R]))))
-            o_own, _ = O.v_cache_compute(*oc.v_planes, O.as_bits(np.ascontiguousarray(pg[:, :, None, :R])), amin, R, False,
-                                         return_levels=True)
-        else:
-            o_own = np.zeros((B, H, 1, D), np.float16)
-        if oc.rest_len:
-            o_own = (o_own + O.rest_output(np.ascontiguousarray(pg[:, :, None, R:L]), oc.restv, oc.rest_len)).astype(np.float16)
-        v_side = float(np.abs(out.astype(np.float32) - o_own.reshape(B, 1, H, D).astype(np.float32)).max())
+        v_side = assert_step_stagewise(out, cache._scores.cpu().numpy(), cache._probs.cpu().numpy(), oc, D,
+                                       vc.last_alignment_min.cpu().numpy() if R else None, vc.last_levels.cpu().numpy() if R else None,
+                                       False, f"token {t}")
         worst_v_side = max(worst_v_side, v_side)
         worst_end_to_end = max(worst_end_to_end, float(np.abs(out.astype(np.float32) - want.astype(np.float32)).max()))
-        assert v_side <= 1e-3, f"V side on the kernel's probabilities: {v_side:.3e} at token {t}"
     from tests.common import WORST_STEP_ERR
     key = "stage by stage (q x %g)" % qscale
     WORST_STEP_ERR[key + ", V side on the kernel's own probabilities"] = max(WORST_STEP_ERR.get(key + ", V side on the kernel's own probabilities", 0.0), worst_v_side)

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from oracle import akv_oracle as O
-from tests.common import assert_step_output, make_qkv
+from tests.common import assert_step_output, assert_step_stagewise, make_qkv
 
 pytestmark = pytest.mark.gpu
 
@@ -72,7 +72,12 @@ def _ragged_case_against_oracle(B, Hq, Hkv, lens, steps, D):
             L = lens[b] + s + 1
             probs_equal = bool(np.array_equal(O.as_bits(cache.probs[b, :, :L].cpu().numpy()),
                                               O.as_bits(np.ascontiguousarray(oc.last["probs"][0, :, 0, :L]))))
-            assert_step_output(out[b:b + 1], want, f"ragged grouped step (D={D}, k_block={kb})", probs_equal)
+            def stagewise(b=b, oc=oc):
+                R_ = oc.rest_start
+                return assert_step_stagewise(out[b:b + 1], cache.scores[b:b + 1].cpu().numpy(), cache.probs[b:b + 1].cpu().numpy(), oc, D,
+                                             cache.last_alignment_min[b].cpu().numpy() if R_ else None,
+                                             cache.last_v_levels[b:b + 1].cpu().numpy() if R_ else None, False, f"step {s} sequence {b}")
+            assert_step_output(out[b:b + 1], want, f"ragged grouped step (D={D}, k_block={kb})", probs_equal, stagewise)
             R = oc.rest_start
             if R:
                 assert np.array_equal(cache.last_k_levels[b].cpu().numpy(), oc.last["k_levels"][0]), f"K levels, step {s} seq {b}"

@@ -16,7 +16,7 @@ import torch
 import torch.nn.functional as F
 
 from oracle import akv_oracle as O
-from tests.common import assert_step_output, make_qkv
+from tests.common import assert_step_output, assert_step_stagewise, make_qkv
 
 pytestmark = pytest.mark.gpu
 
@@ -144,4 +144,6 @@ def test_five_ops_with_the_reference_callers_argument_forms(B, H, D, prefill, st
             to = O.v_cache_test_compute(oc.v_planes[0], O.as_bits(tv), ti)
             want_amin = O.alignment_min(O.test_o_exponent(to), oc.v_colmax, True)
             assert np.array_equal(amin.reshape(-1)[:B * H].cpu().numpy().reshape(B, H), want_amin), f"threshold differs at token {t}"
-        assert_step_output(out, want, f"reference callers' forms (D={D})", probs_equal)
+        stagewise = lambda: assert_step_stagewise(out, s[:, :, 0].cpu().numpy(), pn[:, :, 0], oc, D,
+                                                  amin.cpu().numpy() if oc.rest_start else None, None, True, f"token {t}")
+        assert_step_output(out, want, f"reference callers' forms (D={D})", probs_equal, stagewise)

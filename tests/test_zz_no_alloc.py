@@ -1,6 +1,8 @@
 """The allocation-free entry point akv_decode_step_static against akv_decode_step, through the C ABI: two calls in a
 row on the same GPU, the second on a smaller cache, each compared bit for bit (same kernels, same order of sums) with
-the workspace-taking entry point run from an identical copy of the cache state."""
+the workspace-taking entry point run from an identical copy of the cache state.  That it allocates nothing is checked
+on the device-wide free memory (hipMemGetInfo), which also sees a hipMalloc inside the library, once a first round of
+the same calls has loaded the library's code objects and looked up the scratch array's address."""
 import ctypes
 
 import numpy as np
@@ -44,7 +46,7 @@ def _state(B, H, D, L, Lmax, seed, k_block=64):
     return st, tok, nmb, R
 
 
-def _run(static, st, tok, B, H, D, L, Lmax, nmb, R, literal):
+def _run(static, st, tok, B, H, D, L, Lmax, nmb, R, literal, check_free=False):
     import alignedkv_amd
     from alignedkv_amd._lib import check
     lib = alignedkv_amd.load_library()
@@ -61,10 +63,16 @@ def _run(static, st, tok, B, H, D, L, Lmax, nmb, R, literal):
     rec = [res["klv"].data_ptr(), res["vlv"].data_ptr(), res["amin"].data_ptr()]
     geo = [B, H, nmb, Lmax, D, CB, 32, L, R, L - R, 0, int(literal), torch.cuda.current_stream().cuda_stream]
     if static:
-        # no torch allocation between here and the end of the call: the entry point itself must not need any
-        before = torch.cuda.memory_allocated()
+        # no torch allocation between here and the end of the call: the entry point itself must not need any, from
+        # torch's allocator or from the device (free memory of the whole GPU, as hipMemGetInfo reports it)
+        torch.cuda.synchronize()
+        before, free_before = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
         rc = lib.akv_decode_step_static(*head, *rec, *geo)
+        torch.cuda.synchronize()
         assert torch.cuda.memory_allocated() == before
+        if check_free:
+            free_after = torch.cuda.mem_get_info()[0]
+            assert free_after == free_before, f"device free memory changed by {free_after - free_before} bytes across the call"
     else:
         need = lib.akv_decode_step_workspace_bytes(B, H, D, Lmax)
         ws = torch.empty(need, dtype=torch.uint8, device="cuda")
@@ -75,12 +83,12 @@ def _run(static, st, tok, B, H, D, L, Lmax, nmb, R, literal):
     return res
 
 
-def _compare(B, H, D, L, literal, seed):
+def _compare(B, H, D, L, literal, seed, check_free=False):
     Lmax = L + 1 + CB
     got, want = {}, {}
     for static, dst in ((True, got), (False, want)):
         st, tok, nmb, R = _state(B, H, D, L, Lmax, seed)
-        res = _run(static, st, tok, B, H, D, L, Lmax, nmb, R, literal)
+        res = _run(static, st, tok, B, H, D, L, Lmax, nmb, R, literal, check_free)
         dst.update(res)
         dst.update({"state_" + k: v for k, v in st.items()})
     flushed = (L + 1) // CB * CB
@@ -96,12 +104,16 @@ def _compare(B, H, D, L, literal, seed):
 
 
 def test_static_scratch_step_matches_the_workspace_step_twice_in_a_row():
-    print("no-alloc step: 4 x 8 heads x 128, 1279 tokens (this step flushes a block), literal threshold indexing", flush=True)
-    _compare(4, 8, 128, 1279, True, seed=31)       # four launches: partial sums of the V pass go through the scratch array
-    print("no-alloc step: 2 x 4 heads x 128, 200 tokens", flush=True)
-    _compare(2, 4, 128, 200, False, seed=32)       # smaller, right after: one workgroup per (batch, head) row
-    print("no-alloc step: 1 x 4 heads x 64, 70 tokens", flush=True)
-    _compare(1, 4, 64, 70, False, seed=33)
+    # first round: the library's code objects are loaded lazily and the scratch array's address is looked up on the first
+    # call; second round: the same calls must leave the device's free memory untouched
+    for check_free in (False, True):
+        print(f"no-alloc step (free memory checked: {check_free}): 4 x 8 heads x 128, 1279 tokens (this step flushes a block), "
+              "literal threshold indexing", flush=True)
+        _compare(4, 8, 128, 1279, True, seed=31, check_free=check_free)   # four launches: partial sums go through the scratch array
+        print("no-alloc step: 2 x 4 heads x 128, 200 tokens", flush=True)
+        _compare(2, 4, 128, 200, False, seed=32, check_free=check_free)   # smaller, right after: one workgroup per (batch, head) row
+        print("no-alloc step: 1 x 4 heads x 64, 70 tokens", flush=True)
+        _compare(1, 4, 64, 70, False, seed=33, check_free=check_free)
 
 
 def test_static_scratch_step_rejects_shapes_beyond_its_array():
