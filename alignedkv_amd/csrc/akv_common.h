@@ -135,6 +135,21 @@ __device__ __forceinline__ float div_by(float x, float d, float r) {
     return fmaf(fmaf(-q, d, x), r, q);
 }
 
+// exp(x) for x <= 0 (a score minus the row maximum): the hardware's 2^y on y = x * log2(e), with the product's rounding
+// error and the low part of log2(e) put back as a first-order correction, so the result is within an ulp or two of the
+// correctly rounded one for every x whose exponential is a normal float; below that it goes to zero (a probability
+// that small rounds to zero in fp16 anyway).  Six instructions against the thirteen of the library routine, which
+// matters where a compute unit runs a whole row's softmax on its own.
+__device__ __forceinline__ float exp_nonpositive(float x) {
+    const float l2e_hi = 1.44269502162933349609375f, l2e_lo = 1.925963033500011e-8f, ln2 = 0.693147182464599609375f;
+    x = fmaxf(x, -200.f);      // (minus infinity, a masked score, included: the result is zero)
+    const float y = x * l2e_hi;
+    float err = fmaf(x, l2e_hi, -y);
+    err = fmaf(x, l2e_lo, err);
+    const float e = __builtin_amdgcn_exp2f(y);
+    return fmaf(e, err * ln2, e);
+}
+
 constexpr int kSkip = 0x7fffffff;   // an offset no plane slice reaches
 
 // Cache-policy bits of buffer loads/stores on gfx950: sc1 = device (agent) scope.  Data that one
@@ -164,5 +179,56 @@ __device__ __forceinline__ u32x4 load_b128_device(const __amdgpu_buffer_rsrc_t r
 __device__ __forceinline__ int wave_index() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 
 __device__ __forceinline__ float wave_xor_add(float v, int mask) { return v + __shfl_xor(v, mask, 64); }
+
+// Wave-wide reductions with the result in every lane: two quad permutes and the two mirrors inside the 16-lane rows
+// (data-parallel primitives: no LDS round trip per step, unlike a shuffle), then the four row totals through scalar
+// registers.  The order of the additions is fixed, so the bits of a sum are reproducible.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int CTRL>
+__device__ __forceinline__ u32 dpp_u32(u32 v) {
+    return (u32)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+}
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
+__device__ __forceinline__ float rows_to_wave_f32(float v, bool is_max) {
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return is_max ? fmaxf(fmaxf(r0, r1), fmaxf(r2, r3)) : (r0 + r1) + (r2 + r3);
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f32<kDppXor1>(v);
+    v += dpp_f32<kDppXor2>(v);
+    v += dpp_f32<kDppHalfMirror>(v);
+    v += dpp_f32<kDppMirror>(v);
+    return rows_to_wave_f32(v, false);
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_f32<kDppXor1>(v));
+    v = fmaxf(v, dpp_f32<kDppXor2>(v));
+    v = fmaxf(v, dpp_f32<kDppHalfMirror>(v));
+    v = fmaxf(v, dpp_f32<kDppMirror>(v));
+    return rows_to_wave_f32(v, true);
+}
+__device__ __forceinline__ u32 wave_min_u32(u32 v) {
+    v = min(v, dpp_u32<kDppXor1>(v));
+    v = min(v, dpp_u32<kDppXor2>(v));
+    v = min(v, dpp_u32<kDppHalfMirror>(v));
+    v = min(v, dpp_u32<kDppMirror>(v));
+    return min(min((u32)__builtin_amdgcn_readlane((int)v, 0), (u32)__builtin_amdgcn_readlane((int)v, 16)),
+               min((u32)__builtin_amdgcn_readlane((int)v, 32), (u32)__builtin_amdgcn_readlane((int)v, 48)));
+}
+__device__ __forceinline__ int wave_sum_i32(int v) {
+    v += (int)dpp_u32<kDppXor1>((u32)v);
+    v += (int)dpp_u32<kDppXor2>((u32)v);
+    v += (int)dpp_u32<kDppHalfMirror>((u32)v);
+    v += (int)dpp_u32<kDppMirror>((u32)v);
+    return (__builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16)) +
+           (__builtin_amdgcn_readlane(v, 32) + __builtin_amdgcn_readlane(v, 48));
+}
+
 
 }  // namespace akv

@@ -12,6 +12,22 @@ template <int N>
 __device__ __forceinline__ void reduce_scatter_step(float *a, int lane_mask) {
     // N partial sums per lane -> N/2: the lane keeps one half and receives the partner's sums of
     // that half.  After the step a[i] belongs to original index i + (lane & lane_mask ? N/2 : 0).
+    // Partners 32 and 16 lanes apart exchange through the half-wave / row swap instructions (one instruction per
+    // pair of sums, no LDS round trip); the sums are the same bits as with a shuffle (own + partner's either way).
+    if (lane_mask == 32 || lane_mask == 16) {
+#pragma unroll
+        for (int i = 0; i < N / 2; ++i) {
+            const u32 x = __float_as_uint(a[i]), y = __float_as_uint(a[i + N / 2]);
+            if (lane_mask == 32) {
+                const auto r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
+                a[i] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+            } else {
+                const auto r = __builtin_amdgcn_permlane16_swap(x, y, false, false);
+                a[i] = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+            }
+        }
+        return;
+    }
     const bool up = (threadIdx.x & lane_mask) != 0;
 #pragma unroll
     for (int i = 0; i < N / 2; ++i) {
@@ -439,6 +455,10 @@ struct VListed {
                                                      const __amdgpu_buffer_rsrc_t rH, const __amdgpu_buffer_rsrc_t rM,
                                                      const __amdgpu_buffer_rsrc_t rL, unsigned char amin, int tok_base) {
         if (count <= 0) return;
+        if (count <= TPL) {       // the usual case: nothing more to request (and to wait for)
+            apply(acc, first);
+            return;
+        }
         Step other;
         for (int e0 = 0; e0 < count; e0 += 2 * TPL) {
             request(other, list, count, e0 + TPL, rH, rM, rL, amin, tok_base);
@@ -537,15 +557,12 @@ struct VRing {
     u32 sb[NR][VStream<D>::HV];
 };
 
-// The wave's i-th half tile: interleaved over the n_waves waves of the workgroup (at any time the waves read
-// neighbouring rows).  Past the wave's share: n_halves (nothing is fetched).
+// A wave's share of the half tiles of a row: its i-th half tile is start + i * stride (i < count), so that at any time
+// the waves of a workgroup read neighbouring rows.  Past the share: n_halves (nothing is fetched).
 struct VSeq {
-    int wave, n_waves, n_per_wave, n_halves;
-    int first = 0;   // the wave's share starts at its first-th half tile (a caller that has done the ones before)
-    __device__ __forceinline__ int half(int i) const {
-        return i + first < n_per_wave ? (i + first) * n_waves + wave : n_halves;
-    }
-    __device__ __forceinline__ int left() const { return n_per_wave - first; }
+    int start, stride, count, n_halves;
+    __device__ __forceinline__ int half(int i) const { return i < count ? start + i * stride : n_halves; }
+    __device__ __forceinline__ int left() const { return count; }
 };
 
 // High bytes of half tile `half`: one address per lane, the HV rows at constant distances from it.  A half tile past the
@@ -674,9 +691,7 @@ __device__ __forceinline__ int v_stream_count_fine(const unsigned short *s_row, 
             n += on ? __builtin_popcount((t.u >> 15) & 0x00010001u) : 0;
         }
     }
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) n += __shfl_xor(n, m, 64);
-    return n;
+    return wave_sum_i32(n);
 }
 
 // The same with the tokens below level 2 taken out of the loop (VListed); the caller adds the listed tokens at the end
@@ -741,6 +756,80 @@ __device__ __forceinline__ void v_stream_run_deferred(VRing<D, NRING> &ring, con
         for (int i0 = NR; i0 < seq.left(); i0 += NR) round(i0);
     }
 }
+
+// The stream with every token multiplied at level 2 (high bytes only) and no look at the fetch levels: for a caller that
+// does not know the row's threshold yet, or has listed the tokens below level 2 some other way (v_stream_list_fine).
+// One half tile in flight while one is multiplied; the probabilities come from LDS (probs_lds: the row's, token-indexed).
+// prefetched: the share's first half tile has been requested into ring.hi[0] already (by the caller with
+// v_stream_issue_high, or by the call for the share before this one through next_half).
+// next_half: requested into ring.hi[0] when the share's last half tile is being multiplied (the first half tile of the
+// share the wave takes next, so that the pipeline does not drain between the two calls), or n_halves for none.
+// extra(i0): called once per round of two half tiles, when the round's first request is on its way (work that is to hide
+// behind the stream's memory time).
+struct NoExtra {
+    __device__ __forceinline__ void operator()(int) const {}
+};
+template <int D, typename Extra = NoExtra>
+__device__ __forceinline__ void v_stream_run_coarse(VRing<D, 2> &ring, const uint8_t *f8, int n_tokens,
+                                                   const unsigned short *probs_lds, const VSeq &seq, bool prefetched, int next_half,
+                                                   float *acc, Extra extra = Extra()) {
+    using S = VStream<D>;
+    constexpr int HV = S::HV;
+    const int lane = threadIdx.x & 63, tl = lane / S::LPR;
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
+    if (seq.count <= 0) return;
+    if (!prefetched) v_stream_issue_high<D>(ring.hi[0], rH, seq.half(0));
+    __builtin_amdgcn_sched_barrier(0);
+    auto round = [&](int i0) {
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            // (slot 0 after the share's last round: the next share's first half tile)
+            const int ahead = (k == 1 && i0 + 2 >= seq.count) ? next_half : seq.half(i0 + k + 1);
+            v_stream_issue_high<D>(ring.hi[k ^ 1], rH, ahead);
+            __builtin_amdgcn_sched_barrier(0);
+            if (k == 0) {
+                extra(i0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            const int half = seq.half(i0 + k);
+            // (a half tile past the wave's share: its high bytes came back as zeros, its probabilities count as zeros)
+            const bool on = half < seq.n_halves;
+            u32 sb[HV];
+#pragma unroll
+            for (int u = 0; u < HV; ++u) sb[u] = on ? (u32)probs_lds[half * S::HT + tl + u * S::TPL] : 0u;
+            v_compute_half_coarse<HV>(acc, ring.hi[k], sb);
+            pin_accumulators(acc);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // (the first round stands outside the loop: see v_stream_run)
+    round(0);
+    for (int i0 = 2; i0 < seq.count; i0 += 2) round(i0);
+}
+
+// Lists the tokens below level 2 of a wave's shares a and b (in that order) from the row's probabilities in LDS, 64 tokens
+// per step: list[count ...] gets (token | probability bits << 16).  A token with probability zero never counts.
+template <int D>
+struct VFineScan {
+    using S = VStream<D>;
+    static constexpr int TPI = 64 / S::HT;       // half tiles per step
+    const unsigned short *probs_lds;
+    unsigned char amin;
+    VSeq a, b;
+    int pos = 0;
+    __device__ __forceinline__ bool done() const { return pos >= a.count + b.count; }
+    __device__ __forceinline__ int steps_left() const { return (a.count + b.count - pos + TPI - 1) / TPI; }
+    __device__ __forceinline__ void step(u32 *list, int &count) {
+        const int lane = threadIdx.x & 63;
+        const int i = pos + lane / S::HT;
+        const int half = i < a.count ? a.start + i * a.stride : b.half(i - a.count);
+        const bool on = half < a.n_halves;
+        const int tok = half * S::HT + lane % S::HT;
+        const u32 pb = on ? (u32)probs_lds[tok] : 0u;
+        VListed<D>::append(list, count, pb != 0u && v_level(amin, (unsigned short)pb) < 2, tok, pb);
+        pos += TPI;
+    }
+};
 
 template <int D>
 __device__ __forceinline__ void v_stream_apply_list(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_tokens,

@@ -318,7 +318,8 @@ __global__ __launch_bounds__(64 * NWV) void fused_k_pass256_split_kernel(
 // grid (B*H), 256 threads: the middle stage on its own (no flushed block yet, or fusion switched off).
 template <int D, int NT>
 __global__ __launch_bounds__(NT) void fused_middle_kernel(MiddleArgs a) {
-    middle_body<D, NT>(a, blockIdx.x);
+    __shared__ MiddleShared<D, NT / 64> ms;
+    middle_body<D, NT>(a, blockIdx.x, ms);
 }
 
 constexpr int tail_rows_per_cu = 2, tail_max_tokens = 8192;
@@ -328,59 +329,198 @@ constexpr int tail_rows_per_cu = 2, tail_max_tokens = 8192;
 // workgroup of 8 waves, after a K pass that ran as a launch of its own.  With about as many (batch, head) pairs as
 // compute units (or a multiple of them) every unit streams one row of V planes from start to end: no partial sums,
 // no combine launch, and the first high-byte tiles of every wave travel while the middle stage runs.
-// grid (B*H), 512 threads.
-template <int D, bool REF, int NR, int PF, int NT>
+//
+// The V planes start to stream as soon as the row's probabilities are known: one wave works out the probe and the
+// row's alignment threshold (a gather of 32 rows: a memory round trip of its own) while the other waves multiply
+// their first `fa` half tiles each at level 2, which needs no threshold.  After a barrier every wave lists the tokens
+// of its share that are below level 2 (from the probabilities in LDS), requests the first of them, streams the rest
+// of its share at level 2 and then adds p * (value at the token's level - value at level 2) for the listed tokens.
+// A wave whose tokens are below level 2 more often than one in 16 (flat attention) lists only the ones it has
+// multiplied already and takes the nibble rows of the others along with their half tiles (v_stream_run).
+// grid (B*H), NT threads.
+template <int D, int NT, int PRE>
 __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict__ v_first_8,
                                                         const uint8_t *__restrict__ v_mid_4,
                                                         const uint8_t *__restrict__ v_last_4, MiddleArgs ma,
                                                         unsigned short *__restrict__ out,
                                                         uint8_t *__restrict__ v_levels_out,
-                                                        uint8_t *__restrict__ amin_out) {
+                                                        uint8_t *__restrict__ amin_out, int fa) {
     constexpr int NW = NT / 64;
+    using S = VStream<D>;
+    __shared__ MiddleShared<D, NW> ms;
     __shared__ float wave_part[NW][D];
-    __shared__ u32 row_amin;
+    // the row's probabilities stay in LDS for the V part (the copy in memory is the step's debug output)
+    __shared__ __attribute__((aligned(16))) unsigned short probs_lds[tail_max_tokens + 64];
+    __shared__ u32 fine_list[NW][tail_max_tokens / NW];
+    const int wave = wave_index();
+    const int bh = blockIdx.x;
+    AKV_MARK(bh, 0);
+    int R, nrest_unused;
+    seq_state(ma.g, bh / ma.g.Hq, R, nrest_unused);
+    const int64_t row0 = (int64_t)bh * ma.g.max_seq_len;
+    const uint8_t *f8 = v_first_8 + row0 * D, *m4 = v_mid_4 + row0 * (D / 2), *l4 = v_last_4 + row0 * (D / 2);
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)R * D);
+    // Part A, before the threshold is known: the first n_a half tiles of the row, dealt out to the waves 1 .. NW - 1
+    // (wave 0 runs the probe meanwhile); part B: the others, dealt out to all waves.
+    const int n_halves = (R + S::HT - 1) / S::HT;
+    const int n_a = min(fa * (NW - 1), n_halves);
+    VSeq seq_a, seq_b;
+    seq_a.n_halves = seq_b.n_halves = n_halves;
+    seq_a.start = wave - 1; seq_a.stride = NW - 1;
+    seq_a.count = (wave >= 1 && wave - 1 < n_a) ? (n_a - (wave - 1) + NW - 2) / (NW - 1) : 0;
+    seq_b.start = n_a + wave; seq_b.stride = NW;
+    seq_b.count = n_a + wave < n_halves ? (n_halves - n_a - wave + NW - 1) / NW : 0;
+    // Requested before the middle stage, right behind its first loads, and held in registers until the probabilities
+    // are known: the first PRE half tiles of the wave's part A, and the half tile it streams first afterwards.  (The
+    // waves 1 .. NW - 1 have no other loads between the stage's first ones and the stream, so nothing of theirs queues
+    // behind these; wave 0 has the probe's gather to come and requests only its first half tile of part B.)
+    VHighPart<S::HV> pre[PRE > 0 ? PRE : 1];
+    VRing<D, 2> ring;
+    VSeq seq_a2 = seq_a;        // part A beyond the PRE half tiles held in registers
+    seq_a2.start = seq_a.start + PRE * seq_a.stride;
+    seq_a2.count = max(seq_a.count - PRE, 0);
+    const int first_streamed = wave == 0 ? seq_b.half(0) : (seq_a2.count > 0 ? seq_a2.half(0) : seq_b.half(0));
+    MiddleCarry<D, NT> carry;
+    static_assert(PRE <= 3, "one half tile per phase of the middle stage");
+    middle_body<D, NT, true>(ma, bh, ms, [&](auto point) {
+        constexpr int i = decltype(point)::value;
+        if constexpr (i < PRE) {
+            if (wave != 0) v_stream_issue_high<D>(pre[i], rH, seq_a.half(i));
+        }
+        if constexpr (i == 3) v_stream_issue_high<D>(ring.hi[0], rH, first_streamed);
+    }, probs_lds, &carry);
+    AKV_MARK(bh, 1);
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+    // the tail's share of the output: once per wave, where it hides behind memory time
+    bool tail_done = false;
+    auto tail_once = [&]() {
+        if (!tail_done) middle_tail_partials<D, NT>(ms, carry);
+        tail_done = true;
+    };
+    if (wave == 0) {
+        middle_probe_wave<D, NW>(ma, ms, bh, R, tail_once);
+    } else {
+        const int tl = (threadIdx.x & 63) / S::LPR;
+#pragma unroll
+        for (int k = 0; k < PRE; ++k) {
+            const int half = seq_a.half(k);
+            const bool on = half < n_halves;
+            u32 sb[S::HV];
+#pragma unroll
+            for (int u = 0; u < S::HV; ++u) sb[u] = on ? (u32)probs_lds[half * S::HT + tl + u * S::TPL] : 0u;
+            v_compute_half_coarse<S::HV>(acc, pre[k], sb);
+        }
+        pin_accumulators(acc);
+        // (ends with part B's first half tile requested, unless it was the one requested up front)
+        v_stream_run_coarse<D>(ring, f8, R, probs_lds, seq_a2, true, seq_b.half(0), acc, [&](int) { tail_once(); });
+    }
+    AKV_MARK(bh, 2);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    AKV_MARK(bh, 3);
+    const unsigned char amin = (unsigned char)ms.amin;
+    if (amin_out != nullptr && threadIdx.x == 0) amin_out[bh] = amin;
+    const unsigned short *prow = ma.probs + (int64_t)bh * ma.g.row_stride;
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)R * (D / 2)), rL = make_rsrc(l4, (u32)R * (D / 2));
+    u32 *list = fine_list[wave];
+    int count = 0;
+    const int n_fine = v_stream_count_fine<D, true>(probs_lds, R, amin, seq_a) + v_stream_count_fine<D, true>(probs_lds, R, amin, seq_b);
+    const bool few = n_fine * 16 <= (seq_a.count + seq_b.count) * S::HT;
+    VFineScan<D> scan;
+    scan.probs_lds = probs_lds; scan.amin = amin; scan.a = seq_a; scan.b = seq_b;
+    if (!few) scan.b.count = 0;     // (the others are read at their level as they stream)
+    typename VListed<D>::Step first;
+    AKV_MARK(bh, 4);
+    if (few) {
+        // Part B in two stretches: during the first the tokens below level 2 are listed, two steps of 64 tokens per
+        // round of the stream; then the first of them are requested, and arrive while the second stretch streams.
+        const int n_b1 = min(seq_b.count, 2 * ((scan.steps_left() + 1) / 2));
+        VSeq b1 = seq_b, b2 = seq_b;
+        b1.count = n_b1;
+        b2.start = seq_b.start + n_b1 * seq_b.stride; b2.count = seq_b.count - n_b1;
+        v_stream_run_coarse<D>(ring, f8, R, probs_lds, b1, true, b2.half(0), acc, [&](int) {
+            tail_once();
+            if (!scan.done()) scan.step(list, count);
+            if (!scan.done()) scan.step(list, count);
+        });
+        while (!scan.done()) scan.step(list, count);
+        VListed<D>::request(first, list, count, 0, rH, rM, rL, amin, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        v_stream_run_coarse<D>(ring, f8, R, probs_lds, b2, true, n_halves, acc);
+    } else {
+        while (!scan.done()) scan.step(list, count);
+        VListed<D>::request(first, list, count, 0, rH, rM, rL, amin, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        // (the share's first half tile, requested early, is asked for again: the rare path)
+        VRing<D, 4> ring4;
+        v_stream_run<D, false, 4, 0>(ring4, f8, m4, l4, R, prow, amin, seq_b, acc);
+    }
+    tail_once();
+    AKV_MARK(bh, 5);
+    VListed<D>::apply_all(acc, first, list, count, rH, rM, rL, amin, 0);
+    AKV_MARK(bh, 6);
+    if (v_levels_out != nullptr)
+        for (int t = threadIdx.x; t < R; t += NT) v_levels_out[(int64_t)bh * R + t] = (uint8_t)v_level(amin, probs_lds[t]);
+    v_fold_lanes<D, NW>(acc, wave_part);
+    __syncthreads();
+    AKV_MARK(bh, 7);
+    if (threadIdx.x == 0) {
+#ifdef AKV_TRACE
+        if (g_tail_trace != nullptr) {
+            u32 xcc;
+            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+            g_tail_trace[((int64_t)bh * 8) * 24 + 8] = (long long)(xcc & 0xf);
+            g_tail_trace[((int64_t)bh * 8) * 24 + 9] = (long long)count;
+        }
+#endif
+    }
+    for (int d = threadIdx.x; d < D; d += NT) {
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) sum += wave_part[w][d];
+        const float o16 = half_bits_to_float(float_to_half_bits(sum));
+        // fp16(planes) + fp16(tail), the fp16 `o += tail` of the reference (extension/v_cache_file.py:189)
+        const float t16 = half_bits_to_float(float_to_half_bits(middle_tail_output<D, NW>(ms, d)));
+        out[(int64_t)bh * D + d] = float_to_half_bits(o16 + t16);
+    }
+}
+
+// The same for the mode that reads every plane (the reference's `reference=True`): no fetch levels, so the whole
+// middle stage runs first and every wave then streams its share with the nibble rows (ring of NR half tiles, the
+// first PF of them requested before the middle stage).  grid (B*H), NT threads.
+template <int D, int NR, int PF, int NT>
+__global__ __launch_bounds__(NT) void tail_step_ref_kernel(const uint8_t *__restrict__ v_first_8,
+                                                            const uint8_t *__restrict__ v_mid_4,
+                                                            const uint8_t *__restrict__ v_last_4, MiddleArgs ma,
+                                                            unsigned short *__restrict__ out,
+                                                            uint8_t *__restrict__ v_levels_out) {
+    constexpr int NW = NT / 64;
+    __shared__ MiddleShared<D, NW> ms;
+    __shared__ float wave_part[NW][D];
     const int wave = wave_index();
     const int bh = blockIdx.x;
     int R, nrest_unused;
     seq_state(ma.g, bh / ma.g.Hq, R, nrest_unused);
     const int64_t row0 = (int64_t)bh * ma.g.max_seq_len;
     const uint8_t *f8 = v_first_8 + row0 * D, *m4 = v_mid_4 + row0 * (D / 2), *l4 = v_last_4 + row0 * (D / 2);
-    // wave w takes the half tiles w, w + 8, ...
+    // wave w takes the half tiles w, w + NW, ...
     VSeq seq;
-    seq.wave = wave; seq.n_waves = NW;
     seq.n_halves = (R + VStream<D>::HT - 1) / VStream<D>::HT;
-    seq.n_per_wave = (seq.n_halves + NW - 1) / NW;
+    seq.start = wave; seq.stride = NW;
+    seq.count = wave < seq.n_halves ? (seq.n_halves - wave + NW - 1) / NW : 0;
     VRing<D, NR> ring;
-    // the row's probabilities stay in LDS for the V part (the copy in memory is the step's debug output)
-    __shared__ __attribute__((aligned(16))) unsigned short probs_lds[tail_max_tokens + 64];
-    middle_body<D, NT>(ma, bh, &row_amin, [&]() { v_stream_prefetch<D, NR, PF>(ring, f8, R, seq); }, probs_lds);
+    middle_body<D, NT, false>(ma, bh, ms, [&](auto) { v_stream_prefetch<D, NR, PF>(ring, f8, R, seq); });
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
-    const unsigned char amin = REF ? 0 : (unsigned char)row_amin;
-    if (!REF && amin_out != nullptr && threadIdx.x == 0) amin_out[bh] = amin;
     float acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
     const unsigned short *prow = ma.probs + (int64_t)bh * ma.g.row_stride;
-    if constexpr (REF) {
-        v_stream_run<D, REF, NR, PF>(ring, f8, m4, l4, R, prow, amin, seq, acc);
-    } else {
-        // Few tokens below level 2 (the usual case): they are taken out of the loop, which then keeps one half tile
-        // per wave in flight (measured faster than 2, 3, 5 and 7: 29.9 / 30.9 / 30.3 / 32.1 / 32.1 us at batch 8 x 32
-        // heads x 4096 tokens).  More than one in 16 among the wave's tokens (flat attention): the loop that takes
-        // their nibble rows along with the half tiles, ring of NR.  (A row has at most tail_max_tokens flushed tokens.)
-        __shared__ u32 fine_list[NW][tail_max_tokens / NW];
-        const int n_fine = v_stream_count_fine<D, true>(probs_lds, R, amin, seq);
-        if (n_fine * 16 <= seq.n_per_wave * VStream<D>::HT) {
-            int count = 0;
-            v_stream_run_deferred<D, 2, PF, NR, true>(ring, f8, R, probs_lds, amin, seq, acc, fine_list[wave], count);
-            v_stream_apply_list<D>(f8, m4, l4, R, amin, acc, fine_list[wave], count);
-        } else {
-            v_stream_run<D, REF, NR, PF>(ring, f8, m4, l4, R, prow, amin, seq, acc);
-        }
-    }
+    v_stream_run<D, true, NR, PF>(ring, f8, m4, l4, R, prow, 0, seq, acc);
     if (v_levels_out != nullptr)
-        for (int t = threadIdx.x; t < R; t += NT) v_levels_out[(int64_t)bh * R + t] = (uint8_t)(REF ? 0 : v_level(amin, prow[t]));
+        for (int t = threadIdx.x; t < R; t += NT) v_levels_out[(int64_t)bh * R + t] = 0;
     v_fold_lanes<D, NW>(acc, wave_part);
     __syncthreads();
     for (int d = threadIdx.x; d < D; d += NT) {
@@ -676,12 +816,21 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     tail = tail && n_blocks >= 1 && R <= tail_max_tokens && geo.G == 1 && !ragged && !(literal_broadcast && !ref);
     if (tail) {
         // (16 waves per workgroup measured 1 us slower than 8)
-        if (ref)
-            hipLaunchKernelGGL((tail_step_kernel<D, true, 4, 3, 512>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
-                               reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out);
-        else
-            hipLaunchKernelGGL((tail_step_kernel<D, false, 4, 1, 512>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
-                               reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out);
+        if (ref) {
+            hipLaunchKernelGGL((tail_step_ref_kernel<D, 4, 3, 512>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
+                               reinterpret_cast<unsigned short *>(out), v_levels_out);
+        } else {
+            // half tiles per wave that stream before the row's threshold is known: about what the probe's gather takes
+            int fa = 5;
+            { AKV_TUNE("AKV_TUNE_TAIL_FA", v); if (has_v) fa = v; }
+            int pre = 2;
+            { AKV_TUNE("AKV_TUNE_TAIL_PRE", v); if (has_v) pre = v; }
+            fa = max(fa, pre);
+#define AKV_TAIL(P) hipLaunchKernelGGL((tail_step_kernel<D, 512, P>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,   \
+                                       reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out, fa)
+            if (pre <= 0) AKV_TAIL(0); else if (pre == 1) AKV_TAIL(1); else if (pre == 2) AKV_TAIL(2); else AKV_TAIL(3);
+#undef AKV_TAIL
+        }
         mark(2, st);
         mark(3, st);
         mark(4, st);
@@ -742,6 +891,13 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
 }  // namespace akv
 
 using namespace akv;
+
+#ifdef AKV_TRACE
+extern "C" __attribute__((visibility("default"))) int akv_debug_tail_trace_buffer(void *buf) {
+    long long *p = static_cast<long long *>(buf);
+    return hipMemcpyToSymbol(HIP_SYMBOL(g_tail_trace), &p, sizeof(p)) == hipSuccess ? 0 : 1;
+}
+#endif
 
 extern "C" int akv_profile_enable(int enable) {
     if (enable && !g_ev_ready) {

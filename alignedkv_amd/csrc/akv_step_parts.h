@@ -6,16 +6,17 @@
 
 namespace akv {
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
-    return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
-    return v;
-}
+#ifdef AKV_TRACE
+// development build only: timestamps per (row, wave, mark) of the step's second kernel
+static __device__ long long *g_tail_trace;
+#define AKV_MARK(bh, slot)                                                                                            \
+    do {                                                                                                              \
+        if (g_tail_trace != nullptr && (threadIdx.x & 63) == 0)                                                       \
+            g_tail_trace[((int64_t)(bh) * 8 + (threadIdx.x >> 6)) * 24 + (slot)] = wall_clock64();                    \
+    } while (0)
+#else
+#define AKV_MARK(bh, slot) do {} while (0)
+#endif
 
 // K pass over the 256-token stretch `chunk` of a row of planes with 64-token blocks, by a workgroup of four waves: a wave
 // takes one block and requests all its rows at once (16 KiB in flight for head_dim 128, no loop).  bh_kv / bh: row of
@@ -164,15 +165,37 @@ struct MiddleArgs {
 };
 
 struct NoHook {
-    __device__ __forceinline__ void operator()() const {}
+    template <typename I>
+    __device__ __forceinline__ void operator()(I) const {}
 };
-// hook: called once the loads that depend on nothing have been requested (a caller that goes on in the same
-// workgroup requests its own data there: loads return in order, so these come back first)
-// probs_lds (may be null): LDS copy of the row's probabilities, tokens 0 .. R + tail, for a caller that goes on in the
-// same workgroup
-template <int D, int NT, typename Hook = NoHook>
-__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u32 *amin_lds = nullptr, Hook hook = Hook(),
-                                            unsigned short *probs_lds = nullptr);
+template <int I>
+struct HookPoint {
+    static constexpr int value = I;
+};
+
+// LDS of the middle stage of one (batch, head) row, NW waves.
+template <int D, int NW>
+struct MiddleShared {
+    float red[NW];
+    unsigned short tail_s[64];     // fp16 scores of the tail (mask not yet added)
+    float tail_p[64];              // probabilities of the tail
+    u32 cand_key[4 * NW][32];      // [16-lane row of the workgroup][residue class]: best (probability, token) key
+    float probe_p[32];
+    int probe_t[32];
+    u32 red_min[NW];
+    float tail_o[NW][D];           // per-wave sums of the tail's share of the output
+    u32 vcm[D];                    // V column maxima after the append (SPLIT)
+    u32 amin;                      // the row's alignment threshold (SPLIT)
+};
+
+// the tail's share of channel d of the output: the waves' sums in a fixed order
+template <int D, int NW>
+__device__ __forceinline__ float middle_tail_output(const MiddleShared<D, NW> &ms, int d) {
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) sum += ms.tail_o[w][d];
+    return sum;
+}
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every outstanding
 // global store of the wave (here: 8 KiB of probabilities on their way to memory), which nobody inside the
@@ -209,19 +232,71 @@ __device__ __forceinline__ void decode_scores8(const u32x4 w, const unsigned sho
     }
 }
 
-// NT threads (a multiple of 256) of one workgroup run the stage for one (batch, head).
-template <int D, int NT, typename Hook>
-__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u32 *amin_lds, Hook hook, unsigned short *probs_lds) {
+// What a thread of the middle stage keeps for the tail's share of the output (middle_tail_partials): its 16-byte
+// pieces of the tail's value rows, requested with the stage's first loads.
+template <int D, int NT>
+struct MiddleCarry {
+    static constexpr int VPR = D / 8;                // 16-byte vectors per row
+    static constexpr int NRG = NT / VPR;             // row groups
+    static constexpr int MAXR = (64 + NRG - 1) / NRG;
+    static_assert(VPR <= 32, "head_dim above 256 needs another tail mapping");
+    u32x4 tvw[MAXR];
+    int nrest;
+};
+
+// The tail's share of the output, an fp16 matmul result (extension/v_cache_file.py:189): a thread takes 8 channels of
+// every NRG-th tail token, lanes of a wave that share the channels fold by shuffles; leaves the wave's sums in
+// ms.tail_o[wave] (the caller synchronises and adds the waves up: middle_tail_output).  Needs ms.tail_p.
+template <int D, int NT>
+__device__ __forceinline__ void middle_tail_partials(MiddleShared<D, NT / 64> &ms, const MiddleCarry<D, NT> &c) {
+    using C = MiddleCarry<D, NT>;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c8 = tid % C::VPR, rg = tid / C::VPR;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int k = 0; k < C::MAXR; ++k) {
+        const int r = rg + k * C::NRG;
+        const u32 vv[4] = {c.tvw[k].x, c.tvw[k].y, c.tvw[k].z, c.tvw[k].w};
+        const float pr = r < c.nrest ? ms.tail_p[r] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            acc[2 * i] = fmaf(lo_half_to_float(vv[i]), pr, acc[2 * i]);
+            acc[2 * i + 1] = fmaf(hi_half_to_float(vv[i]), pr, acc[2 * i + 1]);
+        }
+    }
+#pragma unroll
+    for (int mk = C::VPR; mk < 64; mk <<= 1)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] += __shfl_xor(acc[i], mk, 64);
+    if (lane < C::VPR) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ms.tail_o[wave][c8 * 8 + i] = acc[i];
+    }
+}
+
+// The middle stage of one (batch, head) row by the NT threads (a multiple of 256) of one workgroup: append, scores of
+// the tail, softmax, probe, threshold, the tail's share of the output.
+// hook(HookPoint<i>): a caller that goes on in the same workgroup requests its own data there.  SPLIT = false: i = 0,
+// called once the loads that depend on nothing have been requested (loads return in order, so these come back first).
+// SPLIT = true: called when the stage's own loads have all arrived (i = 0; requests made earlier share the memory
+// system with the stage's first loads and hold them back by as long as they take themselves: measured 4 us for 16 KiB
+// per wave), after the row maximum (1), after the row sum (2) and when the probabilities are out (3): a wave cannot
+// run ahead of a load the compute unit's memory pipeline has no room for yet, so what is to travel during the stage
+// is requested piece by piece between its phases.
+// probs_lds (may be null): LDS copy of the row's probabilities, tokens 0 .. R + tail, for a caller that goes on in the
+// same workgroup.
+// SPLIT = false: the whole stage; threshold in a.amin (and ms.amin), tail output in a.otail.
+// SPLIT = true (needs R > 0): everything up to the probabilities, the residue classes' candidates (ms.cand_key), the
+// column maxima (ms.vcm) and the tail's probabilities (ms.tail_p), ending with an LDS barrier; the caller lets one wave
+// run middle_probe_wave (probe and threshold, no barrier inside) while the others go on, and calls
+// middle_tail_partials with `carry` when it suits it (every wave, before the workgroup adds up ms.tail_o).
+template <int D, int NT, bool SPLIT = false, typename Hook = NoHook>
+__device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, MiddleShared<D, NT / 64> &ms, Hook hook = Hook(),
+                                            unsigned short *probs_lds = nullptr, MiddleCarry<D, NT> *carry_out = nullptr) {
     constexpr int VPT = 4;                    // 16-byte score vectors a thread keeps in registers
     constexpr int NW = NT / 64;               // waves
-    __shared__ float red[NW];
-    __shared__ unsigned short tail_s[64];     // fp16 scores of the tail (mask not yet added)
-    __shared__ float tail_p[64];              // probabilities of the tail
-    __shared__ u32 cand_key[NW][32];
-    __shared__ float probe_p[32];
-    __shared__ int probe_t[32];
-    __shared__ u32 red_min[NW];
-    __shared__ float tail_o[NW][D];           // per-wave sums of the tail's share of the output
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // bh indexes (batch, query head); the keys, values, column maxima and rest buffers belong to its KV head
     const int b = bh / a.g.Hq, hq = bh - b * a.g.Hq, h = hq / a.g.G;
@@ -251,7 +326,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
     };
 
     // Everything that does not depend on anything else is requested first: the score vectors of the
-    // flushed part, the new token and the column maxima.
+    // flushed part, the new token, the column maxima and the tail's key and value rows.
     u32x4 sv[VPT];
     if (in_regs) {
 #pragma unroll
@@ -285,9 +360,11 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
         const int d = on ? tid : 0;
         u32 kc = a.kcm[(int64_t)bh_kv * D + d], vc = a.vcm[(int64_t)bh_kv * D + d];
         const u32 kb = knew[d], vb = vnew[d];
-        __builtin_amdgcn_sched_barrier(0);
-        hook();
-        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (!SPLIT) {
+            __builtin_amdgcn_sched_barrier(0);
+            hook(HookPoint<0>());
+            __builtin_amdgcn_sched_barrier(0);
+        }
         if (a.persist) {
             // every query head of the group derives the updated maxima itself (max is idempotent, so it does
             // not matter whether it reads them before or after the owner's store); only the owner stores
@@ -302,7 +379,23 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
             }
         }
         vcm_mine = vc;
+        if (SPLIT && on) ms.vcm[d] = vc;
     }
+    // value rows of the tail, used by (f): a thread takes 8 channels of every NRG-th tail token
+    using Carry = MiddleCarry<D, NT>;
+    Carry carry;
+    carry.nrest = nrest;
+    auto request_tail_values = [&]() {
+        const int c8 = tid % Carry::VPR, rg = tid / Carry::VPR;
+#pragma unroll
+        for (int k = 0; k < Carry::MAXR; ++k) {
+            const int r = rg + k * Carry::NRG;
+            const unsigned short *vrow = (r == newest && a.persist) ? vnew : a.restv + (((int64_t)b * cb + r) * Hkv + h) * D;
+            carry.tvw[k] = r < nrest ? *reinterpret_cast<const u32x4 *>(vrow + c8 * 8) : (u32x4){0u, 0u, 0u, 0u};
+        }
+    };
+    // (SPLIT: with the first loads, so that nothing the stage needs later queues behind the caller's stream)
+    if (SPLIT) request_tail_values();
     // (b) scores of the tail: fp16(fp16(q.k) / sqrt(D)), the two roundings of an fp16 matmul followed by
     //     an fp16 division (extension/k_cache_file.py:156)
     const float sqrt_d = sqrtf((float)D);
@@ -322,11 +415,21 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
         if (tr < nrest && tj == 0) {
             const float dot16 = half_bits_to_float(float_to_half_bits(part));
             const unsigned short sc = float_to_half_bits(dot16 / sqrt_d);
-            tail_s[tr] = sc;
+            ms.tail_s[tr] = sc;
             srow[R + tr] = sc;
         }
     }
     lds_barrier();
+    AKV_MARK(bh, 10);
+    // SPLIT: the stage's loads are all back; from here to the probe it only computes, and memory is the caller's
+    auto hook_at = [&](auto point) {
+        if constexpr (SPLIT) {
+            __builtin_amdgcn_sched_barrier(0);
+            hook(point);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    hook_at(HookPoint<0>());
 
     // (c) softmax over [0, R + nrest): scores + mask in fp16, softmax in fp32, probabilities in fp16
     //     (model/KVCache_AlignedKV.py:119-121), and the running arg-max of the residue classes mod 32:
@@ -342,8 +445,21 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
     u32 best[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) best[j] = 0u;
-    const float xt = tid < nrest ? masked1(tail_s[tid], R + tid) : -INFINITY;
+    const float xt = tid < nrest ? masked1(ms.tail_s[tid], R + tid) : -INFINITY;
     float m = xt, sum = 0.f;
+    auto emit_probs8 = [&](int i, const float *e, float rsum) {
+        u32 out[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const u32 p0 = float_to_half_bits(div_by(e[2 * j], sum, rsum)), p1 = float_to_half_bits(div_by(e[2 * j + 1], sum, rsum));
+            out[j] = p0 | (p1 << 16);
+            const u32 grp = 0xffffu - (u32)(i >> 2);     // token / 32 = vector index / 4
+            best[2 * j] = max(best[2 * j], (p0 << 16) | grp);
+            best[2 * j + 1] = max(best[2 * j + 1], (p1 << 16) | grp);
+        }
+        const u32x4 o = {out[0], out[1], out[2], out[3]};
+        store_probs8(i, o);
+    };
     if (in_regs) {
         float x[VPT][8];
 #pragma unroll
@@ -355,40 +471,32 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
                 for (int j = 0; j < 8; ++j) m = fmaxf(m, x[v][j]);
             }
         }
-        m = block_reduce<NW>(m, true, red);
+        m = block_reduce<NW>(m, true, ms.red);
+        AKV_MARK(bh, 11);
+        hook_at(HookPoint<1>());
 #pragma unroll
         for (int v = 0; v < VPT; ++v)
             if (tid + NT * v < nvec) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    x[v][j] = expf(x[v][j] - m);
+                    x[v][j] = exp_nonpositive(x[v][j] - m);
                     sum += x[v][j];
                 }
             }
-        const float et = tid < nrest ? expf(xt - m) : 0.f;
-        sum = block_reduce<NW>(sum + et, false, red);
+        const float et = tid < nrest ? exp_nonpositive(xt - m) : 0.f;
+        sum = block_reduce<NW>(sum + et, false, ms.red);
+        AKV_MARK(bh, 12);
+        hook_at(HookPoint<2>());
         const float rsum = 1.0f / sum;
 #pragma unroll
         for (int v = 0; v < VPT; ++v) {
             const int i = tid + NT * v;
-            if (i < nvec) {
-                u32 out[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const u32 p0 = float_to_half_bits(div_by(x[v][2 * j], sum, rsum)), p1 = float_to_half_bits(div_by(x[v][2 * j + 1], sum, rsum));
-                    out[j] = p0 | (p1 << 16);
-                    const u32 grp = 0xffffu - (u32)(i >> 2);     // token / 32 = vector index / 4
-                    best[2 * j] = max(best[2 * j], (p0 << 16) | grp);
-                    best[2 * j + 1] = max(best[2 * j + 1], (p1 << 16) | grp);
-                }
-                const u32x4 o = {out[0], out[1], out[2], out[3]};
-                store_probs8(i, o);
-            }
+            if (i < nvec) emit_probs8(i, x[v], rsum);
         }
         if (tid < nrest) {
             const unsigned short p = float_to_half_bits(div_by(et, sum, rsum));
             store_prob1(R + tid, p);
-            tail_p[tid] = half_bits_to_float(p);
+            ms.tail_p[tid] = half_bits_to_float(p);
         }
     } else {
         // long rows: three passes over the scores (they stay in the L2 of this workgroup's XCD)
@@ -398,138 +506,156 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, u
 #pragma unroll
             for (int j = 0; j < 8; ++j) m = fmaxf(m, x[j]);
         }
-        m = block_reduce<NW>(m, true, red);
+        m = block_reduce<NW>(m, true, ms.red);
         for (int i = tid; i < nvec; i += NT) {
             decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) sum += expf(x[j] - m);
+            for (int j = 0; j < 8; ++j) sum += exp_nonpositive(x[j] - m);
         }
-        const float et = tid < nrest ? expf(xt - m) : 0.f;
-        sum = block_reduce<NW>(sum + et, false, red);
+        const float et = tid < nrest ? exp_nonpositive(xt - m) : 0.f;
+        sum = block_reduce<NW>(sum + et, false, ms.red);
         const float rsum = 1.0f / sum;
+        hook_at(HookPoint<1>());
+        hook_at(HookPoint<2>());
         for (int i = tid; i < nvec; i += NT) {
             decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
-            u32 out[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const u32 p0 = float_to_half_bits(div_by(expf(x[2 * j] - m), sum, rsum)), p1 = float_to_half_bits(div_by(expf(x[2 * j + 1] - m), sum, rsum));
-                out[j] = p0 | (p1 << 16);
-                const u32 grp = 0xffffu - (u32)(i >> 2);
-                best[2 * j] = max(best[2 * j], (p0 << 16) | grp);
-                best[2 * j + 1] = max(best[2 * j + 1], (p1 << 16) | grp);
-            }
-            const u32x4 o = {out[0], out[1], out[2], out[3]};
-            store_probs8(i, o);
+            for (int j = 0; j < 8; ++j) x[j] = exp_nonpositive(x[j] - m);
+            emit_probs8(i, x, rsum);
         }
         if (tid < nrest) {
             const unsigned short p = float_to_half_bits(div_by(et, sum, rsum));
             store_prob1(R + tid, p);
-            tail_p[tid] = half_bits_to_float(p);
+            ms.tail_p[tid] = half_bits_to_float(p);
         }
     }
 
-    // value rows of the tail, used by (f): requested here so that they travel while the probe runs
-    constexpr int VPR = D / 8;                // 16-byte vectors per row
-    constexpr int NRG = NT / VPR;             // row groups
-    constexpr int MAXR = (64 + NRG - 1) / NRG;
-    static_assert(VPR <= 32, "head_dim above 256 needs another tail mapping");
-    const int c8 = tid % VPR, rg = tid / VPR;
-    u32x4 tvw[MAXR];
-#pragma unroll
-    for (int k = 0; k < MAXR; ++k) {
-        const int r = rg + k * NRG;
-        const unsigned short *vrow = (r == newest && a.persist) ? vnew : a.restv + (((int64_t)b * cb + r) * Hkv + h) * D;
-        tvw[k] = r < nrest ? *reinterpret_cast<const u32x4 *>(vrow + c8 * 8) : (u32x4){0u, 0u, 0u, 0u};
-    }
+    AKV_MARK(bh, 13);
+    hook_at(HookPoint<3>());
+    // value rows of the tail: requested here so that they travel while the probe runs
+    if (!SPLIT) request_tail_values();
 
-    // (d)+(e) probe over the flushed part (extension/v_cache_file.py:119-143) and the alignment threshold
-    //     of this (batch, head) (extension/v_cache_file.py:156-160)
+    // (d) candidates of the probe over the flushed part (extension/v_cache_file.py:119-143): thread tid saw residues
+    //     8*(tid&3)+j.  Lanes of a 16-lane row that share (tid&3): two row rotations (DPP); then one LDS row per
+    //     16-lane row (the arg-max over these rows is taken by whoever runs the probe).
     if (R > 0) {
-        // thread tid saw residues 8*(tid&3)+j.  Lanes of a wave that share (tid&3): two row rotations (DPP)
-        // inside a 16-lane row, two shuffles across rows; then one LDS row per wave and a last scan.
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             best[j] = max(best[j], (u32)__builtin_amdgcn_update_dpp(0, (int)best[j], 0x124, 0xf, 0xf, false));   // row_ror:4
             best[j] = max(best[j], (u32)__builtin_amdgcn_update_dpp(0, (int)best[j], 0x128, 0xf, 0xf, false));   // row_ror:8
-            best[j] = max(best[j], (u32)__shfl_xor((int)best[j], 16, 64));
-            best[j] = max(best[j], (u32)__shfl_xor((int)best[j], 32, 64));
         }
-        if (lane < 4) {
+        if ((lane & 15) < 4) {
 #pragma unroll
-            for (int j = 0; j < 8; ++j) cand_key[wave][8 * lane + j] = best[j];
+            for (int j = 0; j < 8; ++j) ms.cand_key[tid >> 4][8 * (lane & 3) + j] = best[j];
         }
-        lds_barrier();
-        if (tid < 32) {
-            u32 key = 0u;
-#pragma unroll
-            for (int k = 0; k < NW; ++k) key = max(key, cand_key[k][tid]);
-            probe_p[tid] = half_bits_to_float(key >> 16);
-            probe_t[tid] = (int)(0xffffu - (key & 0xffffu)) * 32 + tid;
-        }
-        lds_barrier();
-        u32 align = 0xffu;
-        for (int d = tid; d < D; d += NT) {
-            // the 32 gathered bytes first, then the sum: 32 independent loads in flight instead of a chain
-            u32 hi[32];
-#pragma unroll
-            for (int i = 0; i < 32; ++i) hi[i] = a.v_first_8[((int64_t)bh_kv * a.g.max_seq_len + probe_t[i]) * D + d];
-            float acc = 0.f;
-#pragma unroll
-            for (int i = 0; i < 32; ++i)
-                acc = fmaf(half_bits_to_float(((hi[i] << 8) | 0x80u) & 0x7fffu), probe_p[i], acc);
-            // exponent with the lowest bit cleared (`& 0x1F - 1`, extension/v_cache_file.py:142)
-            const u32 e = exp_field(float_to_half_bits(acc)) & 0x1eu;
-            a.toe[(int64_t)bh * D + d] = (uint8_t)e;
-            align = min(align, (e + 15u - vcm_mine) & 0xffu);     // uint8 wrap, as the reference's tensor arithmetic
-        }
-#pragma unroll
-        for (int mk = 32; mk >= 1; mk >>= 1) align = min(align, (u32)__shfl_xor((int)align, mk, 64));
-        if (lane == 0) red_min[wave] = align;
-        lds_barrier();
-        if (tid == 0) {
-            u32 mn = red_min[0];
-#pragma unroll
-            for (int w = 1; w < NW; ++w) mn = min(mn, red_min[w]);
-            a.amin[bh] = (uint8_t)mn;
-            if (amin_lds != nullptr) *amin_lds = mn;   // for a caller that goes on in the same workgroup
-        }
-    } else {
-        lds_barrier();
     }
-    // (f) the tail's share of the output, an fp16 matmul result (extension/v_cache_file.py:189): a thread takes 8
-    //     channels of every NRG-th tail token (requested before the probe), lanes of a wave that share the channels
-    //     fold by shuffles, waves by LDS
-    {
-        float acc[8];
+    lds_barrier();
+    // (e) the probe's arg-max per residue class, its 32 gathered rows and the alignment threshold of this (batch, head)
+    //     (extension/v_cache_file.py:156-160)
+    if constexpr (!SPLIT) {
+        if (R > 0) {
+            if (tid < 32) {
+                u32 key = 0u;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+                for (int k = 0; k < 4 * NW; ++k) key = max(key, ms.cand_key[k][tid]);
+                ms.probe_p[tid] = half_bits_to_float(key >> 16);
+                ms.probe_t[tid] = (int)(0xffffu - (key & 0xffffu)) * 32 + tid;
+            }
+            lds_barrier();
+            u32 align = 0xffu;
+            for (int d = tid; d < D; d += NT) {
+                // the 32 gathered bytes first, then the sum: 32 independent loads in flight instead of a chain
+                u32 hi[32];
 #pragma unroll
-        for (int k = 0; k < MAXR; ++k) {
-            const int r = rg + k * NRG;
-            const u32 vv[4] = {tvw[k].x, tvw[k].y, tvw[k].z, tvw[k].w};
-            const float pr = r < nrest ? tail_p[r] : 0.f;
+                for (int i = 0; i < 32; ++i) hi[i] = a.v_first_8[((int64_t)bh_kv * a.g.max_seq_len + ms.probe_t[i]) * D + d];
+                float acc = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                acc[2 * i] = fmaf(lo_half_to_float(vv[i]), pr, acc[2 * i]);
-                acc[2 * i + 1] = fmaf(hi_half_to_float(vv[i]), pr, acc[2 * i + 1]);
+                for (int i = 0; i < 32; ++i)
+                    acc = fmaf(half_bits_to_float(((hi[i] << 8) | 0x80u) & 0x7fffu), ms.probe_p[i], acc);
+                // exponent with the lowest bit cleared (`& 0x1F - 1`, extension/v_cache_file.py:142)
+                const u32 e = exp_field(float_to_half_bits(acc)) & 0x1eu;
+                a.toe[(int64_t)bh * D + d] = (uint8_t)e;
+                align = min(align, (e + 15u - vcm_mine) & 0xffu);     // uint8 wrap, as the reference's tensor arithmetic
+            }
+#pragma unroll
+            for (int mk = 32; mk >= 1; mk >>= 1) align = min(align, (u32)__shfl_xor((int)align, mk, 64));
+            if (lane == 0) ms.red_min[wave] = align;
+            lds_barrier();
+            if (tid == 0) {
+                u32 mn = ms.red_min[0];
+#pragma unroll
+                for (int w = 1; w < NW; ++w) mn = min(mn, ms.red_min[w]);
+                a.amin[bh] = (uint8_t)mn;
+                ms.amin = mn;   // for a caller that goes on in the same workgroup
             }
         }
-#pragma unroll
-        for (int mk = VPR; mk < 64; mk <<= 1)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) acc[i] += __shfl_xor(acc[i], mk, 64);
-        if (lane < VPR) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) tail_o[wave][c8 * 8 + i] = acc[i];
-        }
-        lds_barrier();
-        for (int d = tid; d < D; d += NT) {
-            float sum = 0.f;
-#pragma unroll
-            for (int w = 0; w < NW; ++w) sum += tail_o[w][d];
-            a.otail[(int64_t)bh * D + d] = float_to_half_bits(sum);
-        }
     }
+    // (f) the tail's share of the output
+    if constexpr (SPLIT) {
+        *carry_out = carry;
+    } else {
+        middle_tail_partials<D, NT>(ms, carry);
+        lds_barrier();
+        for (int d = tid; d < D; d += NT) a.otail[(int64_t)bh * D + d] = float_to_half_bits(middle_tail_output<D, NW>(ms, d));
+    }
+}
+
+// The probe and the alignment threshold of a row by ONE wave (no workgroup barrier inside), after middle_body<SPLIT>:
+// the arg-max of every residue class from the waves' candidates, the 32 gathered high-byte rows (lane = D / 64
+// neighbouring channels, a row per load instruction, the row's token in a scalar register), the probe's exponents and
+// the threshold, which goes to a.amin and ms.amin.  extension/v_cache_file.py:119-143,156-160.
+// while_waiting: called once the gather has been requested.
+template <int D, int NW, typename Waiting>
+__device__ __forceinline__ u32 middle_probe_wave(const MiddleArgs &a, MiddleShared<D, NW> &ms, int bh, int R, Waiting while_waiting) {
+    constexpr int CPL = D / 64;               // channels per lane
+    static_assert(CPL == 1 || CPL == 2 || CPL == 4, "head_dim 64, 128 or 256");
+    const int lane = threadIdx.x & 63;
+    const int b = bh / a.g.Hq, hq = bh - b * a.g.Hq, h = hq / a.g.G;
+    const int bh_kv = b * a.g.Hkv + h;
+    // arg-max of residue class r = lane % 32 over the candidates of half of the rows; the two halves meet in scalar
+    // registers below
+    const int r = lane & 31, half = lane >> 5;
+    u32 key = 0u;
+#pragma unroll
+    for (int k = 0; k < 2 * NW; ++k) key = max(key, ms.cand_key[half * 2 * NW + k][r]);
+    const __amdgpu_buffer_rsrc_t rF = make_rsrc(a.v_first_8 + (int64_t)bh_kv * a.g.max_seq_len * D, (u32)R * D);
+    u32 hi[32], pbits[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        const u32 k_i = max((u32)__builtin_amdgcn_readlane((int)key, i), (u32)__builtin_amdgcn_readlane((int)key, i + 32));
+        pbits[i] = k_i >> 16;
+        const int row = ((int)(0xffffu - (k_i & 0xffffu)) * 32 + i) * D;
+        if constexpr (CPL == 1) hi[i] = (u32)(unsigned char)__builtin_amdgcn_raw_buffer_load_b8(rF, lane, row, 0);
+        else if constexpr (CPL == 2) hi[i] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rF, lane * 2, row, 0);
+        else hi[i] = __builtin_amdgcn_raw_buffer_load_b32(rF, lane * 4, row, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    while_waiting();
+    __builtin_amdgcn_sched_barrier(0);
+    float acc[CPL];
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) acc[c] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+        const float p = half_bits_to_float(pbits[i]);
+#pragma unroll
+        for (int c = 0; c < CPL; ++c)
+            acc[c] = fmaf(half_bits_to_float(((((hi[i] >> (8 * c)) & 0xffu) << 8) | 0x80u) & 0x7fffu), p, acc[c]);
+    }
+    u32 align = 0xffu;
+#pragma unroll
+    for (int c = 0; c < CPL; ++c) {
+        // exponent with the lowest bit cleared (`& 0x1F - 1`, extension/v_cache_file.py:142)
+        const u32 e = exp_field(float_to_half_bits(acc[c])) & 0x1eu;
+        a.toe[(int64_t)bh * D + lane * CPL + c] = (uint8_t)e;
+        align = min(align, (e + 15u - ms.vcm[lane * CPL + c]) & 0xffu);     // uint8 wrap, as the reference's tensor arithmetic
+    }
+    align = wave_min_u32(align);
+    if (lane == 0) {
+        a.amin[bh] = (uint8_t)align;
+        ms.amin = align;
+    }
+    return align;
 }
 
 }  // namespace akv
