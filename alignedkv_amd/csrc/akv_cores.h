@@ -769,8 +769,8 @@ __device__ __forceinline__ void v_stream_run_deferred(VRing<D, NRING> &ring, con
 struct NoExtra {
     __device__ __forceinline__ void operator()(int) const {}
 };
-template <int D, typename Extra = NoExtra>
-__device__ __forceinline__ void v_stream_run_coarse(VRing<D, 2> &ring, const uint8_t *f8, int n_tokens,
+template <int D, int RN, typename Extra = NoExtra>
+__device__ __forceinline__ void v_stream_run_coarse(VRing<D, RN> &ring, const uint8_t *f8, int n_tokens,
                                                    const unsigned short *probs_lds, const VSeq &seq, bool prefetched, int next_half,
                                                    float *acc, Extra extra = Extra()) {
     using S = VStream<D>;
