@@ -35,8 +35,18 @@ SIGNATURES = {
     "akv_profile_read_empty": (c_int, [_P]),
     "akv_decode_step_workspace_bytes": (c_size_t, [_I, _I, _I, _I]),
     "akv_decode_step": (c_int, [_P] * 14 + [_I] + [_P] * 3 + [_I, _P, c_size_t] + [_P] * 3 + [_I] * 12 + [_P]),
+    "akv_decode_step_desc": (c_int, [_P] * 5 + [_I] + [_P] * 4 + [_I, _P, _I, _I, _P]),
     "akv_decode_step_static": (c_int, [_P] * 14 + [_I] + [_P] * 3 + [_I] + [_P] * 3 + [_I] * 12 + [_P]),
 }
+
+
+class StepDesc(ctypes.Structure):
+    """akv_step_desc of include/alignedkv.h."""
+    _fields_ = ([(n, _P) for n in ("k_first_8", "k_mid_4", "k_last_4", "v_first_8", "v_mid_4", "v_last_4", "k_exp_column_max",
+                                   "v_exp_column_max", "restk", "restv", "scores", "probs", "workspace")]
+                + [("workspace_bytes", c_size_t)]
+                + [(n, _I) for n in ("row_stride", "bsz", "n_q_heads", "n_kv_heads", "n_max_blocks", "max_seq_len", "head_dim",
+                                     "d_block", "k_block", "top_max_k")])
 
 
 def build(verbose: bool = False) -> str:

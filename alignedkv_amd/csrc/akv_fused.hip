@@ -997,6 +997,18 @@ extern "C" int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t
 #undef AKV_STEP
 }
 
+extern "C" int akv_decode_step_desc(const akv_step_desc *d, const uint8_t *q, const uint8_t *k_new, const uint8_t *v_new,
+                                    const uint8_t *mask, int mask_stride, uint8_t *out, uint8_t *k_levels_out,
+                                    uint8_t *v_levels_out, uint8_t *amin_out, int cur_len, int *seq_lens, int reference,
+                                    int literal_broadcast, akv_stream_t stream) {
+    AKV_REQUIRE(d != nullptr, "decode_step: null descriptor");
+    return akv_decode_step_gqa(d->k_first_8, d->k_mid_4, d->k_last_4, d->v_first_8, d->v_mid_4, d->v_last_4, d->k_exp_column_max,
+                               d->v_exp_column_max, d->restk, d->restv, q, k_new, v_new, mask, mask_stride, out, d->scores,
+                               d->probs, d->row_stride, d->workspace, d->workspace_bytes, k_levels_out, v_levels_out, amin_out,
+                               d->bsz, d->n_q_heads, d->n_kv_heads, d->n_max_blocks, d->max_seq_len, d->head_dim, d->d_block,
+                               d->k_block, d->top_max_k, cur_len, seq_lens, reference, literal_broadcast, stream);
+}
+
 extern "C" int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,
                                uint8_t *v_mid_4, uint8_t *v_last_4, uint8_t *k_exp_column_max,
                                uint8_t *v_exp_column_max, uint8_t *restk, uint8_t *restv, const uint8_t *q,

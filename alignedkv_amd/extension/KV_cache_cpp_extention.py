@@ -15,7 +15,12 @@ from .._lib import check, load_library
 
 
 def _stream_ptr(device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """Raw handle of the current stream of `device` (the fast path of torch.cuda.current_stream(device).cuda_stream)."""
+    try:
+        index = device.index if isinstance(device, torch.device) else torch.device(device).index
+        return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if index is None else index)
+    except (AttributeError, TypeError):
+        return torch.cuda.current_stream(device).cuda_stream
 
 
 def _ptr(t):
@@ -260,17 +265,18 @@ class _AlignedKVModule:
 
 
 class PreparedDecodeStep:
-    """akv_decode_step_gqa for one layer of a multi-head cache with everything that does not change between its steps
-    checked and converted once: plane, column-maximum, rest-buffer, score and workspace pointers and the geometry.
-    A call checks only the three token tensors and the output.  Made by `cuda_module.prepare_decode_step`; `key`
-    lets the owner notice that one of the captured tensors was replaced (then it prepares again)."""
+    """The fused step for one layer of a multi-head cache with everything that does not change between its steps
+    checked and converted once into an akv_step_desc: plane, column-maximum, rest-buffer, score and workspace pointers
+    and the geometry.  A call checks only the three token tensors and the output (fp16 or uint8 views, contiguous) and
+    passes 15 arguments.  Made by `cuda_module.prepare_decode_step`; `key` lets the owner notice that one of the
+    captured tensors was replaced (then it prepares again)."""
 
-    def __init__(self, lib, static_head, static_mid, geometry, tok_bytes, device, stream, key, keep):
-        self._fn = lib.akv_decode_step_gqa
+    def __init__(self, lib, desc, tok_bytes, device, stream, key, keep):
+        import ctypes
+        self._fn = lib.akv_decode_step_desc
         self._lib = lib
-        self._head = static_head        # 10 pointers: planes, column maxima, rest buffers
-        self._mid = static_mid          # scores, probs, row_stride, workspace, workspace bytes
-        self._geo = geometry            # bsz, q heads, kv heads, n_max_blocks, max_seq_len, head_dim, d_block, k_block, top_max_k
+        self._desc = desc
+        self._desc_ref = ctypes.byref(desc)
         self._tok = tok_bytes
         self.device = device
         self.stream = stream
@@ -281,12 +287,12 @@ class PreparedDecodeStep:
                  k_levels_out=None, v_levels_out=None, amin_out=None):
         tok = self._tok
         for t in (q, k_new, v_new, out):
-            if t.dtype != torch.uint8 or t.numel() != tok or not t.is_contiguous() or t.device != self.device:
-                raise RuntimeError("decode step: q, k_new, v_new and out must be contiguous uint8 views of "
+            if t.numel() * t.element_size() != tok or not t.is_contiguous() or t.device != self.device:
+                raise RuntimeError("decode step: q, k_new, v_new and out must be contiguous fp16 tensors (or uint8 views) of "
                                    f"{tok} bytes on {self.device}")
-        rc = self._fn(*self._head, q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), _ptr(mask), mask_stride,
-                      out.data_ptr(), *self._mid, _ptr(k_levels_out), _ptr(v_levels_out), _ptr(amin_out), *self._geo,
-                      cur_len, None, int(bool(reference)), int(bool(literal_broadcast)), self.stream)
+        rc = self._fn(self._desc_ref, q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), _ptr(mask), mask_stride,
+                      out.data_ptr(), _ptr(k_levels_out), _ptr(v_levels_out), _ptr(amin_out), cur_len, None,
+                      1 if reference else 0, 1 if literal_broadcast else 0, self.stream)
         if rc != 0:
             check(rc, self._lib)
 
@@ -312,11 +318,12 @@ def _prepare_decode_step(self, k_planes, v_planes, k_exp_column_max, v_exp_colum
     _require("probs", probs, bsz * n_kv_heads * row_stride * 2, dev)
     need = lib.akv_decode_step_workspace_bytes(bsz, n_kv_heads, head_dim, max_seq_len)
     ws = self._workspace(dev, need)
-    head = tuple(_ptr(t) for t in (*k_planes, *v_planes, k_exp_column_max, v_exp_column_max, restk, restv))
-    mid = (_ptr(scores), _ptr(probs), row_stride, _ptr(ws), ws.numel())
-    geo = (bsz, n_kv_heads, n_kv_heads, n_max_blocks, max_seq_len, head_dim, d_block, k_block, top_max_k)
+    from .._lib import StepDesc
+    desc = StepDesc(*(_ptr(t) for t in (*k_planes, *v_planes, k_exp_column_max, v_exp_column_max, restk, restv, scores, probs, ws)),
+                    ws.numel(), row_stride, bsz, n_kv_heads, n_kv_heads, n_max_blocks, max_seq_len, head_dim, d_block, k_block,
+                    top_max_k)
     keep = (k_planes, v_planes, k_exp_column_max, v_exp_column_max, restk, restv, scores, probs, ws)
-    return PreparedDecodeStep(lib, head, mid, geo, tok, dev, _stream_ptr(dev), key, keep)
+    return PreparedDecodeStep(lib, desc, tok, dev, _stream_ptr(dev), key, keep)
 
 
 _AlignedKVModule.prepare_decode_step = _prepare_decode_step

@@ -169,12 +169,12 @@ class QuantizedCache_AlignedKV(_HFCache):
         vc._check_save(v, start_pos, 1, "new_v")
         assert tuple(q.shape) == tuple(k.shape), f"q.shape: {tuple(q.shape)} != {tuple(k.shape)}"
         assert kc.reststartpos + kc._restlen == start_pos
-        B, H, D = self.max_batch_size, self.num_key_value_heads, self.head_dim
         step = self._prepared_step(layer_id, q.device)
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         out = torch.empty_like(q)
         klv = vlv = amin = None
         if kc.record_levels or vc.record_levels:
+            B, H, D = self.max_batch_size, self.num_key_value_heads, self.head_dim
             flushed = kc.reststartpos + (column_block if kc._restlen + 1 == column_block else 0)
             klv = torch.empty((B, H, D), dtype=torch.uint8, device=q.device)
             vlv = torch.empty((B, H, flushed), dtype=torch.uint8, device=q.device) if flushed else None
@@ -184,13 +184,12 @@ class QuantizedCache_AlignedKV(_HFCache):
             if mask2d.shape[1] < 2 * (start_pos + 1):
                 raise RuntimeError(f"mask: shape {tuple(mask2d.shape)} does not cover {start_pos + 1} halves")
             mask_stride = 0 if mask2d.shape[0] == 1 else mask2d.stride(0) // 2
-        if q.device != torch.device("cuda", torch.cuda.current_device()):
+        # (the step takes the fp16 tensors as they are: it reads their bytes)
+        if q.device.index != torch.cuda.current_device():
             with torch.cuda.device(q.device):
-                step(q.view(torch.uint8), k.view(torch.uint8), v.view(torch.uint8), out.view(torch.uint8), mask2d,
-                     mask_stride, start_pos, self.reference, self.literal_broadcast, klv, vlv, amin)
+                step(q, k, v, out, mask2d, mask_stride, start_pos, self.reference, self.literal_broadcast, klv, vlv, amin)
         else:
-            step(q.view(torch.uint8), k.view(torch.uint8), v.view(torch.uint8), out.view(torch.uint8), mask2d,
-                 mask_stride, start_pos, self.reference, self.literal_broadcast, klv, vlv, amin)
+            step(q, k, v, out, mask2d, mask_stride, start_pos, self.reference, self.literal_broadcast, klv, vlv, amin)
         kc._advance_after_fused_step()
         vc._advance_after_fused_step()
         if klv is not None:

@@ -208,6 +208,26 @@ AKV_API int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k
                                 int literal_broadcast, akv_stream_t stream);
 
 /*
+ * akv_decode_step_gqa with everything that stays the same from step to step of one layer gathered in a descriptor the
+ * caller fills once: a step then passes 15 arguments instead of 38, which is what a host binding pays per call (the
+ * reference's Python layer calls its ops once per layer and decode step, model/KVCache_AlignedKV.py:116-124).  Same
+ * checks, same kernels, same results as akv_decode_step_gqa with the descriptor's fields in place of its arguments.
+ */
+typedef struct akv_step_desc {
+    uint8_t *k_first_8, *k_mid_4, *k_last_4, *v_first_8, *v_mid_4, *v_last_4;
+    uint8_t *k_exp_column_max, *v_exp_column_max, *restk, *restv;
+    uint8_t *scores, *probs;
+    void *workspace;
+    size_t workspace_bytes;
+    int row_stride;
+    int bsz, n_q_heads, n_kv_heads, n_max_blocks, max_seq_len, head_dim, d_block, k_block, top_max_k;
+} akv_step_desc;
+AKV_API int akv_decode_step_desc(const akv_step_desc *desc, const uint8_t *q, const uint8_t *k_new, const uint8_t *v_new,
+                                 const uint8_t *mask, int mask_stride, uint8_t *out, uint8_t *k_levels_out,
+                                 uint8_t *v_levels_out, uint8_t *amin_out, int cur_len, int *seq_lens, int reference,
+                                 int literal_broadcast, akv_stream_t stream);
+
+/*
  * Dense fp16 decode attention, the baseline of the benchmark (semantics of the reference's dense branch,
  * model/Llama_AlignedKV.py:130-139): appends k_new / v_new at row cur_len of the head-major fp16 caches
  * [bsz, heads, max_seq_len, head_dim] and attends over cur_len + 1 tokens.  q, k_new, v_new, out: fp16
