@@ -178,8 +178,6 @@ __device__ __forceinline__ u32x4 load_b128_device(const __amdgpu_buffer_rsrc_t r
 // vector instructions.  (threadIdx.x >> 6 alone is a per-lane value to the compiler.)
 __device__ __forceinline__ int wave_index() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 
-__device__ __forceinline__ float wave_xor_add(float v, int mask) { return v + __shfl_xor(v, mask, 64); }
-
 // Wave-wide reductions with the result in every lane: two quad permutes and the two mirrors inside the 16-lane rows
 // (data-parallel primitives: no LDS round trip per step, unlike a shuffle), then the four row totals through scalar
 // registers.  The order of the additions is fixed, so the bits of a sum are reproducible.

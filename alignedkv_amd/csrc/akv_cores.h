@@ -694,69 +694,6 @@ __device__ __forceinline__ int v_stream_count_fine(const unsigned short *s_row, 
     return wave_sum_i32(n);
 }
 
-// The same with the tokens below level 2 taken out of the loop (VListed); the caller adds the listed tokens at the end
-// (v_stream_apply_list).  For rows where they are rare: a listed token costs a second fetch of its high bytes and a
-// share of a memory round trip of its own (at one token in nine the pass takes 52 instead of 30 us).
-// list: LDS, room for every token of the wave (n_per_wave * HT entries); count: its length.
-// LDSP: s_row is a copy of the row's probabilities in LDS; a half tile's probabilities are then read when it is
-// multiplied instead of travelling with its high bytes (four fewer memory instructions per half tile).
-template <int D, int NR, int PF, int NRING, bool LDSP = false>
-__device__ __forceinline__ void v_stream_run_deferred(VRing<D, NRING> &ring, const uint8_t *f8, int n_tokens,
-                                                     const unsigned short *s_row, unsigned char amin, const VSeq &seq,
-                                                     float *acc, u32 *list, int &count) {
-    using S = VStream<D>;
-    static_assert(NR >= 2 && NR <= NRING, "one slot is multiplied while the others travel");
-    constexpr int HV = S::HV;
-    const int lane = threadIdx.x & 63, tl = lane / S::LPR, cl = lane % S::LPR;
-    const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
-    const __amdgpu_buffer_rsrc_t rS = make_rsrc(s_row, (u32)n_tokens * 2);
-    auto issue = [&](int k, int half) {
-        if constexpr (LDSP) v_stream_issue_high<D>(ring.hi[k], rH, half);
-        else v_stream_issue<D, NRING>(ring, k, rH, rS, half);
-    };
-#pragma unroll
-    for (int k = PF; k < NR - 1; ++k) v_stream_issue_high<D>(ring.hi[k], rH, seq.half(k));
-    if constexpr (!LDSP) {
-#pragma unroll
-        for (int k = 0; k < NR - 1; ++k) v_stream_issue_probs<D>(ring.sb[k], rS, seq.half(k));
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    auto round = [&](int i0) {
-#pragma unroll
-        for (int k = 0; k < NR; ++k) {
-            issue((k + NR - 1) % NR, seq.half(i0 + k + NR - 1));
-            __builtin_amdgcn_sched_barrier(0);
-            const int half = seq.half(i0 + k);
-            if constexpr (LDSP) {
-                // (a half tile past the wave's share: its high bytes came back as zeros, its probabilities count as zeros)
-                const bool on = half < seq.n_halves;
-#pragma unroll
-                for (int u = 0; u < HV; ++u) ring.sb[k][u] = on ? (u32)s_row[half * S::HT + tl + u * S::TPL] : 0u;
-            }
-            // tokens of this half tile below level 2 (one lane per token notes it: the first of its row)
-            bool fine[HV];
-            bool any = false;
-#pragma unroll
-            for (int u = 0; u < HV; ++u) {
-                fine[u] = cl == 0 && v_level(amin, (unsigned short)ring.sb[k][u]) < 2 && ring.sb[k][u] != 0u;
-                any = any || fine[u];
-            }
-            if (__builtin_amdgcn_ballot_w64(any) != 0ull) {
-                const int base = half * S::HT + tl;
-#pragma unroll
-                for (int u = 0; u < HV; ++u) VListed<D>::append(list, count, fine[u], base + u * S::TPL, ring.sb[k][u]);
-            }
-            v_compute_half_coarse<HV>(acc, ring.hi[k], ring.sb[k]);
-            pin_accumulators(acc);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    };
-    if (seq.left() > 0) {
-        round(0);
-        for (int i0 = NR; i0 < seq.left(); i0 += NR) round(i0);
-    }
-}
-
 // The stream with every token multiplied at level 2 (high bytes only) and no look at the fetch levels: for a caller that
 // does not know the row's threshold yet, or has listed the tokens below level 2 some other way (v_stream_list_fine).
 // One half tile in flight while one is multiplied; the probabilities come from LDS (probs_lds: the row's, token-indexed).
@@ -830,17 +767,6 @@ struct VFineScan {
         pos += TPI;
     }
 };
-
-template <int D>
-__device__ __forceinline__ void v_stream_apply_list(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_tokens,
-                                                    unsigned char amin, float *acc, const u32 *list, int count) {
-    const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
-    const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_tokens * (D / 2));
-    const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_tokens * (D / 2));
-    typename VListed<D>::Step first;
-    VListed<D>::request(first, list, count, 0, rH, rM, rL, amin, 0);
-    VListed<D>::apply_all(acc, first, list, count, rH, rM, rL, amin, 0);
-}
 
 // Folds the token lanes of a wave together and adds the 4 waves of the workgroup:
 // out[d] (d < D) = sum over all 256 lanes of their acc for channel d.  wave_part: LDS [4][D].

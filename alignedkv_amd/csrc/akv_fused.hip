@@ -354,7 +354,6 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     __shared__ u32 fine_list[NW][tail_max_tokens / NW];
     const int wave = wave_index();
     const int bh = blockIdx.x;
-    AKV_MARK(bh, 0);
     int R, nrest_unused;
     seq_state(ma.g, bh / ma.g.Hq, R, nrest_unused);
     const int64_t row0 = (int64_t)bh * ma.g.max_seq_len;
@@ -389,7 +388,6 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
         }
         if constexpr (i == 3) v_stream_issue_high<D>(ring.hi[0], rH, first_streamed);
     }, probs_lds, &carry);
-    AKV_MARK(bh, 1);
     float acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
@@ -416,10 +414,8 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
         // (ends with part B's first half tile requested, unless it was the one requested up front)
         v_stream_run_coarse<D>(ring, f8, R, probs_lds, seq_a2, true, seq_b.half(0), acc, [&](int) { tail_once(); });
     }
-    AKV_MARK(bh, 2);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
-    AKV_MARK(bh, 3);
     const unsigned char amin = (unsigned char)ms.amin;
     if (amin_out != nullptr && threadIdx.x == 0) amin_out[bh] = amin;
     const unsigned short *prow = ma.probs + (int64_t)bh * ma.g.row_stride;
@@ -432,7 +428,6 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     scan.probs_lds = probs_lds; scan.amin = amin; scan.a = seq_a; scan.b = seq_b;
     if (!few) scan.b.count = 0;     // (the others are read at their level as they stream)
     typename VListed<D>::Step first;
-    AKV_MARK(bh, 4);
     if (few) {
         // Part B in two stretches: during the first the tokens below level 2 are listed, two steps of 64 tokens per
         // round of the stream; then the first of them are requested, and arrive while the second stretch streams.
@@ -458,24 +453,11 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
         v_stream_run<D, false, 4, 0>(ring4, f8, m4, l4, R, prow, amin, seq_b, acc);
     }
     tail_once();
-    AKV_MARK(bh, 5);
     VListed<D>::apply_all(acc, first, list, count, rH, rM, rL, amin, 0);
-    AKV_MARK(bh, 6);
     if (v_levels_out != nullptr)
         for (int t = threadIdx.x; t < R; t += NT) v_levels_out[(int64_t)bh * R + t] = (uint8_t)v_level(amin, probs_lds[t]);
     v_fold_lanes<D, NW>(acc, wave_part);
     __syncthreads();
-    AKV_MARK(bh, 7);
-    if (threadIdx.x == 0) {
-#ifdef AKV_TRACE
-        if (g_tail_trace != nullptr) {
-            u32 xcc;
-            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-            g_tail_trace[((int64_t)bh * 8) * 24 + 8] = (long long)(xcc & 0xf);
-            g_tail_trace[((int64_t)bh * 8) * 24 + 9] = (long long)count;
-        }
-#endif
-    }
     for (int d = threadIdx.x; d < D; d += NT) {
         float sum = 0.f;
 #pragma unroll
@@ -820,16 +802,13 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
             hipLaunchKernelGGL((tail_step_ref_kernel<D, 4, 3, 512>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
                                reinterpret_cast<unsigned short *>(out), v_levels_out);
         } else {
-            // half tiles per wave that stream before the row's threshold is known: about what the probe's gather takes
-            int fa = 5;
-            { AKV_TUNE("AKV_TUNE_TAIL_FA", v); if (has_v) fa = v; }
-            int pre = 2;
-            { AKV_TUNE("AKV_TUNE_TAIL_PRE", v); if (has_v) pre = v; }
-            fa = max(fa, pre);
-#define AKV_TAIL(P) hipLaunchKernelGGL((tail_step_kernel<D, 512, P>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,   \
-                                       reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out, fa)
-            if (pre <= 0) AKV_TAIL(0); else if (pre == 1) AKV_TAIL(1); else if (pre == 2) AKV_TAIL(2); else AKV_TAIL(3);
-#undef AKV_TAIL
+            // Half tiles per wave that stream before the row's threshold is known (about what the probe's gather takes under
+            // load), the first two of them requested between the phases of the softmax.  Measured at batch 8 x 32 heads x
+            // 4096 tokens, second kernel alone: 27.9 us with 4 and none requested early, 26.9 / 26.0 / 26.2 with one /
+            // two / three requested early (4, 5, 5 before the threshold), 27.1 with three and 6.
+            constexpr int fa = 5;
+            hipLaunchKernelGGL((tail_step_kernel<D, 512, 2>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
+                               reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out, fa);
         }
         mark(2, st);
         mark(3, st);
@@ -891,13 +870,6 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
 }  // namespace akv
 
 using namespace akv;
-
-#ifdef AKV_TRACE
-extern "C" __attribute__((visibility("default"))) int akv_debug_tail_trace_buffer(void *buf) {
-    long long *p = static_cast<long long *>(buf);
-    return hipMemcpyToSymbol(HIP_SYMBOL(g_tail_trace), &p, sizeof(p)) == hipSuccess ? 0 : 1;
-}
-#endif
 
 extern "C" int akv_profile_enable(int enable) {
     if (enable && !g_ev_ready) {

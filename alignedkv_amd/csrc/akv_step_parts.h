@@ -6,18 +6,6 @@
 
 namespace akv {
 
-#ifdef AKV_TRACE
-// development build only: timestamps per (row, wave, mark) of the step's second kernel
-static __device__ long long *g_tail_trace;
-#define AKV_MARK(bh, slot)                                                                                            \
-    do {                                                                                                              \
-        if (g_tail_trace != nullptr && (threadIdx.x & 63) == 0)                                                       \
-            g_tail_trace[((int64_t)(bh) * 8 + (threadIdx.x >> 6)) * 24 + (slot)] = wall_clock64();                    \
-    } while (0)
-#else
-#define AKV_MARK(bh, slot) do {} while (0)
-#endif
-
 // K pass over the 256-token stretch `chunk` of a row of planes with 64-token blocks, by a workgroup of four waves: a wave
 // takes one block and requests all its rows at once (16 KiB in flight for head_dim 128, no loop).  bh_kv / bh: row of
 // the planes (KV head) and of q / the scores (query head).  Scores are stored at device scope.
@@ -176,7 +164,7 @@ struct HookPoint {
 // LDS of the middle stage of one (batch, head) row, NW waves.
 template <int D, int NW>
 struct MiddleShared {
-    float red[NW];
+    float red_max[NW], red_sum[NW];    // the waves' row maxima / sums (each written once per stage)
     unsigned short tail_s[64];     // fp16 scores of the tail (mask not yet added)
     float tail_p[64];              // probabilities of the tail
     u32 cand_key[4 * NW][32];      // [16-lane row of the workgroup][residue class]: best (probability, token) key
@@ -204,10 +192,10 @@ __device__ __forceinline__ void lds_barrier() {
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 }
 
+// red: written once between two uses of the stage (no barrier needed in front of the write)
 template <int NW>
 __device__ __forceinline__ float block_reduce(float v, bool is_max, float *red) {
     v = is_max ? wave_max(v) : wave_sum(v);
-    lds_barrier();
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
     lds_barrier();
     float r = red[0];
@@ -420,7 +408,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
         }
     }
     lds_barrier();
-    AKV_MARK(bh, 10);
     // SPLIT: the stage's loads are all back; from here to the probe it only computes, and memory is the caller's
     auto hook_at = [&](auto point) {
         if constexpr (SPLIT) {
@@ -471,8 +458,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
                 for (int j = 0; j < 8; ++j) m = fmaxf(m, x[v][j]);
             }
         }
-        m = block_reduce<NW>(m, true, ms.red);
-        AKV_MARK(bh, 11);
+        m = block_reduce<NW>(m, true, ms.red_max);
         hook_at(HookPoint<1>());
 #pragma unroll
         for (int v = 0; v < VPT; ++v)
@@ -484,8 +470,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
                 }
             }
         const float et = tid < nrest ? exp_nonpositive(xt - m) : 0.f;
-        sum = block_reduce<NW>(sum + et, false, ms.red);
-        AKV_MARK(bh, 12);
+        sum = block_reduce<NW>(sum + et, false, ms.red_sum);
         hook_at(HookPoint<2>());
         const float rsum = 1.0f / sum;
 #pragma unroll
@@ -506,14 +491,14 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
 #pragma unroll
             for (int j = 0; j < 8; ++j) m = fmaxf(m, x[j]);
         }
-        m = block_reduce<NW>(m, true, ms.red);
+        m = block_reduce<NW>(m, true, ms.red_max);
         for (int i = tid; i < nvec; i += NT) {
             decode_scores8(load_b128_device(rScores, i * 16), mrow, i * 8, x);
 #pragma unroll
             for (int j = 0; j < 8; ++j) sum += exp_nonpositive(x[j] - m);
         }
         const float et = tid < nrest ? exp_nonpositive(xt - m) : 0.f;
-        sum = block_reduce<NW>(sum + et, false, ms.red);
+        sum = block_reduce<NW>(sum + et, false, ms.red_sum);
         const float rsum = 1.0f / sum;
         hook_at(HookPoint<1>());
         hook_at(HookPoint<2>());
@@ -530,7 +515,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
         }
     }
 
-    AKV_MARK(bh, 13);
     hook_at(HookPoint<3>());
     // value rows of the tail: requested here so that they travel while the probe runs
     if (!SPLIT) request_tail_values();
