@@ -99,6 +99,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=10)
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--q-scale", type=float, default=1.0,
+                    help="c2 only: factor on the query (0 or 0.05: flat attention rows, many V tokens below level 2; "
+                         "1: the headline workload)")
     ap.add_argument("--workload", default="c2", choices=["c2", "c3"],
                     help="c2: the headline configuration (shape flags apply); c3: grouped-query heads (32 over 8), batch 32, "
                          "lengths uniform in [2048, 8192] -- an extra line, not the headline metric")
@@ -576,7 +579,7 @@ def main():
         cache.value_cache[layer].save(v, 0, L)
         del k, v
     g = torch.Generator(device="cuda").manual_seed(a.seed + 999)
-    q = torch.randn((B, 1, H, D), device="cuda", generator=g).half()
+    q = (a.q_scale * torch.randn((B, 1, H, D), device="cuda", generator=g)).half()
     k_new = torch.randn((B, 1, H, D), device="cuda", generator=g).half()
     v_new = (0.5 * torch.randn((B, 1, H, D), device="cuda", generator=g)).half()
     out = torch.empty_like(q)
@@ -674,7 +677,8 @@ def main():
         "ms_per_step": round(us / 1e3, 5), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: batch %d, %d heads x %d, cache %d + 1 appended token, K %s, %d layers rotated, K plane blocks of %d tokens"
-                               % ({(8, 32, 128, 4096): "C2", (1, 32, 128, 1024): "C1", (4, 32, 128, 32768): "C4"}.get((B, H, D, L), "other shape"),
+                               % ({(8, 32, 128, 4096): "C2", (1, 32, 128, 1024): "C1", (4, 32, 128, 32768): "C4"}.get((B, H, D, L), "other shape")
+                                  if a.q_scale == 1.0 else "other queries (q x %g)" % a.q_scale,
                                   B, H, D, L, a.k_kind, a.layers, a.k_block)},
         "us_per_step_percentiles": pct,
         "steady_state": {"us_per_step": round(sec_steady * 1e6, 2), "steps": steady_steps,
