@@ -450,17 +450,18 @@ struct VListed {
         fma8_even_odd(acc, st.h.x, st.h.y, 0x80808080u, 0x80808080u, -st.p);
         fma8_even_odd(acc + 8, st.h.z, st.h.w, 0x80808080u, 0x80808080u, -st.p);
     }
-    // the whole list; `first` holds the entries 0 .. TPL - 1, requested by the caller earlier
+    // the list from entry e0 on; `first` holds the entries e0 .. e0 + TPL - 1, requested by the caller earlier
     static __device__ __forceinline__ void apply_all(float *acc, Step &first, const u32 *list, int count,
                                                      const __amdgpu_buffer_rsrc_t rH, const __amdgpu_buffer_rsrc_t rM,
-                                                     const __amdgpu_buffer_rsrc_t rL, unsigned char amin, int tok_base) {
-        if (count <= 0) return;
-        if (count <= TPL) {       // the usual case: nothing more to request (and to wait for)
+                                                     const __amdgpu_buffer_rsrc_t rL, unsigned char amin, int tok_base,
+                                                     int e0 = 0) {
+        if (count <= e0) return;
+        if (count <= e0 + TPL) {       // the usual case: nothing more to request (and to wait for)
             apply(acc, first);
             return;
         }
         Step other;
-        for (int e0 = 0; e0 < count; e0 += 2 * TPL) {
+        for (; e0 < count; e0 += 2 * TPL) {
             request(other, list, count, e0 + TPL, rH, rM, rL, amin, tok_base);
             __builtin_amdgcn_sched_barrier(0);
             apply(acc, first);
@@ -695,14 +696,14 @@ __device__ __forceinline__ int v_stream_count_fine(const unsigned short *s_row, 
 }
 
 // The stream with every token multiplied at level 2 (high bytes only) and no look at the fetch levels: for a caller that
-// does not know the row's threshold yet, or has listed the tokens below level 2 some other way (v_stream_list_fine).
+// does not know the row's threshold yet, or lists the tokens below level 2 some other way (VFineScan).
 // One half tile in flight while one is multiplied; the probabilities come from LDS (probs_lds: the row's, token-indexed).
 // prefetched: the share's first half tile has been requested into ring.hi[0] already (by the caller with
 // v_stream_issue_high, or by the call for the share before this one through next_half).
 // next_half: requested into ring.hi[0] when the share's last half tile is being multiplied (the first half tile of the
 // share the wave takes next, so that the pipeline does not drain between the two calls), or n_halves for none.
-// extra(i0): called once per round of two half tiles, when the round's first request is on its way (work that is to hide
-// behind the stream's memory time).
+// extra(i): called once per half tile, when the request of the next one is on its way (work that is to hide behind the
+// stream's memory time).
 struct NoExtra {
     __device__ __forceinline__ void operator()(int) const {}
 };
@@ -724,10 +725,8 @@ __device__ __forceinline__ void v_stream_run_coarse(VRing<D, RN> &ring, const ui
             const int ahead = (k == 1 && i0 + 2 >= seq.count) ? next_half : seq.half(i0 + k + 1);
             v_stream_issue_high<D>(ring.hi[k ^ 1], rH, ahead);
             __builtin_amdgcn_sched_barrier(0);
-            if (k == 0) {
-                extra(i0);
-                __builtin_amdgcn_sched_barrier(0);
-            }
+            extra(i0 + k);
+            __builtin_amdgcn_sched_barrier(0);
             const int half = seq.half(i0 + k);
             // (a half tile past the wave's share: its high bytes came back as zeros, its probabilities count as zeros)
             const bool on = half < seq.n_halves;
@@ -742,6 +741,53 @@ __device__ __forceinline__ void v_stream_run_coarse(VRing<D, RN> &ring, const ui
     // (the first round stands outside the loop: see v_stream_run)
     round(0);
     for (int i0 = 2; i0 < seq.count; i0 += 2) round(i0);
+}
+
+// The stream with every token read at its own fetch level, for rows where tokens below level 2 are frequent (flat
+// attention).  The levels come from the row's probabilities in LDS (probs_lds, token-indexed) and the threshold, so a half
+// tile's nibble rows are requested together with its high bytes, NR - 1 half tiles before it is multiplied; a row that is
+// not needed is an out-of-range offset and fetches nothing.  extra(i): called once per half tile, between the request
+// of the newest half tile and the multiplication of the oldest.
+template <int D, int NR, typename Extra = NoExtra>
+__device__ __forceinline__ void v_stream_run_levels(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_tokens,
+                                                   const unsigned short *probs_lds, unsigned char amin, const VSeq &seq,
+                                                   float *acc, Extra extra = Extra()) {
+    using S = VStream<D>;
+    constexpr int HV = S::HV;
+    static_assert(NR >= 2, "one half tile is multiplied while the others travel");
+    if (seq.count <= 0) return;
+    const int lane = threadIdx.x & 63, tl = lane / S::LPR;
+    const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)n_tokens * D);
+    const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)n_tokens * (D / 2));
+    const __amdgpu_buffer_rsrc_t rL = make_rsrc(l4, (u32)n_tokens * (D / 2));
+    VHalfTile<HV> t[NR];
+    u32 sb[NR][HV];
+    auto issue = [&](VHalfTile<HV> &x, u32 *p, int half) {
+        // (a half tile past the wave's share: probabilities of zero, level 2, nothing fetched)
+        const bool on = half < seq.n_halves;
+#pragma unroll
+        for (int u = 0; u < HV; ++u) p[u] = on ? (u32)probs_lds[half * S::HT + tl + u * S::TPL] : 0u;
+        v_stream_issue_high<D>(x, rH, half);
+        v_issue_half_ml<D, false, HV>(x, rM, rL, half * S::HT, n_tokens, p, amin);
+    };
+#pragma unroll
+    for (int k = 0; k < NR - 1; ++k) issue(t[k], sb[k], seq.half(k));
+    __builtin_amdgcn_sched_barrier(0);
+    auto round = [&](int i0) {
+#pragma unroll
+        for (int k = 0; k < NR; ++k) {
+            issue(t[(k + NR - 1) % NR], sb[(k + NR - 1) % NR], seq.half(i0 + k + NR - 1));
+            __builtin_amdgcn_sched_barrier(0);
+            extra(i0 + k);
+            __builtin_amdgcn_sched_barrier(0);
+            v_compute_half<HV>(acc, t[k], sb[k]);
+            pin_accumulators(acc);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // (the first round stands outside the loop: see v_stream_run)
+    round(0);
+    for (int i0 = NR; i0 < seq.count; i0 += NR) round(i0);
 }
 
 // Lists the tokens below level 2 of a wave's shares a and b (in that order) from the row's probabilities in LDS, 64 tokens

@@ -418,7 +418,6 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     __syncthreads();
     const unsigned char amin = (unsigned char)ms.amin;
     if (amin_out != nullptr && threadIdx.x == 0) amin_out[bh] = amin;
-    const unsigned short *prow = ma.probs + (int64_t)bh * ma.g.row_stride;
     const __amdgpu_buffer_rsrc_t rM = make_rsrc(m4, (u32)R * (D / 2)), rL = make_rsrc(l4, (u32)R * (D / 2));
     u32 *list = fine_list[wave];
     int count = 0;
@@ -428,9 +427,10 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     scan.probs_lds = probs_lds; scan.amin = amin; scan.a = seq_a; scan.b = seq_b;
     if (!few) scan.b.count = 0;     // (the others are read at their level as they stream)
     typename VListed<D>::Step first;
+    int listed_from = 0;      // `first` holds the list's entries from here on
     if (few) {
-        // Part B in two stretches: during the first the tokens below level 2 are listed, two steps of 64 tokens per
-        // round of the stream; then the first of them are requested, and arrive while the second stretch streams.
+        // Part B in two stretches: during the first the tokens below level 2 are listed, 64 tokens per half tile of the
+        // stream; then they are requested, and arrive while the second stretch streams.
         const int n_b1 = min(seq_b.count, 2 * ((scan.steps_left() + 1) / 2));
         VSeq b1 = seq_b, b2 = seq_b;
         b1.count = n_b1;
@@ -438,22 +438,25 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
         v_stream_run_coarse<D>(ring, f8, R, probs_lds, b1, true, b2.half(0), acc, [&](int) {
             tail_once();
             if (!scan.done()) scan.step(list, count);
-            if (!scan.done()) scan.step(list, count);
         });
         while (!scan.done()) scan.step(list, count);
         VListed<D>::request(first, list, count, 0, rH, rM, rL, amin, 0);
         __builtin_amdgcn_sched_barrier(0);
         v_stream_run_coarse<D>(ring, f8, R, probs_lds, b2, true, n_halves, acc);
     } else {
+        // Frequent tokens below level 2 (flat attention): the rest of the row streams at the tokens' own levels, and the
+        // corrections of what part A multiplied at level 2 ride along, one batch of listed rows per half tile.
         while (!scan.done()) scan.step(list, count);
         VListed<D>::request(first, list, count, 0, rH, rM, rL, amin, 0);
         __builtin_amdgcn_sched_barrier(0);
-        // (the share's first half tile, requested early, is asked for again: the rare path)
-        VRing<D, 4> ring4;
-        v_stream_run<D, false, 4, 0>(ring4, f8, m4, l4, R, prow, amin, seq_b, acc);
+        v_stream_run_levels<D, 2>(f8, m4, l4, R, probs_lds, amin, seq_b, acc, [&](int) {
+            VListed<D>::apply(acc, first);
+            listed_from += VListed<D>::TPL;
+            VListed<D>::request(first, list, count, listed_from, rH, rM, rL, amin, 0);
+        });
     }
     tail_once();
-    VListed<D>::apply_all(acc, first, list, count, rH, rM, rL, amin, 0);
+    VListed<D>::apply_all(acc, first, list, count, rH, rM, rL, amin, 0, listed_from);
     if (v_levels_out != nullptr)
         for (int t = threadIdx.x; t < R; t += NT) v_levels_out[(int64_t)bh * R + t] = (uint8_t)v_level(amin, probs_lds[t]);
     v_fold_lanes<D, NW>(acc, wave_part);
@@ -778,14 +781,14 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     // Second half of the step in one launch (see tail_step_kernel)
     // It is used when the (batch, head) pairs spread evenly over the compute units (every unit gets the same one or
     // two rows) and the rows are not long: measured on MI355X with 32 heads x 128, against the three launches it
-    // replaces: 43.2 vs 46.3 us per step at batch 8 x 2048 tokens, 69.2 vs 74.7 at 8 x 4096, 99.4 vs 105.0 at 8 x 6144,
-    // 134.1 vs 133.0 at 8 x 8192, 130.4 vs 133.2 at 16 x 4096, 184.3 vs 188.4 at 16 x 6144, but 250.7 vs 241.5 at
-    // 16 x 8192 (two long rows per unit: one workgroup per row streams at 4.5 TB/s, the V pass of many small workgroups
-    // at 6): up to 12288 tokens per compute unit.
+    // replaces, us per step: 61.9 vs 72 at batch 8 x 4096 tokens, 76.4 vs 84.2 at 8 x 5120, 89.5 vs 96.9 at 8 x 6144,
+    // 104.9 vs 110.6 at 8 x 7168, 125.9 vs 128.6 at 8 x 8192, 116.4 vs 127.7 at 16 x 4096, 143.9 vs 152.9 at 16 x 5120,
+    // 169.8 vs 180.9 at 16 x 6144; with two rows of 8192 tokens per unit the V pass of many small workgroups was ahead
+    // (241.5 vs 250.7 with an earlier form of the kernel), hence up to 12288 tokens per compute unit.
     // With fewer rows than compute units a row's workgroup streams alone at about 45 GB/s, while the V pass of many
     // small workgroups needs 4 us or the time of its bytes at 5 TB/s and then two more launches (2.5 us): measured
-    // with 32 heads x 128 at batch 1 x 1024 tokens 21.7 vs 23.9 us per step, 2 x 2048: 25.5 vs 26.3, 4 x 4096: 43.7
-    // vs 45.6, but 1 x 4096: 30.3 vs 27.0.
+    // with 32 heads x 128 at batch 1 x 1024 tokens 15.9 vs 20.1 us per step, 2 x 2048: 21.0 vs 26.3, 4 x 4096: 39.2
+    // vs 45.6, but 1 x 4096: 30.3 vs 23.8.
     const int cus = compute_units();
     const int rows = B * Hq;
     bool tail = cus > 0 && rows % cus == 0 && rows / cus <= tail_rows_per_cu && (rows / cus) * R <= 12288;
@@ -804,8 +807,8 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         } else {
             // Half tiles per wave that stream before the row's threshold is known (about what the probe's gather takes under
             // load), the first two of them requested between the phases of the softmax.  Measured at batch 8 x 32 heads x
-            // 4096 tokens, second kernel alone: 27.9 us with 4 and none requested early, 26.9 / 26.0 / 26.2 with one /
-            // two / three requested early (4, 5, 5 before the threshold), 27.1 with three and 6.
+            // 4096 tokens, second kernel alone by events: 27.4 us with 4 and none requested early, 25.7 with 4 and two
+            // early, 25.5 with 5 and two, 25.8 with 5 and three.
             constexpr int fa = 5;
             hipLaunchKernelGGL((tail_step_kernel<D, 512, 2>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
                                reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out, fa);
