@@ -102,6 +102,8 @@ def parse():
     ap.add_argument("--q-scale", type=float, default=1.0,
                     help="c2 only: factor on the query (0 or 0.05: flat attention rows, many V tokens below level 2; "
                          "1: the headline workload)")
+    ap.add_argument("--extra-capacity", type=int, default=0,
+                    help="c2 only: tokens of cache capacity beyond cache-len + 64 (changes the pitch of the plane rows)")
     ap.add_argument("--workload", default="c2", choices=["c2", "c3"],
                     help="c2: the headline configuration (shape flags apply); c3: grouped-query heads (32 over 8), batch 32, "
                          "lengths uniform in [2048, 8192] -- an extra line, not the headline metric")
@@ -571,8 +573,8 @@ def main():
         a.k_block = 64      # the 256-token layout is built for head_dim 64 and 128
     assert L % 64 == 0, "the cache length of the benchmark must be a multiple of the 64-token flush block"
     cfg = SimpleNamespace(num_hidden_layers=a.layers, num_attention_heads=H, num_key_value_heads=H, hidden_size=H * D,
-                          max_position_embeddings=L + 64)
-    cache = QuantizedCache_AlignedKV(cfg, B, L + 64, "cuda", torch.half, k_block=a.k_block)
+                          max_position_embeddings=L + 64 + a.extra_capacity)
+    cache = QuantizedCache_AlignedKV(cfg, B, L + 64 + a.extra_capacity, "cuda", torch.half, k_block=a.k_block)
     for layer in range(a.layers):
         k, v = make_layer_inputs(torch, B, L, H, D, a.seed + layer, a.k_kind)
         cache.key_cache[layer].save(k, 0, L)
@@ -647,7 +649,7 @@ def main():
     other = None
     if D <= 128:      # (head_dim 256 has the 64-token layout only)
         other_kb = 64 if a.k_block == 256 else 256
-        cache2 = QuantizedCache_AlignedKV(cfg, B, L + 64, "cuda", torch.half, k_block=other_kb)
+        cache2 = QuantizedCache_AlignedKV(cfg, B, L + 64 + a.extra_capacity, "cuda", torch.half, k_block=other_kb)
         for layer in range(a.layers):
             k, v = make_layer_inputs(torch, B, L, H, D, a.seed + layer, a.k_kind)
             cache2.key_cache[layer].save(k, 0, L)
