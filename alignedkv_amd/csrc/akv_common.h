@@ -166,9 +166,6 @@ __device__ __forceinline__ void store_u16_device(const __amdgpu_buffer_rsrc_t r,
 __device__ __forceinline__ void store_f32_device(const __amdgpu_buffer_rsrc_t r, int byte_off, float v) {
     __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, byte_off, 0, kDeviceScope);
 }
-__device__ __forceinline__ float load_f32_device(const __amdgpu_buffer_rsrc_t r, int byte_off) {
-    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, byte_off, 0, kDeviceScope));
-}
 __device__ __forceinline__ u32x4 load_b128_device(const __amdgpu_buffer_rsrc_t r, int byte_off) {
     return __builtin_amdgcn_raw_buffer_load_b128(r, byte_off, 0, kDeviceScope);
 }

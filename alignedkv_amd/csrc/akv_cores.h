@@ -345,14 +345,6 @@ __device__ __forceinline__ void v_issue_half_ml(VLowPart<HV> &t, const __amdgpu_
     }
 }
 
-template <int D, bool REF, int HV>
-__device__ __forceinline__ void v_issue_half(VHalfTile<HV> &t, const __amdgpu_buffer_rsrc_t rH,
-                                             const __amdgpu_buffer_rsrc_t rM, const __amdgpu_buffer_rsrc_t rL, int base,
-                                             int t_end, const u32 *sb, unsigned char amin) {
-    v_issue_half_h<D, HV>(t, rH, base, t_end);
-    v_issue_half_ml<D, REF, HV>(t, rM, rL, base, t_end, sb, amin);
-}
-
 template <int D>
 struct VFirstTile {
     VHalfTile<(D / 16 < 8 ? D / 16 : 8) / 2> t;
