@@ -201,6 +201,18 @@ __device__ __forceinline__ float wave_sum(float v) {
     v += dpp_f32<kDppMirror>(v);
     return rows_to_wave_f32(v, false);
 }
+// Sum over groups of N consecutive lanes (N = 2, 4, 8 or 16, aligned): every lane of a group ends up with the group's
+// sum, added in the order of a butterfly over lane distances 1, 2, 4, 8 (the mirrors pair the same partial sums as
+// those distances do).
+template <int N>
+__device__ __forceinline__ float lane_group_sum(float v) {
+    static_assert(N == 1 || N == 2 || N == 4 || N == 8 || N == 16, "a group lies inside a 16-lane row");
+    if constexpr (N >= 2) v += dpp_f32<kDppXor1>(v);
+    if constexpr (N >= 4) v += dpp_f32<kDppXor2>(v);
+    if constexpr (N >= 8) v += dpp_f32<kDppHalfMirror>(v);
+    if constexpr (N >= 16) v += dpp_f32<kDppMirror>(v);
+    return v;
+}
 __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, dpp_f32<kDppXor1>(v));
     v = fmaxf(v, dpp_f32<kDppXor2>(v));
@@ -215,6 +227,17 @@ __device__ __forceinline__ u32 wave_min_u32(u32 v) {
     v = min(v, dpp_u32<kDppMirror>(v));
     return min(min((u32)__builtin_amdgcn_readlane((int)v, 0), (u32)__builtin_amdgcn_readlane((int)v, 16)),
                min((u32)__builtin_amdgcn_readlane((int)v, 32), (u32)__builtin_amdgcn_readlane((int)v, 48)));
+}
+// Maximum over the wave of a value that every lane of a 16-lane row holds alike: four lane reads, a scalar result.
+__device__ __forceinline__ u32 rows_max_u32(u32 v) {
+    return max(max((u32)__builtin_amdgcn_readlane((int)v, 0), (u32)__builtin_amdgcn_readlane((int)v, 16)),
+               max((u32)__builtin_amdgcn_readlane((int)v, 32), (u32)__builtin_amdgcn_readlane((int)v, 48)));
+}
+// Maximum over the wave of a value that the lanes 4k .. 4k + 3 hold alike: two row rotations, then the rows.
+__device__ __forceinline__ u32 quads_max_u32(u32 v) {
+    v = max(v, (u32)__builtin_amdgcn_update_dpp(0, (int)v, 0x124, 0xf, 0xf, false));   // row_ror:4
+    v = max(v, (u32)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xf, 0xf, false));   // row_ror:8
+    return rows_max_u32(v);
 }
 __device__ __forceinline__ int wave_sum_i32(int v) {
     v += (int)dpp_u32<kDppXor1>((u32)v);

@@ -8,18 +8,8 @@
 
 namespace akv {
 
-__device__ __forceinline__ float d_wave_sum(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
-    return v;
-}
-__device__ __forceinline__ float d_wave_max(float v) {
-#pragma unroll
-    for (int m = 32; m >= 1; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, 64));
-    return v;
-}
 __device__ __forceinline__ float d_block_reduce(float v, bool is_max, float *red) {
-    v = is_max ? d_wave_max(v) : d_wave_sum(v);
+    v = is_max ? wave_max(v) : wave_sum(v);
     __syncthreads();
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
     __syncthreads();
@@ -129,7 +119,7 @@ __global__ __launch_bounds__(256) void dense_middle_kernel(DenseMiddleArgs a) {
     if (wave == 0) {
         float part = 0.f;
         for (int c = lane; c < D; c += 64) part = fmaf(half_bits_to_float(knew[c]), half_bits_to_float(qrow[c]), part);
-        part = d_wave_sum(part);
+        part = wave_sum(part);
         if (lane == 0) {
             const unsigned short sc = float_to_half_bits(half_bits_to_float(float_to_half_bits(part)) / sqrtf((float)D));
             srow[n] = sc;

@@ -280,8 +280,7 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
         esum[g] = w >> 16;
         mx = max(mx, esum[g]);
     }
-#pragma unroll
-    for (int m = 4; m <= 32; m <<= 1) mx = max(mx, (u32)__shfl_xor((int)mx, m, 64));
+    mx = quads_max_u32(mx);
     u32 need_mid = 0, need_last = 0;
 #pragma unroll
     for (int g = 0; g < NG; ++g) {

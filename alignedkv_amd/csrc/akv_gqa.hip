@@ -85,8 +85,7 @@ __global__ __launch_bounds__(256) void group_k_pass_kernel(
             esum[g] = (exp_field(qb) + cmax[g]) & 0xffu;
             mx = max(mx, esum[g]);
         }
-#pragma unroll
-        for (int m = 4; m <= 32; m <<= 1) mx = max(mx, (u32)__shfl_xor((int)mx, m, 64));
+        mx = quads_max_u32(mx);
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
             const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)esum[g]);

@@ -45,8 +45,7 @@ __device__ __forceinline__ void k_pass64_whole_blocks(
         esum[g] = w >> 16;
         mx = max(mx, esum[g]);
     }
-#pragma unroll
-    for (int m = 4; m <= 32; m <<= 1) mx = max(mx, (u32)__shfl_xor((int)mx, m, 64));
+    mx = quads_max_u32(mx);
     u32 need_mid = 0, need_last = 0;
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
@@ -100,8 +99,7 @@ __device__ __forceinline__ void k_pass256_split_block(
     u32 mx = 0;
 #pragma unroll
     for (int g = 0; g < NG; ++g) mx = max(mx, staged[4 * g + (lane >> 4)] >> 16);
-    mx = max(mx, (u32)__shfl_xor((int)mx, 16, 64));
-    mx = max(mx, (u32)__shfl_xor((int)mx, 32, 64));
+    mx = rows_max_u32(mx);
     float qf[GW];
     u32 need_mid = 0, need_last = 0;   // bit g: of the wave's group g
 #pragma unroll
@@ -398,8 +396,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
                 part = fmaf(hi_half_to_float(kk[c]), hi_half_to_float(qq[c]), part);
             }
         }
-#pragma unroll
-        for (int mk = 1; mk < LPT; mk <<= 1) part += __shfl_xor(part, mk, 64);
+        part = lane_group_sum<LPT>(part);
         if (tr < nrest && tj == 0) {
             const float dot16 = half_bits_to_float(float_to_half_bits(part));
             const unsigned short sc = float_to_half_bits(dot16 / sqrt_d);
