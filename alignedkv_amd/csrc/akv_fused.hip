@@ -337,7 +337,7 @@ constexpr int tail_rows_per_cu = 2, tail_max_tokens = 8192;
 // A wave whose tokens are below level 2 more often than one in 16 (flat attention) lists only the ones it has
 // multiplied already and takes the nibble rows of the others along with their half tiles (v_stream_run).
 // grid (B*H), NT threads.
-template <int D, int NT, int PRE>
+template <int D, int NT, int PRE, bool MASKED>
 __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict__ v_first_8,
                                                         const uint8_t *__restrict__ v_mid_4,
                                                         const uint8_t *__restrict__ v_last_4, MiddleArgs ma,
@@ -354,7 +354,7 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     const int wave = wave_index();
     const int bh = blockIdx.x;
     int R, nrest_unused;
-    seq_state(ma.g, bh / ma.g.Hq, R, nrest_unused);
+    seq_state<true>(ma.g, 0, R, nrest_unused);
     const int64_t row0 = (int64_t)bh * ma.g.max_seq_len;
     const uint8_t *f8 = v_first_8 + row0 * D, *m4 = v_mid_4 + row0 * (D / 2), *l4 = v_last_4 + row0 * (D / 2);
     const __amdgpu_buffer_rsrc_t rH = make_rsrc(f8, (u32)R * D);
@@ -380,13 +380,14 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     const int first_streamed = wave == 0 ? seq_b.half(0) : (seq_a2.count > 0 ? seq_a2.half(0) : seq_b.half(0));
     MiddleCarry<D, NT> carry;
     static_assert(PRE <= 3, "one half tile per phase of the middle stage");
-    middle_body<D, NT, true>(ma, bh, ms, [&](auto point) {
+    auto between_phases = [&](auto point) {
         constexpr int i = decltype(point)::value;
         if constexpr (i < PRE) {
             if (wave != 0) v_stream_issue_high<D>(pre[i], rH, seq_a.half(i));
         }
         if constexpr (i == 3) v_stream_issue_high<D>(ring.hi[0], rH, first_streamed);
-    }, probs_lds, &carry);
+    };
+    middle_body<D, NT, true, decltype(between_phases), MASKED ? 1 : 0, tail_max_tokens>(ma, bh, ms, between_phases, probs_lds, &carry);
     float acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
@@ -809,8 +810,12 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
             // 4096 tokens, second kernel alone by events: 27.4 us with 4 and none requested early, 25.7 with 4 and two
             // early, 25.5 with 5 and two, 25.8 with 5 and three.
             constexpr int fa = 5;
-            hipLaunchKernelGGL((tail_step_kernel<D, 512, 2>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
-                               reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out, fa);
+            if (ma.mask != nullptr)
+                hipLaunchKernelGGL((tail_step_kernel<D, 512, 2, true>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
+                                   reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out, fa);
+            else
+                hipLaunchKernelGGL((tail_step_kernel<D, 512, 2, false>), dim3(B * Hq), dim3(512), 0, st, vf8, vm4, vl4, ma,
+                                   reinterpret_cast<unsigned short *>(out), v_levels_out, amin_out, fa);
         }
         mark(2, st);
         mark(3, st);

@@ -27,11 +27,15 @@ constexpr u32 kNoTask = 0xffffffffu;
 __host__ __device__ inline u32 pack_task(int x, int y, int z) { return (u32)x | ((u32)y << 12) | ((u32)z << 20); }
 inline bool task_map_fits(const PassShape &s, int B) { return s.grid_x <= 4096 && s.grid_y <= 256 && B <= 4096; }
 
-// tokens flushed into the planes / held in the rest buffer once this step's token has been appended
+// tokens flushed into the planes / held in the rest buffer once this step's token has been appended.  The fused step
+// flushes 64 tokens at a time (g.cb == 64, checked by the entry points).  UNIFORM: the caller knows that there are no
+// per-sequence lengths (no pointer test and no dependent load in front of a one-shot kernel's first requests).
+constexpr int kFlush = 64;
+template <bool UNIFORM = false>
 __device__ __forceinline__ void seq_state(const StepGeom &g, int b, int &R, int &nrest) {
-    const int L = (g.seq_lens != nullptr ? g.seq_lens[b] : g.cur_len) + 1;
-    R = (L / g.cb) * g.cb;
-    nrest = L - R;
+    const int L = ((!UNIFORM && g.seq_lens != nullptr) ? g.seq_lens[b] : g.cur_len) + 1;
+    R = L & ~(kFlush - 1);
+    nrest = L & (kFlush - 1);
 }
 
 // Workgroup -> (chunk x, head index y, batch z) of a launch with grid (chunks, heads, batch); false: nothing to do.

@@ -278,10 +278,14 @@ __device__ __forceinline__ void middle_tail_partials(MiddleShared<D, NT / 64> &m
 // column maxima (ms.vcm) and the tail's probabilities (ms.tail_p), ending with an LDS barrier; the caller lets one wave
 // run middle_probe_wave (probe and threshold, no barrier inside) while the others go on, and calls
 // middle_tail_partials with `carry` when it suits it (every wave, before the workgroup adds up ms.tail_o).
-template <int D, int NT, bool SPLIT = false, typename Hook = NoHook>
+// MASKED: 1 / 0 = the caller knows that there is / is no mask row (the other case is not compiled), -1 = looked up at
+// run time.  MAXTOK: an upper bound of the flushed tokens per row that the caller guarantees (0: none; rows beyond
+// what the registers hold take three passes over the scores): both keep a one-shot kernel's code short.
+template <int D, int NT, bool SPLIT = false, typename Hook = NoHook, int MASKED = -1, int MAXTOK = 0>
 __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, MiddleShared<D, NT / 64> &ms, Hook hook = Hook(),
                                             unsigned short *probs_lds = nullptr, MiddleCarry<D, NT> *carry_out = nullptr) {
-    constexpr int VPT = 4;                    // 16-byte score vectors a thread keeps in registers
+    // 16-byte score vectors a thread keeps in registers
+    constexpr int VPT = MAXTOK > 0 ? (MAXTOK / 8 + NT - 1) / NT : 4;
     constexpr int NW = NT / 64;               // waves
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // bh indexes (batch, query head); the keys, values, column maxima and rest buffers belong to its KV head
@@ -290,16 +294,16 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
     const int Hkv = a.g.Hkv, cb = a.g.cb;
     const bool owner = hq % a.g.G == 0;       // one query head of the group writes the shared state
     int R, nrest;
-    seq_state(a.g, b, R, nrest);
+    seq_state<SPLIT>(a.g, b, R, nrest);      // (SPLIT: the one-launch second half of the step, uniform lengths only)
     const int newest = nrest - 1;
     const unsigned short *qrow = a.q + (int64_t)bh * D;
     const unsigned short *knew = a.k_new + (int64_t)bh_kv * D;
     const unsigned short *vnew = a.v_new + (int64_t)bh_kv * D;
     unsigned short *srow = a.scores + (int64_t)bh * a.g.row_stride;
     unsigned short *prow = a.probs + (int64_t)bh * a.g.row_stride;
-    const unsigned short *mrow = a.mask ? a.mask + (int64_t)b * a.mask_stride : nullptr;
+    const unsigned short *mrow = MASKED == 0 ? nullptr : ((MASKED == 1 || a.mask) ? a.mask + (int64_t)b * a.mask_stride : nullptr);
     const int nvec = R >> 3;
-    const bool in_regs = nvec <= NT * VPT;
+    const bool in_regs = MAXTOK > 0 || nvec <= NT * VPT;
     // scores of the flushed part are read at device scope: other workgroups of the same launch wrote them
     const __amdgpu_buffer_rsrc_t rScores = make_rsrc(srow, (u32)R * 2);
     auto store_probs8 = [&](int i, const u32x4 o) {
@@ -327,45 +331,25 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
     constexpr int NKV = (D / 8 + LPT - 1) / LPT;
     const int tr = tid / LPT, tj = tid % LPT;
     u32x4 tkw[NKV], tqw[NKV];
+    // All of these are buffer loads whose offset is out of range where a lane has nothing to fetch (zeros come back):
+    // no load sits under a branch, so the compiler issues them back to back and the stage starts with one round trip.
+    // Rest buffers of this (batch, KV head): row r at r * Hkv * D; the newest token comes from k_new / v_new while
+    // this kernel is the one that appends it.
+    const u32 rest_bytes = (u32)(((cb - 1) * Hkv + 1) * D * 2);
+    const __amdgpu_buffer_rsrc_t rRK = make_rsrc(a.restk + ((int64_t)b * cb * Hkv + h) * D, rest_bytes);
+    const __amdgpu_buffer_rsrc_t rRV = make_rsrc(a.restv + ((int64_t)b * cb * Hkv + h) * D, rest_bytes);
+    const __amdgpu_buffer_rsrc_t rQ = make_rsrc(qrow, D * 2), rKN = make_rsrc(knew, D * 2), rVN = make_rsrc(vnew, D * 2);
+    const bool fresh = a.persist != 0;
     {
-        const unsigned short *krow = (tr == newest && a.persist) ? knew : a.restk + (((int64_t)b * cb + tr) * Hkv + h) * D;
 #pragma unroll
         for (int i = 0; i < NKV; ++i) {
             const int v8 = tj + i * LPT;
-            const bool on = tr < nrest && v8 < D / 8;
-            tkw[i] = on ? *reinterpret_cast<const u32x4 *>(krow + v8 * 8) : (u32x4){0u, 0u, 0u, 0u};
-            tqw[i] = on ? *reinterpret_cast<const u32x4 *>(qrow + v8 * 8) : (u32x4){0u, 0u, 0u, 0u};
+            const bool on = tr < nrest && v8 < D / 8, is_new = fresh && tr == newest;
+            const u32x4 kr = __builtin_amdgcn_raw_buffer_load_b128(rRK, (on && !is_new) ? (tr * Hkv * D + v8 * 8) * 2 : kSkip, 0, 0);
+            const u32x4 kn = __builtin_amdgcn_raw_buffer_load_b128(rKN, (on && is_new) ? v8 * 16 : kSkip, 0, 0);
+            tkw[i] = kr | kn;
+            tqw[i] = __builtin_amdgcn_raw_buffer_load_b128(rQ, on ? v8 * 16 : kSkip, 0, 0);
         }
-    }
-    // (a) append the token: rest buffers and column maxima (extension/k_cache_file.py:98-101).
-    //     vcm_mine: this thread's channel of the V column maxima after the update (threads < D).
-    static_assert(D <= NT, "one channel per thread");
-    u32 vcm_mine = 0;
-    {
-        const bool on = tid < D;
-        const int d = on ? tid : 0;
-        u32 kc = a.kcm[(int64_t)bh_kv * D + d], vc = a.vcm[(int64_t)bh_kv * D + d];
-        const u32 kb = knew[d], vb = vnew[d];
-        if constexpr (!SPLIT) {
-            __builtin_amdgcn_sched_barrier(0);
-            hook(HookPoint<0>());
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        if (a.persist) {
-            // every query head of the group derives the updated maxima itself (max is idempotent, so it does
-            // not matter whether it reads them before or after the owner's store); only the owner stores
-            kc = max(kc, exp_field(kb));
-            vc = max(vc, exp_field(vb));
-            if (owner && on) {
-                const int64_t at = (((int64_t)b * cb + newest) * Hkv + h) * D + d;
-                a.restk[at] = (unsigned short)kb;
-                a.restv[at] = (unsigned short)vb;
-                a.kcm[(int64_t)bh_kv * D + d] = (uint8_t)kc;
-                a.vcm[(int64_t)bh_kv * D + d] = (uint8_t)vc;
-            }
-        }
-        vcm_mine = vc;
-        if (SPLIT && on) ms.vcm[d] = vc;
     }
     // value rows of the tail, used by (f): a thread takes 8 channels of every NRG-th tail token
     using Carry = MiddleCarry<D, NT>;
@@ -376,12 +360,46 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
 #pragma unroll
         for (int k = 0; k < Carry::MAXR; ++k) {
             const int r = rg + k * Carry::NRG;
-            const unsigned short *vrow = (r == newest && a.persist) ? vnew : a.restv + (((int64_t)b * cb + r) * Hkv + h) * D;
-            carry.tvw[k] = r < nrest ? *reinterpret_cast<const u32x4 *>(vrow + c8 * 8) : (u32x4){0u, 0u, 0u, 0u};
+            const bool on = r < nrest, is_new = fresh && r == newest;
+            const u32x4 vr = __builtin_amdgcn_raw_buffer_load_b128(rRV, (on && !is_new) ? (r * Hkv * D + c8 * 8) * 2 : kSkip, 0, 0);
+            const u32x4 vn = __builtin_amdgcn_raw_buffer_load_b128(rVN, (on && is_new) ? c8 * 16 : kSkip, 0, 0);
+            carry.tvw[k] = vr | vn;
         }
     };
     // (SPLIT: with the first loads, so that nothing the stage needs later queues behind the caller's stream)
     if (SPLIT) request_tail_values();
+    // (a) append the token: rest buffers and column maxima (extension/k_cache_file.py:98-101).
+    //     vcm_mine: this thread's channel of the V column maxima after the update (threads < D).
+    static_assert(D <= NT, "one channel per thread");
+    const bool ch_on = tid < D;               // this thread looks after channel tid of the column maxima
+    const int ch = ch_on ? tid : 0;
+    u32 kc = (u32)(unsigned char)__builtin_amdgcn_raw_buffer_load_b8(make_rsrc(a.kcm + (int64_t)bh_kv * D, D), ch_on ? ch : kSkip, 0, 0);
+    u32 vc = (u32)(unsigned char)__builtin_amdgcn_raw_buffer_load_b8(make_rsrc(a.vcm + (int64_t)bh_kv * D, D), ch_on ? ch : kSkip, 0, 0);
+    const u32 kb = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rKN, ch_on ? ch * 2 : kSkip, 0, 0);
+    const u32 vb = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rVN, ch_on ? ch * 2 : kSkip, 0, 0);
+    if constexpr (!SPLIT) {
+        __builtin_amdgcn_sched_barrier(0);
+        hook(HookPoint<0>());
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // Every query head of the group derives the updated maxima itself (max is idempotent, so it does not matter
+    // whether it reads them before or after the owner's store, nor whether an earlier kernel of the step has
+    // appended the token already).
+    kc = max(kc, exp_field(kb));
+    vc = max(vc, exp_field(vb));
+    const u32 vcm_mine = vc;
+    if (SPLIT && ch_on) ms.vcm[ch] = vc;
+    // The stores of the append wait until the tail's scores are out (below): nothing in this kernel reads them back,
+    // and the two waves that issue them would otherwise reach the stage's first barrier a round trip late.
+    auto store_append = [&]() {
+        if (a.persist && owner && ch_on) {
+            const int64_t at = (((int64_t)b * cb + newest) * Hkv + h) * D + ch;
+            a.restk[at] = (unsigned short)kb;
+            a.restv[at] = (unsigned short)vb;
+            a.kcm[(int64_t)bh_kv * D + ch] = (uint8_t)kc;
+            a.vcm[(int64_t)bh_kv * D + ch] = (uint8_t)vc;
+        }
+    };
     // (b) scores of the tail: fp16(fp16(q.k) / sqrt(D)), the two roundings of an fp16 matmul followed by
     //     an fp16 division (extension/k_cache_file.py:156)
     const float sqrt_d = sqrtf((float)D);
@@ -405,6 +423,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
         }
     }
     lds_barrier();
+    store_append();
     // SPLIT: the stage's loads are all back; from here to the probe it only computes, and memory is the caller's
     auto hook_at = [&](auto point) {
         if constexpr (SPLIT) {

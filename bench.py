@@ -672,7 +672,7 @@ def main():
         k_kernel = "akv::fused_k_pass_kernel<%d, false, true>" % D if D <= 128 else "akv::fused_k_pass_kernel<%d, false, false>" % D
     else:
         k_kernel = "akv::fused_k_pass256_split_kernel<%d, false, 4>" % D
-    tail_kernel = "akv::tail_step_kernel<%d, 512, 2>" % D
+    tail_kernel = "akv::tail_step_kernel<%d, 512, 2, false>" % D
     res = {
         "metric": "decode-attn us/step (+ effective HBM GB/s, %% of peak), B=%d L=%d %dx%d" % (B, L, H, D),
         "value": round(us, 2), "unit": "us/step", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
