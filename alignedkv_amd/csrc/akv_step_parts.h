@@ -389,17 +389,16 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
     vc = max(vc, exp_field(vb));
     const u32 vcm_mine = vc;
     if (SPLIT && ch_on) ms.vcm[ch] = vc;
-    // The stores of the append wait until the tail's scores are out (below): nothing in this kernel reads them back,
-    // and the two waves that issue them would otherwise reach the stage's first barrier a round trip late.
-    auto store_append = [&]() {
-        if (a.persist && owner && ch_on) {
-            const int64_t at = (((int64_t)b * cb + newest) * Hkv + h) * D + ch;
-            a.restk[at] = (unsigned short)kb;
-            a.restv[at] = (unsigned short)vb;
-            a.kcm[(int64_t)bh_kv * D + ch] = (uint8_t)kc;
-            a.vcm[(int64_t)bh_kv * D + ch] = (uint8_t)vc;
-        }
-    };
+    // The stores of the append: issued here, where the wave waits for its first loads anyway, and in front of the
+    // tail's score store -- a wait for a loaded value placed behind a store would also wait for that store to be
+    // acknowledged (one counter covers both), a round trip in front of the stage's first barrier.
+    if (a.persist && owner && ch_on) {
+        const int64_t at = (((int64_t)b * cb + newest) * Hkv + h) * D + ch;
+        a.restk[at] = (unsigned short)kb;
+        a.restv[at] = (unsigned short)vb;
+        a.kcm[(int64_t)bh_kv * D + ch] = (uint8_t)kc;
+        a.vcm[(int64_t)bh_kv * D + ch] = (uint8_t)vc;
+    }
     // (b) scores of the tail: fp16(fp16(q.k) / sqrt(D)), the two roundings of an fp16 matmul followed by
     //     an fp16 division (extension/k_cache_file.py:156)
     const float sqrt_d = sqrtf((float)D);
@@ -423,7 +422,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
         }
     }
     lds_barrier();
-    store_append();
     // SPLIT: the stage's loads are all back; from here to the probe it only computes, and memory is the caller's
     auto hook_at = [&](auto point) {
         if constexpr (SPLIT) {
