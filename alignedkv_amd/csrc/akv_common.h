@@ -150,6 +150,14 @@ __device__ __forceinline__ float exp_nonpositive(float x) {
     return fmaf(e, err * ln2, e);
 }
 
+// Makes the compiler fetch kernel arguments where this stands (the entry block) instead of in the block of their first
+// use: arguments that are first needed behind a branch otherwise arrive in a scalar load of their own there, a
+// dependent round trip in front of the loads that need them.
+template <typename... T>
+__device__ __forceinline__ void fetch_arguments_now(T... p) {
+    (..., [](auto x) { asm volatile("" ::"s"(x)); }(p));
+}
+
 constexpr int kSkip = 0x7fffffff;   // an offset no plane slice reaches
 
 // Cache-policy bits of buffer loads/stores on gfx950: sc1 = device (agent) scope.  Data that one
@@ -237,6 +245,13 @@ __device__ __forceinline__ u32 rows_max_u32(u32 v) {
 __device__ __forceinline__ u32 quads_max_u32(u32 v) {
     v = max(v, (u32)__builtin_amdgcn_update_dpp(0, (int)v, 0x124, 0xf, 0xf, false));   // row_ror:4
     v = max(v, (u32)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xf, 0xf, false));   // row_ror:8
+    return rows_max_u32(v);
+}
+__device__ __forceinline__ u32 wave_max_u32(u32 v) {
+    v = max(v, dpp_u32<kDppXor1>(v));
+    v = max(v, dpp_u32<kDppXor2>(v));
+    v = max(v, dpp_u32<kDppHalfMirror>(v));
+    v = max(v, dpp_u32<kDppMirror>(v));
     return rows_max_u32(v);
 }
 __device__ __forceinline__ int wave_sum_i32(int v) {

@@ -298,15 +298,20 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
 // channels each, request all their rows at once (12 KiB per wave, five waves per SIMD) and add their partial scores
 // through LDS.  (A block per wave with double-buffered half tiles measured behind on every shape: 33.9 vs 33.6 us at
 // batch 8 x 4096 tokens, 155.2 vs 146.9 at 4 x 32768, 8.1 vs 5.2 at 1 x 1024.)  grid (n_kblocks, H, B), 256 threads.
-template <int D, bool REF, int NWV>
+// UNIFORM: one length for every sequence (no task map and no per-sequence lengths to look up in front of a workgroup's
+// first requests).
+template <int D, bool REF, int NWV, bool UNIFORM>
 __global__ __launch_bounds__(64 * NWV) void fused_k_pass256_split_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
     unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, StepGeom geo, float scale) {
-    int blk, h, b;
-    if (!step_block(geo, blk, h, b)) return;
+    fetch_arguments_now(first_8, mid_4, last_4, kcm, q, k_new, scores, levels_out);
+    int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+    if constexpr (!UNIFORM) {
+        if (!step_block(geo, blk, h, b)) return;
+    }
     int R, nrest;
-    seq_state(geo, b, R, nrest);
+    seq_state<UNIFORM>(geo, b, R, nrest);
     if (blk >= (R + 255) / 256) return;
     k_pass256_split_block<D, REF, NWV>(first_8, mid_4, last_4, kcm, q, k_new, scores, levels_out, geo, scale, blk, b * geo.Hq + h, R);
 }
@@ -749,12 +754,13 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     } else if (n_blocks > 0 && kb == 256) {
         dim3 grid(ks.grid_x, ks.grid_y, B);
         if constexpr (D <= 128) {
-            if (ref)
-                hipLaunchKernelGGL((fused_k_pass256_split_kernel<D, true, 4>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                                   k_levels_out, geo_k, scale);
-            else
-                hipLaunchKernelGGL((fused_k_pass256_split_kernel<D, false, 4>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16,
-                                   k_levels_out, geo_k, scale);
+#define AKV_KS(RF, UNI)                                                                                                      \
+    hipLaunchKernelGGL((fused_k_pass256_split_kernel<D, RF, 4, UNI>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16, k16, s16, \
+                       k_levels_out, geo_k, scale)
+            const bool uniform = geo_k.seq_lens == nullptr && geo_k.task_map == nullptr;
+            if (ref) { if (uniform) AKV_KS(true, true); else AKV_KS(true, false); }
+            else { if (uniform) AKV_KS(false, true); else AKV_KS(false, false); }
+#undef AKV_KS
         }
         int rc = check_launch("decode_step(k_pass256 split)");
         if (rc != AKV_OK) return rc;

@@ -88,18 +88,26 @@ __device__ __forceinline__ void k_pass256_split_block(
     for (int i = 0; i < NT; ++i) k256_issue_h<D, HG>(t[i], rH, blk, g_first + HG * i);
     __builtin_amdgcn_sched_barrier(0);
     __shared__ u32 staged[D];      // [channel]: q bits | exponent sum << 16
+    __shared__ u32 staged_max[NWV];  // [wave]: largest exponent sum among the channels the wave staged
     __shared__ float part[NWV][KB];  // [wave][slot]: partial scores
-    for (int c = threadIdx.x; c < D; c += 64 * NWV) {
-        const u32 qb = q[(int64_t)bh * D + c];
-        // column max including the token appended by this step
-        const u32 cm = max((u32)kcm[(int64_t)bh * D + c], exp_field(k_new[(int64_t)bh * D + c]));
-        staged[c] = qb | (((exp_field(qb) + cm) & 0xffu) << 16);
+    static_assert(D <= 64 * NWV, "a thread stages at most one channel");
+    {
+        u32 es = 0;
+        const int c = threadIdx.x;
+        if (c < D) {
+            const u32 qb = q[(int64_t)bh * D + c];
+            // column max including the token appended by this step
+            const u32 cm = max((u32)kcm[(int64_t)bh * D + c], exp_field(k_new[(int64_t)bh * D + c]));
+            es = (exp_field(qb) + cm) & 0xffu;
+            staged[c] = qb | (es << 16);
+        }
+        es = wave_max_u32(es);
+        if (lane == 0) staged_max[wave] = es;
     }
     __syncthreads();
     u32 mx = 0;
 #pragma unroll
-    for (int g = 0; g < NG; ++g) mx = max(mx, staged[4 * g + (lane >> 4)] >> 16);
-    mx = rows_max_u32(mx);
+    for (int w = 0; w < NWV; ++w) mx = max(mx, staged_max[w]);
     float qf[GW];
     u32 need_mid = 0, need_last = 0;   // bit g: of the wave's group g
 #pragma unroll
@@ -109,8 +117,14 @@ __device__ __forceinline__ void k_pass256_split_block(
         const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)(w >> 16));
         need_mid |= (lv < 2 ? 1u : 0u) << g;
         need_last |= (lv == 0 ? 1u : 0u) << g;
-        if (levels_out != nullptr && blk == 0 && (lane & 15) == 0)
+    }
+    // (the optional record of the levels: one branch outside the loop, so that the loop's LDS reads go out together)
+    if (levels_out != nullptr && blk == 0 && (lane & 15) == 0) {
+#pragma unroll
+        for (int g = 0; g < GW; ++g) {
+            const int lv = ((need_last >> g) & 1u) ? 0 : (((need_mid >> g) & 1u) ? 1 : 2);
             levels_out[(int64_t)bh * D + 4 * (g_first + g) + (lane >> 4)] = (uint8_t)lv;
+        }
     }
 #pragma unroll
     for (int i = 0; i < NT; ++i)

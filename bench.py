@@ -671,7 +671,7 @@ def main():
     if a.k_block == 64:
         k_kernel = "akv::fused_k_pass_kernel<%d, false, true>" % D if D <= 128 else "akv::fused_k_pass_kernel<%d, false, false>" % D
     else:
-        k_kernel = "akv::fused_k_pass256_split_kernel<%d, false, 4>" % D
+        k_kernel = "akv::fused_k_pass256_split_kernel<%d, false, 4, true>" % D
     tail_kernel = "akv::tail_step_kernel<%d, 512, 2, false>" % D
     res = {
         "metric": "decode-attn us/step (+ effective HBM GB/s, %% of peak), B=%d L=%d %dx%d" % (B, L, H, D),
