@@ -83,6 +83,15 @@ __device__ __forceinline__ void k_pass256_split_block(
     const __amdgpu_buffer_rsrc_t rM = make_rsrc(mid_4 + plane_off, (u32)n_blocks * (D * KB / 2));
     const __amdgpu_buffer_rsrc_t rL = make_rsrc(last_4 + plane_off, (u32)n_blocks * (D * KB / 2));
     const int g_first = wave * GW;
+    // q, the column maxima and the new key of the thread's channel first: loads come back in the order they were
+    // issued, so behind the plane rows these three would be waited for as long as the rows take, and the nibble rows
+    // (which need the levels) would leave a whole round trip after the high bytes instead of right behind them.
+    static_assert(D <= 64 * NWV, "a thread stages at most one channel");
+    const int sc = threadIdx.x < D ? (int)threadIdx.x : kSkip / 2;
+    const u32 s_q = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(make_rsrc(q + (int64_t)bh * D, D * 2), sc * 2, 0, 0);
+    const u32 s_kn = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(make_rsrc(k_new + (int64_t)bh * D, D * 2), sc * 2, 0, 0);
+    const u32 s_cm = (u32)(unsigned char)__builtin_amdgcn_raw_buffer_load_b8(make_rsrc(kcm + (int64_t)bh * D, D), sc, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
     KHalfTile<HG> t[NT];
 #pragma unroll
     for (int i = 0; i < NT; ++i) k256_issue_h<D, HG>(t[i], rH, blk, g_first + HG * i);
@@ -90,17 +99,11 @@ __device__ __forceinline__ void k_pass256_split_block(
     __shared__ u32 staged[D];      // [channel]: q bits | exponent sum << 16
     __shared__ u32 staged_max[NWV];  // [wave]: largest exponent sum among the channels the wave staged
     __shared__ float part[NWV][KB];  // [wave][slot]: partial scores
-    static_assert(D <= 64 * NWV, "a thread stages at most one channel");
     {
-        u32 es = 0;
-        const int c = threadIdx.x;
-        if (c < D) {
-            const u32 qb = q[(int64_t)bh * D + c];
-            // column max including the token appended by this step
-            const u32 cm = max((u32)kcm[(int64_t)bh * D + c], exp_field(k_new[(int64_t)bh * D + c]));
-            es = (exp_field(qb) + cm) & 0xffu;
-            staged[c] = qb | (es << 16);
-        }
+        // column max including the token appended by this step (a thread without a channel read zeros)
+        const u32 cm = max(s_cm, exp_field(s_kn));
+        u32 es = threadIdx.x < D ? (exp_field(s_q) + cm) & 0xffu : 0u;
+        if (threadIdx.x < D) staged[threadIdx.x] = s_q | (es << 16);
         es = wave_max_u32(es);
         if (lane == 0) staged_max[wave] = es;
     }
