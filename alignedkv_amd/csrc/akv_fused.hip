@@ -233,7 +233,7 @@ __global__ __launch_bounds__(256) void fused_pre_kernel(uint8_t *__restrict__ kf
 // ------------------------------------------------------------------------------------------------
 // K pass.  grid (ceil(n_blocks / (4*blocks_per_wave)), H, B), 256 threads.
 // ------------------------------------------------------------------------------------------------
-template <int D, bool REF, bool WHOLE = false>
+template <int D, bool REF, bool WHOLE = false, bool UNIFORM = false>
 __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
@@ -242,12 +242,16 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     constexpr int CB = 64;
     constexpr int NG = D / 16;
     const int lane = threadIdx.x & 63, wave = wave_index();
-    int bx, hkv, b, chunk, gq;
-    if (!step_block(geo, bx, hkv, b)) return;
-    decode_group_block(geo.G, bx, chunk, gq);
+    fetch_arguments_now(first_8, mid_4, last_4, kcm, q, k_new, scores, levels_out);
+    // UNIFORM: one query head per KV head and one length for every sequence (nothing to look up before the first requests)
+    int bx = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z, chunk = bx, gq = 0;
+    if constexpr (!UNIFORM) {
+        if (!step_block(geo, bx, hkv, b)) return;
+        decode_group_block(geo.G, bx, chunk, gq);
+    }
     const int bh_kv = b * geo.Hkv + hkv, bh = b * geo.Hq + hkv * geo.G + gq;
     int R, nrest;
-    seq_state(geo, b, R, nrest);
+    seq_state<UNIFORM>(geo, b, R, nrest);
     if constexpr (WHOLE) {
         // blocks_per_wave == 1: every channel of the wave's block is requested at once
         if constexpr (D <= 128) k_pass64_whole_blocks<D, REF>(first_8, mid_4, last_4, kcm, q, k_new, scores, levels_out, geo, scale, chunk, bh_kv, bh, R);
@@ -772,7 +776,16 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         bool launched = false;
         if constexpr (D <= 128) {
             if (k_whole) {
-                if (ref) AKV_KP(true, true); else AKV_KP(false, true);
+                if (geo_k.G == 1 && geo_k.seq_lens == nullptr && geo_k.task_map == nullptr) {
+                    if (ref)
+                        hipLaunchKernelGGL((fused_k_pass_kernel<D, true, true, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16,
+                                           k16, s16, k_levels_out, geo_k, bpw, scale);
+                    else
+                        hipLaunchKernelGGL((fused_k_pass_kernel<D, false, true, true>), grid, dim3(256), 0, st, kf8, km4, kl4, kcm, q16,
+                                           k16, s16, k_levels_out, geo_k, bpw, scale);
+                } else {
+                    if (ref) AKV_KP(true, true); else AKV_KP(false, true);
+                }
                 launched = true;
             }
         }

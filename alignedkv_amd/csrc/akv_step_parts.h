@@ -22,38 +22,48 @@ __device__ __forceinline__ void k_pass64_whole_blocks(
     const int n_blocks = R / CB;
     const int blk = chunk * 4 + wave;    // may lie past the end: the wave then only helps staging
     const int64_t plane_off = (int64_t)bh_kv * geo.n_max_blocks * (D * (CB / 2));
+    // q, the column maxima and the new key of the thread's channel first (loads come back in the order they were issued:
+    // behind the plane rows these three would be waited for as long as the rows take), then the block's high bytes.
+    static_assert(D <= 256, "a thread stages at most one channel");
+    const int sc = threadIdx.x < D ? (int)threadIdx.x : kSkip / 2;
+    const u32 s_q = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(make_rsrc(q + (int64_t)bh * D, D * 2), sc * 2, 0, 0);
+    const u32 s_kn = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(make_rsrc(k_new + (int64_t)bh_kv * D, D * 2), sc * 2, 0, 0);
+    const u32 s_cm = (u32)(unsigned char)__builtin_amdgcn_raw_buffer_load_b8(make_rsrc(kcm + (int64_t)bh_kv * D, D), sc, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
     KHalfTile<NG> ta;
     k_issue_half_h<D, NG>(ta, make_rsrc(first_8 + plane_off * 2, (u32)n_blocks * (D * CB)), blk, 0);
     __builtin_amdgcn_sched_barrier(0);
     // q and the exponent sums of all channels, staged once per workgroup (three scattered global loads per
     // channel and wave otherwise: half as many load instructions again as the planes themselves need)
     __shared__ u32 staged[D];      // [channel]: q bits | exponent sum << 16
-    for (int c = threadIdx.x; c < D; c += 256) {
-        const u32 qb = q[(int64_t)bh * D + c];
-        // column max including the token appended by this step
-        const u32 cm = max((u32)kcm[(int64_t)bh_kv * D + c], exp_field(k_new[(int64_t)bh_kv * D + c]));
-        staged[c] = qb | (((exp_field(qb) + cm) & 0xffu) << 16);
+    __shared__ u32 staged_max[4];  // [wave]: largest exponent sum among the channels the wave staged
+    {
+        // column max including the token appended by this step (a thread without a channel read zeros)
+        const u32 cm = max(s_cm, exp_field(s_kn));
+        u32 es = threadIdx.x < D ? (exp_field(s_q) + cm) & 0xffu : 0u;
+        if (threadIdx.x < D) staged[threadIdx.x] = s_q | (es << 16);
+        es = wave_max_u32(es);
+        if (lane == 0) staged_max[wave] = es;
     }
     __syncthreads();
+    const u32 mx = max(max(staged_max[0], staged_max[1]), max(staged_max[2], staged_max[3]));
     float qf[NG];
-    u32 esum[NG];
-    u32 mx = 0;
+    u32 need_mid = 0, need_last = 0;
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
         const u32 w = staged[g * 16 + (lane >> 2)];
         qf[g] = lo_half_to_float(w);
-        esum[g] = w >> 16;
-        mx = max(mx, esum[g]);
-    }
-    mx = quads_max_u32(mx);
-    u32 need_mid = 0, need_last = 0;
-#pragma unroll
-    for (int g = 0; g < NG; ++g) {
-        const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)esum[g]);
+        const int lv = REF ? 0 : k_level((unsigned char)mx, (unsigned char)(w >> 16));
         need_mid |= (lv < 2 ? 1u : 0u) << g;
         need_last |= (lv == 0 ? 1u : 0u) << g;
-        if (levels_out != nullptr && chunk == 0 && wave == 0 && (lane & 3) == 0)
+    }
+    // (the optional record of the levels: one branch outside the loop, so that the loop's LDS reads go out together)
+    if (levels_out != nullptr && chunk == 0 && wave == 0 && (lane & 3) == 0) {
+#pragma unroll
+        for (int g = 0; g < NG; ++g) {
+            const int lv = ((need_last >> g) & 1u) ? 0 : (((need_mid >> g) & 1u) ? 1 : 2);
             levels_out[(int64_t)bh * D + g * 16 + (lane >> 2)] = (uint8_t)lv;
+        }
     }
     if (blk < n_blocks)
         k_score_block_whole<D>(ta, mid_4 + plane_off, last_4 + plane_off, n_blocks, blk, qf, need_mid, need_last,

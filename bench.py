@@ -669,7 +669,7 @@ def main():
     default_workload = (B, H, D, L, a.k_kind) == (8, 32, 128, 4096, "outlier")
     prof = profile_figures("decode_step_c2" + ("" if a.k_block == 256 else "_k_block64")) if default_workload else {}
     if a.k_block == 64:
-        k_kernel = "akv::fused_k_pass_kernel<%d, false, true>" % D if D <= 128 else "akv::fused_k_pass_kernel<%d, false, false>" % D
+        k_kernel = "akv::fused_k_pass_kernel<%d, false, true, true>" % D if D <= 128 else "akv::fused_k_pass_kernel<%d, false, false, false>" % D
     else:
         k_kernel = "akv::fused_k_pass256_split_kernel<%d, false, 4, true>" % D
     tail_kernel = "akv::tail_step_kernel<%d, 512, 2, false>" % D
