@@ -360,6 +360,8 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     // the row's probabilities stay in LDS for the V part (the copy in memory is the step's debug output)
     __shared__ __attribute__((aligned(16))) unsigned short probs_lds[tail_max_tokens + 64];
     __shared__ u32 fine_list[NW][tail_max_tokens / NW];
+    fetch_arguments_now(v_first_8, v_mid_4, v_last_4, ma.q, ma.k_new, ma.v_new, ma.mask, ma.restk, ma.restv, ma.scores, ma.probs,
+                        ma.kcm, ma.vcm, ma.toe, ma.amin, ma.v_first_8, out, v_levels_out, amin_out, ma.g.row_stride, ma.persist);
     const int wave = wave_index();
     const int bh = blockIdx.x;
     int R, nrest_unused;
