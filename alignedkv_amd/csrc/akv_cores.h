@@ -467,7 +467,10 @@ struct VListed {
 };
 
 // PAUX: cache policy of the probability loads (kDeviceScope when another workgroup of the same launch wrote them)
-template <int D, bool REF, int NIT, int PAUX = 0>
+// PREFETCHED: the caller has requested the first half tile's high bytes (v_prefetch_first); otherwise they are requested
+// here, behind the probabilities -- loads come back in the order they were issued, so the small loads that the fetch
+// levels depend on go first where nothing else has to happen in between.
+template <int D, bool REF, int NIT, int PAUX = 0, bool PREFETCHED = true>
 __device__ __forceinline__ void v_accumulate(VFirstTile<D> &ft, const uint8_t *f8, const uint8_t *m4, const uint8_t *l4,
                                              int n_tokens, const unsigned short *s_row, unsigned char amin, int t_begin,
                                              int t_end, float *acc, uint8_t *levels_row) {
@@ -493,6 +496,7 @@ __device__ __forceinline__ void v_accumulate(VFirstTile<D> &ft, const uint8_t *f
             sb[hf][u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(rS, t < t_end ? t * 2 : kSkip, 0, PAUX);
         }
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (!PREFETCHED) v_prefetch_first<D>(ft, f8, n_tokens, t_begin, t_end);
     // Software pipeline over half tiles (see k_score_blocks): one half tile is in flight while the other is
     // multiplied; sched_barrier(0) keeps the instruction scheduler from merging the phases.
     VHalfTile<HV> &ta = ft.t;

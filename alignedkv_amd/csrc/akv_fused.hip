@@ -545,34 +545,38 @@ __global__ void fused_amin_literal_kernel(const uint8_t *__restrict__ toe, const
 // ------------------------------------------------------------------------------------------------
 // V pass.  grid (n_chunks, H, B), 256 threads.
 // ------------------------------------------------------------------------------------------------
-template <int D, bool REF, int NIT>
+// UNIFORM: one query head per KV head and one length for every sequence (nothing to look up before the first requests)
+template <int D, bool REF, int NIT, bool UNIFORM = false>
 __global__ __launch_bounds__(256) void fused_v_pass_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const unsigned short *__restrict__ probs, const uint8_t *__restrict__ amin_u8, float *__restrict__ partial,
     uint8_t *__restrict__ levels_out, int levels_stride, uint8_t *__restrict__ amin_out, StepGeom geo,
     int tokens_per_wave, int n_chunks) {
+    fetch_arguments_now(first_8, mid_4, last_4, probs, amin_u8, partial, levels_out, amin_out);
     __shared__ float wave_part[4][D];
     const int wave = wave_index();
-    int bx, hkv, b, chunk, gq;
-    if (!step_block(geo, bx, hkv, b)) return;
-    decode_group_block(geo.G, bx, chunk, gq);
+    int bx = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z, chunk = bx, gq = 0;
+    if constexpr (!UNIFORM) {
+        if (!step_block(geo, bx, hkv, b)) return;
+        decode_group_block(geo.G, bx, chunk, gq);
+    }
     const int bh_kv = b * geo.Hkv + hkv, bh = b * geo.Hq + hkv * geo.G + gq;
     if (chunk >= n_chunks) return;    // padding of the grid (whole workgroup)
     int n_tokens, nrest;
-    seq_state(geo, b, n_tokens, nrest);
+    seq_state<UNIFORM>(geo, b, n_tokens, nrest);
     const int t_begin = (chunk * 4 + wave) * tokens_per_wave;
     const int t_end = min(t_begin + tokens_per_wave, n_tokens);
     const int64_t row0 = (int64_t)bh_kv * geo.max_seq_len;
-    VFirstTile<D> ft;
-    v_prefetch_first<D>(ft, first_8 + row0 * D, n_tokens, t_begin, t_end);
+    // the threshold and (inside v_accumulate) the probabilities before the first rows: the levels wait for them only
     const unsigned char amin = REF ? 0 : amin_u8[bh];
-    if (!REF && amin_out != nullptr && chunk == 0 && threadIdx.x == 0) amin_out[bh] = amin;
+    VFirstTile<D> ft;
     float acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    v_accumulate<D, REF, NIT>(ft, first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
-                              probs + (int64_t)bh * geo.row_stride, amin, t_begin, t_end, acc,
-                              levels_out != nullptr ? levels_out + (int64_t)bh * levels_stride : nullptr);
+    v_accumulate<D, REF, NIT, 0, false>(ft, first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
+                                        probs + (int64_t)bh * geo.row_stride, amin, t_begin, t_end, acc,
+                                        levels_out != nullptr ? levels_out + (int64_t)bh * levels_stride : nullptr);
+    if (!REF && amin_out != nullptr && chunk == 0 && threadIdx.x == 0) amin_out[bh] = amin;
     v_fold_workgroup<D>(acc, wave_part, partial + ((int64_t)bh * n_chunks + chunk) * D);
 }
 
@@ -870,9 +874,15 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         if (rc != AKV_OK) return rc;
     } else if (p.n_chunks > 0) {
         dim3 grid(group_grid_x(p.n_chunks, geo.G), Hkv, B);
-#define AKV_VP(RF, N)                                                                                                  \
-    hipLaunchKernelGGL((fused_v_pass_kernel<D, RF, N>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, amin, partial,     \
+        const bool uniform_v = geo_v.G == 1 && geo_v.seq_lens == nullptr && geo_v.task_map == nullptr;
+#define AKV_VP1(RF, N, UNI)                                                                                               \
+    hipLaunchKernelGGL((fused_v_pass_kernel<D, RF, N, UNI>), grid, dim3(256), 0, st, vf8, vm4, vl4, p16, amin, partial,   \
                        v_levels_out, R, amin_out, geo_v, p.tokens_per_wave, p.n_chunks)
+#define AKV_VP(RF, N)                                                                                                     \
+    do {                                                                                                                  \
+        if (uniform_v) AKV_VP1(RF, N, true);                                                                              \
+        else AKV_VP1(RF, N, false);                                                                                       \
+    } while (0)
         if (ref) {
             if (p.iters_per_wave == 1) AKV_VP(true, 1);
             else if (p.iters_per_wave == 2) AKV_VP(true, 2);
@@ -883,6 +893,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
             else AKV_VP(false, 4);
         }
 #undef AKV_VP
+#undef AKV_VP1
         rc = check_launch("decode_step(v_pass)");
         if (rc != AKV_OK) return rc;
     }
