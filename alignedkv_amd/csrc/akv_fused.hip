@@ -326,6 +326,8 @@ __global__ __launch_bounds__(64 * NWV) void fused_k_pass256_split_kernel(
 // grid (B*H), 256 threads: the middle stage on its own (no flushed block yet, or fusion switched off).
 template <int D, int NT>
 __global__ __launch_bounds__(NT) void fused_middle_kernel(MiddleArgs a) {
+    fetch_arguments_now(a.q, a.k_new, a.v_new, a.mask, a.restk, a.restv, a.scores, a.probs, a.otail, a.kcm, a.vcm, a.toe, a.amin,
+                        a.v_first_8, a.g.seq_lens, a.g.row_stride, a.persist);
     __shared__ MiddleShared<D, NT / 64> ms;
     middle_body<D, NT>(a, blockIdx.x, ms);
 }

@@ -264,6 +264,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && 
     constexpr int PB = 64 / SL;    // pieces (token sets) per block
     constexpr int NBT = 16 / PB;   // blocks per task
     static_assert(KG % (AHEAD + 1) == 0, "the tile ring is rotated by unrolling");
+    fetch_arguments_now(first_8, mid_4, last_4, prep, scores, geo.seq_lens, geo.task_map);
     const int lane = threadIdx.x & 63, wave = wave_index();
     int chunk, hkv, b;
     if (!step_block(geo, chunk, hkv, b)) return;
@@ -511,6 +512,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     constexpr int CPP = D / 16;        // channels per lane
     constexpr int MACRO = 64;          // tokens per macro step: 4 tiles of 16 tokens
     __shared__ float fold[4][4][D];    // [wave][head of the pass][channel]
+    fetch_arguments_now(first_8, mid_4, last_4, probs, amin_u8, partial, levels_out, amin_out, geo.seq_lens, geo.task_map);
     const int lane = threadIdx.x & 63, wave = wave_index();
     int chunk, hkv, b;
     if (!step_block(geo, chunk, hkv, b)) return;
