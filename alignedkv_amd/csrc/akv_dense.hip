@@ -37,6 +37,7 @@ __global__ __launch_bounds__(256) void dense_k_pass_kernel(const unsigned short 
                                                            int max_seq_len, int row_stride, int n_tokens,
                                                            int tokens_per_wave, float sqrt_d) {
     constexpr int D = 128;
+    fetch_arguments_now(k_cache, q, scores);
     const int lane = threadIdx.x & 63, wave = wave_index();
     const int h = blockIdx.y, b = blockIdx.z, bh = b * H + h;
     const int t_begin = (blockIdx.x * 4 + wave) * tokens_per_wave;
@@ -194,6 +195,7 @@ __global__ __launch_bounds__(256) void dense_v_pass_kernel(const unsigned short 
                                                            int row_stride, int n_tokens, int tokens_per_wave,
                                                            int n_chunks) {
     constexpr int D = 128;
+    fetch_arguments_now(v_cache, probs, partial);
     __shared__ float wave_part[4][D];
     const int lane = threadIdx.x & 63, wave = wave_index();
     const int chunk = blockIdx.x, h = blockIdx.y, b = blockIdx.z, bh = b * H + h;
