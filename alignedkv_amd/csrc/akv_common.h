@@ -152,7 +152,9 @@ __device__ __forceinline__ float exp_nonpositive(float x) {
 
 // Makes the compiler fetch kernel arguments where this stands (the entry block) instead of in the block of their first
 // use: arguments that are first needed behind a branch otherwise arrive in a scalar load of their own there, a
-// dependent round trip in front of the loads that need them.
+// dependent round trip in front of the loads that need them.  Only for kernels that look nothing up through uniform
+// loads afterwards (task maps, per-sequence lengths): behind this statement the compiler no longer proves such loads
+// unclobbered and issues them as vector loads.
 template <typename... T>
 __device__ __forceinline__ void fetch_arguments_now(T... p) {
     (..., [](auto x) { asm volatile("" ::"s"(x)); }(p));

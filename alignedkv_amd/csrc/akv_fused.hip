@@ -242,7 +242,7 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
     constexpr int CB = 64;
     constexpr int NG = D / 16;
     const int lane = threadIdx.x & 63, wave = wave_index();
-    fetch_arguments_now(first_8, mid_4, last_4, kcm, q, k_new, scores, levels_out);
+    if constexpr (UNIFORM) fetch_arguments_now(first_8, mid_4, last_4, kcm, q, k_new, scores, levels_out);
     // UNIFORM: one query head per KV head and one length for every sequence (nothing to look up before the first requests)
     int bx = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z, chunk = bx, gq = 0;
     if constexpr (!UNIFORM) {
@@ -309,7 +309,7 @@ __global__ __launch_bounds__(64 * NWV) void fused_k_pass256_split_kernel(
     const uint8_t *__restrict__ first_8, const uint8_t *__restrict__ mid_4, const uint8_t *__restrict__ last_4,
     const uint8_t *__restrict__ kcm, const unsigned short *__restrict__ q, const unsigned short *__restrict__ k_new,
     unsigned short *__restrict__ scores, uint8_t *__restrict__ levels_out, StepGeom geo, float scale) {
-    fetch_arguments_now(first_8, mid_4, last_4, kcm, q, k_new, scores, levels_out);
+    if constexpr (UNIFORM) fetch_arguments_now(first_8, mid_4, last_4, kcm, q, k_new, scores, levels_out);
     int blk = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
     if constexpr (!UNIFORM) {
         if (!step_block(geo, blk, h, b)) return;
@@ -326,8 +326,6 @@ __global__ __launch_bounds__(64 * NWV) void fused_k_pass256_split_kernel(
 // grid (B*H), 256 threads: the middle stage on its own (no flushed block yet, or fusion switched off).
 template <int D, int NT>
 __global__ __launch_bounds__(NT) void fused_middle_kernel(MiddleArgs a) {
-    fetch_arguments_now(a.q, a.k_new, a.v_new, a.mask, a.restk, a.restv, a.scores, a.probs, a.otail, a.kcm, a.vcm, a.toe, a.amin,
-                        a.v_first_8, a.g.seq_lens, a.g.row_stride, a.persist);
     __shared__ MiddleShared<D, NT / 64> ms;
     middle_body<D, NT>(a, blockIdx.x, ms);
 }
@@ -554,7 +552,7 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
     const unsigned short *__restrict__ probs, const uint8_t *__restrict__ amin_u8, float *__restrict__ partial,
     uint8_t *__restrict__ levels_out, int levels_stride, uint8_t *__restrict__ amin_out, StepGeom geo,
     int tokens_per_wave, int n_chunks) {
-    fetch_arguments_now(first_8, mid_4, last_4, probs, amin_u8, partial, levels_out, amin_out);
+    if constexpr (UNIFORM) fetch_arguments_now(first_8, mid_4, last_4, probs, amin_u8, partial, levels_out, amin_out);
     __shared__ float wave_part[4][D];
     const int wave = wave_index();
     int bx = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z, chunk = bx, gq = 0;

@@ -264,7 +264,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && 
     constexpr int PB = 64 / SL;    // pieces (token sets) per block
     constexpr int NBT = 16 / PB;   // blocks per task
     static_assert(KG % (AHEAD + 1) == 0, "the tile ring is rotated by unrolling");
-    fetch_arguments_now(first_8, mid_4, last_4, prep, scores, geo.seq_lens, geo.task_map);
     const int lane = threadIdx.x & 63, wave = wave_index();
     int chunk, hkv, b;
     if (!step_block(geo, chunk, hkv, b)) return;
@@ -512,7 +511,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     constexpr int CPP = D / 16;        // channels per lane
     constexpr int MACRO = 64;          // tokens per macro step: 4 tiles of 16 tokens
     __shared__ float fold[4][4][D];    // [wave][head of the pass][channel]
-    fetch_arguments_now(first_8, mid_4, last_4, probs, amin_u8, partial, levels_out, amin_out, geo.seq_lens, geo.task_map);
     const int lane = threadIdx.x & 63, wave = wave_index();
     int chunk, hkv, b;
     if (!step_block(geo, chunk, hkv, b)) return;
@@ -536,11 +534,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     const __amdgpu_buffer_rsrc_t rP = make_rsrc(probs, probs_bytes);
     const int j = lane & 15, kq = lane >> 4;
     const bool head = j < G;
-    const unsigned char amin = (REF || !head) ? 0 : amin_u8[bh0 + j];
-    if (!REF && head && amin_out != nullptr && chunk == 0 && wave == 0 && kq == 0) amin_out[bh0 + j] = amin;
-    // what the levels are measured against; lanes without a head read probabilities of zero, for which this value says level 2
-    const unsigned short a16 = head ? (unsigned short)((unsigned)amin << 10) : (unsigned short)0x0800;
-    const u16x2 a2 = {a16, a16};
+    // The threshold is requested here and first looked at behind the requests of the first tiles and probabilities (the
+    // barrier below keeps the compiler from waiting for it in front of them: a round trip with nothing else in flight).
+    // (a lane without a head reads out of range: zero comes back, and no load sits under a branch)
+    const unsigned char amin_loaded =
+        (unsigned char)__builtin_amdgcn_raw_buffer_load_b8(make_rsrc(amin_u8 + bh0, (u32)G), (REF || !head) ? kSkip : j, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
     const int lane_p = (int)((bh0 + (head ? j : 0)) * geo.row_stride + 4 * kq) * 2;
     const int lane_h = (4 * kq) * D + (lane & 15) * CPP, lane_m = (4 * kq) * (D / 2) + (lane & 15) * (CPP / 2);
 
@@ -563,6 +562,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     for (int i = 0; i < CPP; ++i) acc[i] = (f32x4){0.f, 0.f, 0.f, 0.f};
     LevelPuts puts;
     puts.pin();
+    // what the levels are measured against; lanes without a head read probabilities of zero, for which this value says
+    // level 2.  (Worked out where it is first needed, behind the first requests.)
+    auto threshold_operand = [&]() -> u16x2 {
+        const unsigned short a16 = head ? (unsigned short)((unsigned)amin_loaded << 10) : (unsigned short)0x0800;
+        return (u16x2){a16, a16};
+    };
 
     // Few tokens of the wave below level 2 for any head of the group (the usual case: under 1 % of the (token, head)
     // pairs at batch 32, 32 over 8 heads, but 39 % of the 16-token tiles hold one): every tile is multiplied at level 2
@@ -592,6 +597,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
             u32x2 pall[LIST / MACRO][4];
 #pragma unroll
             for (int mi = 0; mi < LIST / MACRO; ++mi) load_probs(pall[mi], t_begin + mi * MACRO);
+            __builtin_amdgcn_sched_barrier(0);
+            const u16x2 a2 = threshold_operand();
+            const unsigned char amin = amin_loaded;
             {
                 const i16x2 c8 = {0x0800, 0x0800};
                 unsigned long long mask = 0ull;
@@ -694,10 +702,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     if (!handled) {
     u32x2 pn[4], pnn[4];
     VMacroOps oc, on;
+    u16x2 a2;
     {
         u32x2 pc[4];
         load_probs(pc, t_begin);
         load_probs(pn, t_begin + MACRO);
+        __builtin_amdgcn_sched_barrier(0);
+        a2 = threshold_operand();
         v_macro_ops<REF>(oc, pc, a2, head);
     }
     KTaskTile<CPP> t[4];
@@ -731,6 +742,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
     }
     }
     // optional record of the levels, outside the pipeline
+    if (!REF && head && amin_out != nullptr && chunk == 0 && wave == 0 && kq == 0) amin_out[bh0 + j] = amin_loaded;
     if (levels_out != nullptr) {
         for (int tt = t_begin + lane; tt < t_end; tt += 64)
             for (int h = 0; h < G; ++h)
