@@ -193,12 +193,9 @@ struct MiddleShared {
     unsigned short tail_s[64];     // fp16 scores of the tail (mask not yet added)
     float tail_p[64];              // probabilities of the tail
     u32 cand_key[4 * NW][32];      // [16-lane row of the workgroup][residue class]: best (probability, token) key
-    float probe_p[32];
-    int probe_t[32];
-    u32 red_min[NW];
     float tail_o[NW][D];           // per-wave sums of the tail's share of the output
-    u32 vcm[D];                    // V column maxima after the append (SPLIT)
-    u32 amin;                      // the row's alignment threshold (SPLIT)
+    u32 vcm[D];                    // V column maxima after the append
+    u32 amin;                      // the row's alignment threshold
 };
 
 // the tail's share of channel d of the output: the waves' sums in a fixed order
@@ -308,6 +305,9 @@ __device__ __forceinline__ void middle_tail_partials(MiddleShared<D, NT / 64> &m
 // MASKED: 1 / 0 = the caller knows that there is / is no mask row (the other case is not compiled), -1 = looked up at
 // run time.  MAXTOK: an upper bound of the flushed tokens per row that the caller guarantees (0: none; rows beyond
 // what the registers hold take three passes over the scores): both keep a one-shot kernel's code short.
+template <int D, int NW, typename Waiting>
+__device__ __forceinline__ u32 middle_probe_wave(const MiddleArgs &a, MiddleShared<D, NW> &ms, int bh, int R, Waiting while_waiting);
+
 template <int D, int NT, bool SPLIT = false, typename Hook = NoHook, int MASKED = -1, int MAXTOK = 0>
 __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, MiddleShared<D, NT / 64> &ms, Hook hook = Hook(),
                                             unsigned short *probs_lds = nullptr, MiddleCarry<D, NT> *carry_out = nullptr) {
@@ -396,7 +396,6 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
     // (SPLIT: with the first loads, so that nothing the stage needs later queues behind the caller's stream)
     if (SPLIT) request_tail_values();
     // (a) append the token: rest buffers and column maxima (extension/k_cache_file.py:98-101).
-    //     vcm_mine: this thread's channel of the V column maxima after the update (threads < D).
     static_assert(D <= NT, "one channel per thread");
     const bool ch_on = tid < D;               // this thread looks after channel tid of the column maxima
     const int ch = ch_on ? tid : 0;
@@ -414,8 +413,7 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
     // appended the token already).
     kc = max(kc, exp_field(kb));
     vc = max(vc, exp_field(vb));
-    const u32 vcm_mine = vc;
-    if (SPLIT && ch_on) ms.vcm[ch] = vc;
+    if (ch_on) ms.vcm[ch] = vc;
     // The stores of the append: issued here, where the wave waits for its first loads anyway, and in front of the
     // tail's score store -- a wait for a loaded value placed behind a store would also wait for that store to be
     // acknowledged (one counter covers both), a round trip in front of the stage's first barrier.
@@ -578,42 +576,8 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
     // (e) the probe's arg-max per residue class, its 32 gathered rows and the alignment threshold of this (batch, head)
     //     (extension/v_cache_file.py:156-160)
     if constexpr (!SPLIT) {
-        if (R > 0) {
-            if (tid < 32) {
-                u32 key = 0u;
-#pragma unroll
-                for (int k = 0; k < 4 * NW; ++k) key = max(key, ms.cand_key[k][tid]);
-                ms.probe_p[tid] = half_bits_to_float(key >> 16);
-                ms.probe_t[tid] = (int)(0xffffu - (key & 0xffffu)) * 32 + tid;
-            }
-            lds_barrier();
-            u32 align = 0xffu;
-            for (int d = tid; d < D; d += NT) {
-                // the 32 gathered bytes first, then the sum: 32 independent loads in flight instead of a chain
-                u32 hi[32];
-#pragma unroll
-                for (int i = 0; i < 32; ++i) hi[i] = a.v_first_8[((int64_t)bh_kv * a.g.max_seq_len + ms.probe_t[i]) * D + d];
-                float acc = 0.f;
-#pragma unroll
-                for (int i = 0; i < 32; ++i)
-                    acc = fmaf(half_bits_to_float(((hi[i] << 8) | 0x80u) & 0x7fffu), ms.probe_p[i], acc);
-                // exponent with the lowest bit cleared (`& 0x1F - 1`, extension/v_cache_file.py:142)
-                const u32 e = exp_field(float_to_half_bits(acc)) & 0x1eu;
-                a.toe[(int64_t)bh * D + d] = (uint8_t)e;
-                align = min(align, (e + 15u - vcm_mine) & 0xffu);     // uint8 wrap, as the reference's tensor arithmetic
-            }
-#pragma unroll
-            for (int mk = 32; mk >= 1; mk >>= 1) align = min(align, (u32)__shfl_xor((int)align, mk, 64));
-            if (lane == 0) ms.red_min[wave] = align;
-            lds_barrier();
-            if (tid == 0) {
-                u32 mn = ms.red_min[0];
-#pragma unroll
-                for (int w = 1; w < NW; ++w) mn = min(mn, ms.red_min[w]);
-                a.amin[bh] = (uint8_t)mn;
-                ms.amin = mn;   // for a caller that goes on in the same workgroup
-            }
-        }
+        // one wave runs the probe (no barrier inside); the others go on to the tail's share of the output
+        if (R > 0 && wave == 0) middle_probe_wave<D, NW>(a, ms, bh, R, [] {});
     }
     // (f) the tail's share of the output
     if constexpr (SPLIT) {
