@@ -124,15 +124,39 @@ __device__ __forceinline__ void mfma_k_prepare(const uint8_t *__restrict__ kcm, 
     u32 lv1 = 0, lv2 = 0;
     u32 esum[KG][4];
     u32 mx = 0;
+    // Every load first, 16 channels per 16-byte vector (a lane picks its four of them afterwards), none under a
+    // branch: a lane without a head reads q out of range and gets zeros.  One round trip instead of one per group.
+    const __amdgpu_buffer_rsrc_t rQ = make_rsrc(q + bh0 * D, (u32)(G * D * 2));
+    const __amdgpu_buffer_rsrc_t rC = make_rsrc(kcm + (int64_t)bh_kv * D, D);
+    const __amdgpu_buffer_rsrc_t rN = make_rsrc(k_new + (int64_t)bh_kv * D, D * 2);
+    u32x4 cw[KG], qw[KG][2], nw[KG][2];
+#pragma unroll
+    for (int kg = 0; kg < KG; ++kg) {
+        cw[kg] = __builtin_amdgcn_raw_buffer_load_b128(rC, 16 * kg, 0, 0);
+#pragma unroll
+        for (int h2 = 0; h2 < 2; ++h2) {
+            nw[kg][h2] = __builtin_amdgcn_raw_buffer_load_b128(rN, (16 * kg + 8 * h2) * 2, 0, 0);
+            qw[kg][h2] = __builtin_amdgcn_raw_buffer_load_b128(rQ, head ? (j * D + 16 * kg + 8 * h2) * 2 : kSkip, 0, 0);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // channel 16 kg + 4 r + kq: byte kq of word r of the column maxima, half (kq & 1) of word 2 (r & 1) + kq / 2 of
+    // vector r / 2 of q and the new key
+    auto half_at = [&](const u32x4 (&v)[2], int r) -> u32 {
+        const u32x4 w = v[r >> 1];
+        const u32 lo = (r & 1) ? w.z : w.x, hi = (r & 1) ? w.w : w.y;
+        const u32 word = (kq & 2) ? hi : lo;
+        return (kq & 1) ? word >> 16 : word & 0xffffu;
+    };
 #pragma unroll
     for (int kg = 0; kg < KG; ++kg) {
         u32 qb[4];
+        const u32 cws[4] = {cw[kg].x, cw[kg].y, cw[kg].z, cw[kg].w};
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int c = 16 * kg + 4 * r + kq;
-            qb[r] = head ? (u32)q[(bh0 + j) * D + c] : 0u;
+            qb[r] = half_at(qw[kg], r);
             // column max including the token appended by this step
-            const u32 cm = max((u32)kcm[(int64_t)bh_kv * D + c], exp_field(k_new[(int64_t)bh_kv * D + c]));
+            const u32 cm = max((cws[r] >> (8 * kq)) & 0xffu, exp_field(half_at(nw[kg], r)));
             esum[kg][r] = (exp_field(qb[r]) + cm) & 0xffu;
             mx = max(mx, esum[kg][r]);
         }
