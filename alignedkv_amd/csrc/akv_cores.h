@@ -693,7 +693,9 @@ __device__ __forceinline__ int v_stream_count_fine(const unsigned short *s_row, 
 
 // The stream with every token multiplied at level 2 (high bytes only) and no look at the fetch levels: for a caller that
 // does not know the row's threshold yet, or lists the tokens below level 2 some other way (VFineScan).
-// One half tile in flight while one is multiplied; the probabilities come from LDS (probs_lds: the row's, token-indexed).
+// One half tile in flight while one is multiplied; the probabilities come from LDS (probs_lds: the row's, token-indexed;
+// probs_lds[zero_at ...] holds a half tile's worth of zeros, read for a half tile past the wave's share: a wave-uniform
+// choice of the address instead of a branch around every read).
 // prefetched: the share's first half tile has been requested into ring.hi[0] already (by the caller with
 // v_stream_issue_high, or by the call for the share before this one through next_half).
 // next_half: requested into ring.hi[0] when the share's last half tile is being multiplied (the first half tile of the
@@ -705,8 +707,8 @@ struct NoExtra {
 };
 template <int D, int RN, typename Extra = NoExtra>
 __device__ __forceinline__ void v_stream_run_coarse(VRing<D, RN> &ring, const uint8_t *f8, int n_tokens,
-                                                   const unsigned short *probs_lds, const VSeq &seq, bool prefetched, int next_half,
-                                                   float *acc, Extra extra = Extra()) {
+                                                   const unsigned short *probs_lds, int zero_at, const VSeq &seq, bool prefetched,
+                                                   int next_half, float *acc, Extra extra = Extra()) {
     using S = VStream<D>;
     constexpr int HV = S::HV;
     const int lane = threadIdx.x & 63, tl = lane / S::LPR;
@@ -728,7 +730,7 @@ __device__ __forceinline__ void v_stream_run_coarse(VRing<D, RN> &ring, const ui
             const bool on = half < seq.n_halves;
             u32 sb[HV];
 #pragma unroll
-            for (int u = 0; u < HV; ++u) sb[u] = on ? (u32)probs_lds[half * S::HT + tl + u * S::TPL] : 0u;
+            for (int u = 0; u < HV; ++u) sb[u] = (u32)probs_lds[(on ? half * S::HT : zero_at) + tl + u * S::TPL];
             v_compute_half_coarse<HV>(acc, ring.hi[k], sb);
             pin_accumulators(acc);
             __builtin_amdgcn_sched_barrier(0);
@@ -746,8 +748,8 @@ __device__ __forceinline__ void v_stream_run_coarse(VRing<D, RN> &ring, const ui
 // of the newest half tile and the multiplication of the oldest.
 template <int D, int NR, typename Extra = NoExtra>
 __device__ __forceinline__ void v_stream_run_levels(const uint8_t *f8, const uint8_t *m4, const uint8_t *l4, int n_tokens,
-                                                   const unsigned short *probs_lds, unsigned char amin, const VSeq &seq,
-                                                   float *acc, Extra extra = Extra()) {
+                                                   const unsigned short *probs_lds, int zero_at, unsigned char amin,
+                                                   const VSeq &seq, float *acc, Extra extra = Extra()) {
     using S = VStream<D>;
     constexpr int HV = S::HV;
     static_assert(NR >= 2, "one half tile is multiplied while the others travel");
@@ -762,7 +764,7 @@ __device__ __forceinline__ void v_stream_run_levels(const uint8_t *f8, const uin
         // (a half tile past the wave's share: probabilities of zero, level 2, nothing fetched)
         const bool on = half < seq.n_halves;
 #pragma unroll
-        for (int u = 0; u < HV; ++u) p[u] = on ? (u32)probs_lds[half * S::HT + tl + u * S::TPL] : 0u;
+        for (int u = 0; u < HV; ++u) p[u] = (u32)probs_lds[(on ? half * S::HT : zero_at) + tl + u * S::TPL];
         v_stream_issue_high<D>(x, rH, half);
         v_issue_half_ml<D, false, HV>(x, rM, rL, half * S::HT, n_tokens, p, amin);
     };

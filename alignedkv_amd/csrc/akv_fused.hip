@@ -358,7 +358,10 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
     __shared__ MiddleShared<D, NW> ms;
     __shared__ float wave_part[NW][D];
     // the row's probabilities stay in LDS for the V part (the copy in memory is the step's debug output)
-    __shared__ __attribute__((aligned(16))) unsigned short probs_lds[tail_max_tokens + 64];
+    // (+ 64 zeros behind the row and its tail, for half tiles past a wave's share: see v_stream_run_coarse)
+    constexpr int zero_at = tail_max_tokens + 64;
+    __shared__ __attribute__((aligned(16))) unsigned short probs_lds[tail_max_tokens + 64 + 64];
+    if (threadIdx.x < 64) probs_lds[zero_at + threadIdx.x] = 0;
     __shared__ u32 fine_list[NW][tail_max_tokens / NW];
     fetch_arguments_now(v_first_8, v_mid_4, v_last_4, ma.q, ma.k_new, ma.v_new, ma.mask, ma.restk, ma.restv, ma.scores, ma.probs,
                         ma.kcm, ma.vcm, ma.toe, ma.amin, ma.v_first_8, out, v_levels_out, amin_out, ma.g.row_stride, ma.persist);
@@ -418,12 +421,12 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
             const bool on = half < n_halves;
             u32 sb[S::HV];
 #pragma unroll
-            for (int u = 0; u < S::HV; ++u) sb[u] = on ? (u32)probs_lds[half * S::HT + tl + u * S::TPL] : 0u;
+            for (int u = 0; u < S::HV; ++u) sb[u] = (u32)probs_lds[(on ? half * S::HT : zero_at) + tl + u * S::TPL];
             v_compute_half_coarse<S::HV>(acc, pre[k], sb);
         }
         pin_accumulators(acc);
         // (ends with part B's first half tile requested, unless it was the one requested up front)
-        v_stream_run_coarse<D>(ring, f8, R, probs_lds, seq_a2, true, seq_b.half(0), acc, [&](int) { tail_once(); });
+        v_stream_run_coarse<D>(ring, f8, R, probs_lds, zero_at, seq_a2, true, seq_b.half(0), acc, [&](int) { tail_once(); });
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
@@ -446,21 +449,21 @@ __global__ __launch_bounds__(NT) void tail_step_kernel(const uint8_t *__restrict
         VSeq b1 = seq_b, b2 = seq_b;
         b1.count = n_b1;
         b2.start = seq_b.start + n_b1 * seq_b.stride; b2.count = seq_b.count - n_b1;
-        v_stream_run_coarse<D>(ring, f8, R, probs_lds, b1, true, b2.half(0), acc, [&](int) {
+        v_stream_run_coarse<D>(ring, f8, R, probs_lds, zero_at, b1, true, b2.half(0), acc, [&](int) {
             tail_once();
             if (!scan.done()) scan.step(list, count);
         });
         while (!scan.done()) scan.step(list, count);
         VListed<D>::request(first, list, count, 0, rH, rM, rL, amin, 0);
         __builtin_amdgcn_sched_barrier(0);
-        v_stream_run_coarse<D>(ring, f8, R, probs_lds, b2, true, n_halves, acc);
+        v_stream_run_coarse<D>(ring, f8, R, probs_lds, zero_at, b2, true, n_halves, acc);
     } else {
         // Frequent tokens below level 2 (flat attention): the rest of the row streams at the tokens' own levels, and the
         // corrections of what part A multiplied at level 2 ride along, one batch of listed rows per half tile.
         while (!scan.done()) scan.step(list, count);
         VListed<D>::request(first, list, count, 0, rH, rM, rL, amin, 0);
         __builtin_amdgcn_sched_barrier(0);
-        v_stream_run_levels<D, 2>(f8, m4, l4, R, probs_lds, amin, seq_b, acc, [&](int) {
+        v_stream_run_levels<D, 2>(f8, m4, l4, R, probs_lds, zero_at, amin, seq_b, acc, [&](int) {
             VListed<D>::apply(acc, first);
             listed_from += VListed<D>::TPL;
             VListed<D>::request(first, list, count, listed_from, rH, rM, rL, amin, 0);
