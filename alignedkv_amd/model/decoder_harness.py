@@ -22,6 +22,7 @@ import torch
 import torch.nn.functional as F
 
 from .KVCache_AlignedKV import QuantizedCache_AlignedKV
+from .ragged_gqa_cache import RaggedGQACache
 
 
 @dataclass
@@ -68,11 +69,64 @@ class DenseTorchCache:
             k = torch.cat([self.k[layer], k], dim=2)
             v = torch.cat([self.v[layer], v], dim=2)
         self.k[layer], self.v[layer] = k, v
+        if k.shape[1] != q.shape[1]:     # grouped-query heads: repeat_kv
+            k, v = (t.repeat_interleave(q.shape[1] // t.shape[1], dim=1) for t in (k, v))
         w = torch.matmul(q, k.transpose(2, 3)) / math.sqrt(q.shape[-1])
         if mask is not None:
             w = w + mask[:, :, :, :k.shape[-2]]
         w = F.softmax(w, dim=-1, dtype=torch.float32).to(q.dtype)
         return torch.matmul(w, v).transpose(1, 2).contiguous()
+
+
+class DeviceLengthCache:
+    """`auto_compute` over RaggedGQACache: the lengths live on the device and the step advances them itself, and the
+    launches of a decode step are sized by the capacity, so every argument of a step is the same from step to step
+    and a whole decoder step can be captured in a HIP graph (RandomLlamaDecoder.generate_graphed).  Prefill as the
+    reference's (dense attention on the incoming tensors, planes written on the side, model/KVCache_AlignedKV.py:92-99)."""
+
+    def __init__(self, cfg: "DecoderConfig", bsz: int, max_len: int, device="cuda", k_block: int = 64):
+        self.inner = RaggedGQACache(cfg.num_hidden_layers, bsz, max_len, cfg.num_attention_heads, cfg.num_key_value_heads,
+                                    cfg.head_dim, device, k_block=k_block)
+        self.groups = cfg.num_attention_heads // cfg.num_key_value_heads
+        self._host_len = [0] * cfg.num_hidden_layers     # what get_seq_length reports (eager callers)
+
+    def get_seq_length(self, layer: int = 0) -> int:
+        return self._host_len[layer]
+
+    def device_positions(self) -> torch.Tensor:
+        """[1] int32: the position of the next token, read from the lengths of layer 0 (before its step advances them)."""
+        return self.inner.seq_lens[0][:1]
+
+    def auto_compute(self, q, k, v, layer: int, mask=None):
+        S = q.shape[1]
+        if S > 1:
+            assert self._host_len[layer] == 0, "prefill goes into an empty cache"
+            for b in range(q.shape[0]):
+                self.inner.prefill(layer, b, k[b:b + 1], v[b:b + 1])
+            self._host_len[layer] = S
+            kr, vr = (t.repeat_interleave(self.groups, dim=2) if self.groups > 1 else t for t in (k, v))
+            w = torch.matmul(q.transpose(1, 2), kr.permute(0, 2, 3, 1)) / math.sqrt(q.shape[-1])
+            if mask is not None:
+                w = w + mask
+            w = F.softmax(w.float(), dim=-1).type_as(q)
+            return torch.matmul(w, vr.transpose(1, 2)).transpose(1, 2).contiguous()
+        assert mask is None
+        self._host_len[layer] += 1
+        return self.inner.decode(layer, q, k, v, bound=self.inner.max_seq_len - 1)
+
+    def snapshot(self):
+        c = self.inner
+        return [(c.seq_lens[i].clone(), c.k_colmax[i].clone(), c.v_colmax[i].clone()) for i in range(c.n_layers)], list(self._host_len)
+
+    def restore(self, snap):
+        """Takes back the steps since snapshot(), as long as none of them crossed a 64-token boundary (the token rows
+        they appended to the rest buffers are written again by the steps that follow)."""
+        c = self.inner
+        for i, (n, kc, vc) in enumerate(snap[0]):
+            c.seq_lens[i].copy_(n)
+            c.k_colmax[i].copy_(kc)
+            c.v_colmax[i].copy_(vc)
+        self._host_len = list(snap[1])
 
 
 class RandomLlamaDecoder(torch.nn.Module):
@@ -104,13 +158,16 @@ class RandomLlamaDecoder(torch.nn.Module):
         return emb.cos().to(dtype)[None, :, None, :], emb.sin().to(dtype)[None, :, None, :]
 
     @torch.no_grad()
-    def forward(self, input_ids: torch.Tensor, cache) -> torch.Tensor:
-        """input_ids [bsz, seq]; returns logits of the last position [bsz, vocab] (fp32)."""
+    def forward(self, input_ids: torch.Tensor, cache, positions: torch.Tensor = None) -> torch.Tensor:
+        """input_ids [bsz, seq]; returns logits of the last position [bsz, vocab] (fp32).  positions: [seq] device
+        tensor of the tokens' positions (default: counted from the cache's length on the host)."""
         cfg = self.cfg
         B, S = input_ids.shape
-        start = cache.get_seq_length(0)
         x = self.embed[input_ids]
-        cos, sin = self.rope(torch.arange(start, start + S, device=x.device), x.dtype)
+        if positions is None:
+            start = cache.get_seq_length(0)
+            positions = torch.arange(start, start + S, device=x.device)
+        cos, sin = self.rope(positions, x.dtype)
         mask = None
         if S > 1:
             mask = torch.full((S, S), float("-inf"), device=x.device, dtype=x.dtype).triu(1)[None, None]
@@ -129,11 +186,15 @@ class RandomLlamaDecoder(torch.nn.Module):
         return F.linear(x, self.lm_head).float()
 
     @torch.no_grad()
-    def generate(self, prompt_ids: torch.Tensor, steps: int, cache, forced_tokens: torch.Tensor = None):
+    def generate(self, prompt_ids: torch.Tensor, steps: int, cache, forced_tokens: torch.Tensor = None, timings: dict = None):
         """Prefill + `steps` greedy decode steps.  With forced_tokens [bsz, steps] the model is teacher-forced
         (the fed token is given, the greedy choice is still recorded).  Returns (tokens [bsz, steps],
-        logits [steps, bsz, vocab])."""
+        logits [steps, bsz, vocab]).  timings: filled with prefill_s (one synchronisation after the prefill)."""
+        t0 = time.perf_counter()
         logits = self.forward(prompt_ids, cache)
+        if timings is not None:
+            torch.cuda.synchronize()
+            timings["prefill_s"] = time.perf_counter() - t0
         toks, all_logits = [], []
         for s in range(steps):
             nxt = logits.argmax(-1)
@@ -146,11 +207,59 @@ class RandomLlamaDecoder(torch.nn.Module):
         return torch.stack(toks, dim=1), torch.stack(all_logits, dim=0)
 
 
+    @torch.no_grad()
+    def generate_graphed(self, prompt_ids: torch.Tensor, steps: int, cache: DeviceLengthCache,
+                         forced_tokens: torch.Tensor = None, timings: dict = None):
+        """generate() with the decoder step (embedding to logits, the cache's step in every layer) captured once in a HIP
+        graph and replayed per token: the host pays one graph launch and the arg-max per step.  The token fed and the
+        position are device tensors (the position is the cache's own length).  Needs prefill + steps to stay inside one
+        64-token block for the warm-up step that is taken back (see DeviceLengthCache.restore) -- any prompt length whose
+        remainder modulo 64 is not 63."""
+        assert prompt_ids.shape[1] % 64 != 63
+        t0 = time.perf_counter()
+        logits = self.forward(prompt_ids, cache)
+        torch.cuda.synchronize()
+        if timings is not None:
+            timings["prefill_s"] = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        feed = torch.zeros((prompt_ids.shape[0], 1), dtype=torch.long, device=prompt_ids.device)
+        snap = cache.snapshot()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):       # first use of every library on the capture's kind of stream, outside the capture
+            self.forward(feed, cache, positions=cache.device_positions())
+        torch.cuda.current_stream().wait_stream(side)
+        cache.restore(snap)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step_logits = self.forward(feed, cache, positions=cache.device_positions())
+        cache.restore(snap)                 # (the capture ran nothing; the host-side count moved)
+        torch.cuda.synchronize()
+        if timings is not None:
+            timings["capture_s"] = time.perf_counter() - t0
+        toks, all_logits = [], []
+        for s in range(steps):
+            nxt = logits.argmax(-1)
+            toks.append(nxt)
+            all_logits.append(logits)
+            if s + 1 == steps:
+                break
+            feed.copy_((nxt if forced_tokens is None else forced_tokens[:, s])[:, None])
+            graph.replay()
+            cache._host_len = [n + 1 for n in cache._host_len]
+            logits = step_logits.clone()
+        return torch.stack(toks, dim=1), torch.stack(all_logits, dim=0)
+
+
 def make_cache(kind: str, cfg: DecoderConfig, bsz: int, max_len: int, device="cuda", k_block: int = 64):
     """kind: 'alignedkv' (fused step), 'alignedkv_ops' (the reference's op sequence), 'alignedkv_reference'
-    (every plane read), 'dense_torch'."""
+    (every plane read), 'dense_torch', 'alignedkv_graph' / 'alignedkv_device_lengths' (the step with lengths on the
+    device, replayed from a HIP graph / launched eagerly)."""
     if kind == "dense_torch":
         return DenseTorchCache(cfg.num_hidden_layers)
+    if kind in ("alignedkv_graph", "alignedkv_device_lengths"):
+        return DeviceLengthCache(cfg, bsz, max_len, device, k_block=k_block)
     c = QuantizedCache_AlignedKV(cfg, bsz, max_len, device, torch.half, k_block=k_block)
     c.reference = kind == "alignedkv_reference"
     if kind == "alignedkv_ops":
@@ -179,10 +288,18 @@ def main():
         cache = make_cache(kind, cfg, a.batch, a.prefill + a.steps + 64, k_block=a.k_block)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        toks, logits = model.generate(prompt, a.steps, cache, forced_tokens=base_tokens)
+        timings = {}
+        if kind == "alignedkv_graph":
+            toks, logits = model.generate_graphed(prompt, a.steps, cache, forced_tokens=base_tokens, timings=timings)
+        else:
+            toks, logits = model.generate(prompt, a.steps, cache, forced_tokens=base_tokens, timings=timings)
         torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        line = f"{kind:20s} {dt:7.2f} s  {a.batch * a.steps / dt:8.1f} tok/s"
+        dt = time.perf_counter() - t0 - timings.get("capture_s", 0.0)
+        decode = dt - timings["prefill_s"]
+        line = (f"{kind:20s} {dt:7.2f} s  {a.batch * a.steps / dt:8.1f} tok/s  (prefill {timings['prefill_s']:.2f} s; the "
+                f"{a.steps - 1} decode steps alone {decode * 1e3 / (a.steps - 1):.2f} ms/step = {a.batch * (a.steps - 1) / decode:.1f} tok/s)")
+        if "capture_s" in timings:
+            line += f"  (+ {timings['capture_s']:.2f} s once for the warm-up step and the capture)"
         if base_tokens is None:
             base_tokens, base_logits = toks, logits
         else:

@@ -535,15 +535,21 @@ def workload_c5():
     forced with the first run's tokens.  Whole-model wall clock: the GEMMs are torch's."""
     import re
     import subprocess
-    cmd = [sys.executable, "-m", "alignedkv_amd.model.decoder_harness", "--kinds", "dense_torch,alignedkv", "--k-block", "256"]
+    cmd = [sys.executable, "-m", "alignedkv_amd.model.decoder_harness", "--kinds", "dense_torch,alignedkv,alignedkv_graph",
+           "--k-block", "256"]
     try:
         r = subprocess.run(cmd, capture_output=True, text=True, timeout=400, cwd=ROOT)
         out = {"workload": "C5: 32-layer Llama-2-7B-shaped decoder, batch 8, 128-token prompt + 256 greedy steps",
-               "command": "python -m alignedkv_amd.model.decoder_harness --kinds dense_torch,alignedkv --k-block 256"}
+               "command": "python -m alignedkv_amd.model.decoder_harness --kinds dense_torch,alignedkv,alignedkv_graph --k-block 256",
+               "kinds": "dense_torch: dense torch attention; alignedkv: QuantizedCache_AlignedKV.auto_compute, launched eagerly; "
+                        "alignedkv_graph: the step with lengths on the device, the whole decoder step replayed from a HIP graph"}
         for line in r.stdout.splitlines():
             m = re.match(r"(\w+)\s+([\d.]+) s\s+([\d.]+) tok/s(.*)", line.strip())
             if m:
                 out[m.group(1)] = {"seconds": float(m.group(2)), "tokens_per_s": float(m.group(3))}
+                alone = re.search(r"alone ([\d.]+) ms/step = ([\d.]+) tok/s", m.group(4))
+                if alone:
+                    out[m.group(1)].update(decode_ms_per_step=float(alone.group(1)), decode_tokens_per_s=float(alone.group(2)))
                 extra = re.search(r"agreement.*?([\d.]+) %\s+max \|dlogit\| ([\d.]+)", m.group(4))
                 if extra:
                     out[m.group(1)].update(greedy_agreement_pct=float(extra.group(1)), max_abs_dlogit=float(extra.group(2)))

@@ -28,6 +28,39 @@ def test_decoder_with_alignedkv_cache_tracks_dense_attention(kind, tol):
     assert (tokens == ref_tokens).float().mean().item() >= (0.9 if kind == "alignedkv_reference" else 0.6)
 
 
+@pytest.mark.parametrize("heads,kv_heads,k_block", [(4, 4, 64), (4, 4, 256), (8, 2, 256)])
+def test_decoder_step_replayed_from_a_graph_equals_the_eager_steps(heads, kv_heads, k_block):
+    """The decoder step with the cache's lengths on the device is captured once and replayed per token.  Every replay is
+    checked: its logits must equal those of the same steps launched eagerly on a twin cache, bit for bit (same kernels,
+    same launch sizes), with the host's own work and synchronisations between the replays; the planes, rest buffers and
+    lengths the two runs leave behind must be equal as well.  Crosses the 128- and 192-token flushes."""
+    from alignedkv_amd.model.decoder_harness import DecoderConfig, RandomLlamaDecoder, make_cache
+    cfg = DecoderConfig(num_hidden_layers=3, hidden_size=128 * heads, num_attention_heads=heads, num_key_value_heads=kv_heads,
+                        intermediate_size=1024, vocab_size=2000, max_position_embeddings=512)
+    model = RandomLlamaDecoder(cfg, seed=7)
+    B, prefill, steps = 2, 100, 100
+    prompt = torch.randint(0, cfg.vocab_size, (B, prefill), device="cuda", generator=torch.Generator(device="cuda").manual_seed(8))
+    eager = make_cache("alignedkv_device_lengths", cfg, B, 320, k_block=k_block)
+    want_tokens, want_logits = model.generate(prompt, steps, eager)
+    graphed = make_cache("alignedkv_graph", cfg, B, 320, k_block=k_block)
+    tokens, logits = model.generate_graphed(prompt, steps, graphed, forced_tokens=want_tokens)
+    for s in range(steps):
+        assert torch.equal(logits[s], want_logits[s]), f"replay {s}: max |dlogit| {(logits[s] - want_logits[s]).abs().max().item()}"
+    assert torch.equal(tokens, want_tokens)
+    a, b = eager.inner, graphed.inner
+    for layer in range(cfg.num_hidden_layers):
+        assert a.seq_lens[layer].cpu().tolist() == [prefill + steps - 1] * B == b.seq_lens[layer].cpu().tolist()
+        for x, y in zip(a.k_planes[layer] + a.v_planes[layer], b.k_planes[layer] + b.v_planes[layer]):
+            assert torch.equal(x, y)
+        n = (prefill + steps - 1) % 64
+        assert torch.equal(a.restk[layer][:, :n], b.restk[layer][:, :n]) and torch.equal(a.restv[layer][:, :n], b.restv[layer][:, :n])
+        assert torch.equal(a.k_colmax[layer], b.k_colmax[layer]) and torch.equal(a.v_colmax[layer], b.v_colmax[layer])
+    # and against dense torch attention, as the other cache kinds above
+    ref_tokens, ref_logits = model.generate(prompt, steps, make_cache("dense_torch", cfg, B, 320), forced_tokens=want_tokens)
+    err = (logits - ref_logits).abs().max().item()
+    assert err <= 6e-2 * max(1.0, ref_logits.abs().max().item()), f"max |dlogit| {err}"
+
+
 def test_config5_full_size_decoder_with_alignedkv_cache():
     """The 32-layer Llama-2-7B-shaped decoder (d = 4096, 32 heads x 128, fp16 weights ~ N(0, 0.02)) at batch 8: a
     128-token prompt, then 256 greedy steps with the AlignedKV cache in every layer (the loop of the reference's
