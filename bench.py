@@ -103,7 +103,7 @@ def parse():
                     help="c2 only: factor on the query (0 or 0.05: flat attention rows, many V tokens below level 2; "
                          "1: the headline workload)")
     ap.add_argument("--extra-capacity", type=int, default=0,
-                    help="c2 only: tokens of cache capacity beyond cache-len + 64 (changes the pitch of the plane rows)")
+                    help="tokens of cache capacity beyond cache-len + 64 (changes the pitch of the plane rows)")
     ap.add_argument("--workload", default="c2", choices=["c2", "c3"],
                     help="c2: the headline configuration (shape flags apply); c3: grouped-query heads (32 over 8), batch 32, "
                          "lengths uniform in [2048, 8192] -- an extra line, not the headline metric")
@@ -339,15 +339,16 @@ def cpu_dense_torch(torch, B, H, D, L, n_steps=10, warm=3):
 
 def bench_c3(a):
     """Grouped-query, ragged-length decode step (akv_decode_step_gqa) at batch 32, 32 query heads over 8 KV
-    heads x 128, lengths uniform in [2048, 8192].  The lengths are reset before every step so that each step
-    sees the same state."""
+    heads x 128, lengths uniform in [2048, 8192].  In the timed loop the lengths advance by themselves as in a decode
+    loop (the step increments them on the device, sequences whose rest buffer fills flush it); every `grow` steps of
+    a layer they are set back to the drawn lengths, so the workload stays the one named."""
     import numpy as np
     import torch
     import alignedkv_amd
     from alignedkv_amd.model.ragged_gqa_cache import RaggedGQACache
     lib = alignedkv_amd.load_library()
     B, Hq, Hkv, D, cb = 32, a.c3_q_heads, 8, 128, 64
-    Lmax = 8192 + cb
+    Lmax = 8192 + cb + a.extra_capacity
     lens = np.random.default_rng(a.seed + 3).integers(2048, 8193, B)
     if a.c3_len:
         lens[:] = a.c3_len
@@ -364,6 +365,8 @@ def bench_c3(a):
     bound = int(lens.max())
     cache.record_levels = True
 
+    grow = 32       # steps of a layer between two resets of its lengths (the longest sequence stays inside the capacity)
+
     def run(reference, steps, warmup):
         cache.reference = reference
         t0 = 0.0
@@ -372,8 +375,9 @@ def bench_c3(a):
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
             layer = i % a.layers
-            cache.seq_lens[layer].copy_(lens0)
-            cache.len_bound[layer] = bound
+            if (i // a.layers) % grow == 0:
+                cache.seq_lens[layer].copy_(lens0)
+                cache.len_bound[layer] = bound
             cache.decode(layer, q, k_new, v_new)
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / steps
