@@ -61,12 +61,12 @@ __global__ void fused_persist_kernel(const unsigned short *__restrict__ k_new, c
 // themselves advance while it runs).  One workgroup of 256 threads per sequence and map: it sums the entry counts
 // of the sequences before its own, writes its sequence's entries and its share of the kNoTask tail.
 struct TaskMaps {
-    u32 *map_k, *map_v;      // null: no map for that pass
+    u32x2 *map_k, *map_v;    // null: no map for that pass
     int *v_chunks;
     PassShape k, v;
 };
 
-__device__ __forceinline__ void build_task_map(const StepGeom &geo, u32 *map, const PassShape &sh, int B, int *v_chunks,
+__device__ __forceinline__ void build_task_map(const StepGeom &geo, u32x2 *map, const PassShape &sh, int B, int *v_chunks,
                                                int *red, int b_mine) {
     const int tid = threadIdx.x;
     auto chunks_of = [&](int b) {
@@ -94,13 +94,14 @@ __device__ __forceinline__ void build_task_map(const StepGeom &geo, u32 *map, co
     const int at = red[0] + red[2] + red[4] + red[6], total = red[1] + red[3] + red[5] + red[7];
     const int n = chunks_of(b_mine), cnt = n * sh.grid_y;
     if (v_chunks != nullptr && tid == 0) v_chunks[b_mine] = n;
+    const u32 len_mine = (u32)geo.seq_lens[b_mine];
     for (int i = tid; i < cnt; i += 256) {
         const int y = i / n, x = i - y * n;
-        map[at + i] = pack_task(x, y, b_mine);
+        map[at + i] = u32x2{pack_task(x, y, b_mine), len_mine};
     }
     // the entries past the last task: an equal share per workgroup
     const int grid = sh.grid_x * sh.grid_y * B, tail = grid - total, share = (tail + B - 1) / B;
-    for (int i = b_mine * share + tid; i < min((b_mine + 1) * share, tail); i += 256) map[total + i] = kNoTask;
+    for (int i = b_mine * share + tid; i < min((b_mine + 1) * share, tail); i += 256) map[total + i] = u32x2{kNoTask, 0u};
 }
 
 // extra = index among the 2 * B map workgroups: the first B build the K pass's map, the others the V pass's
@@ -628,8 +629,8 @@ static StepLayout step_layout(int B, int H, int D, int max_seq_len) {
     l.prep = l.partial + up((size_t)B * H * max_chunks * D * sizeof(float));
     l.map_k = l.prep + up((size_t)B * H * mfma_k_prep_words(D) * sizeof(u32));   // B * Hkv <= B * H rows are used
     // task maps: a pass has at most B * H * (max_chunks + 1) workgroups
-    l.map_v = l.map_k + up((size_t)B * H * (max_chunks + 1) * sizeof(u32));
-    l.v_chunks = l.map_v + up((size_t)B * H * (max_chunks + 1) * sizeof(u32));
+    l.map_v = l.map_k + up((size_t)B * H * (max_chunks + 1) * sizeof(u32x2));
+    l.v_chunks = l.map_v + up((size_t)B * H * (max_chunks + 1) * sizeof(u32x2));
     l.total = l.v_chunks + up((size_t)B * sizeof(int));
     return l;
 }
@@ -708,9 +709,9 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     const bool v_mapped = mapped && (geo.G == 1 || grouped || matrix_v);
     StepGeom geo_k = geo, geo_v = geo;
     int *v_chunks = nullptr;
-    if (mapped) geo_k.task_map = reinterpret_cast<const u32 *>(ws + lay.map_k);
+    if (mapped) geo_k.task_map = reinterpret_cast<const u32x2 *>(ws + lay.map_k);
     if (v_mapped) {
-        geo_v.task_map = reinterpret_cast<const u32 *>(ws + lay.map_v);
+        geo_v.task_map = reinterpret_cast<const u32x2 *>(ws + lay.map_v);
         v_chunks = reinterpret_cast<int *>(ws + lay.v_chunks);
     }
 
@@ -720,8 +721,8 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
         // per-sequence lengths live on the device: one small kernel appends every token and flushes the rest
         // buffers that fill up with it; its last 2*B workgroups write the task maps
         TaskMaps maps;
-        maps.map_k = mapped ? reinterpret_cast<u32 *>(ws + lay.map_k) : nullptr;
-        maps.map_v = v_mapped ? reinterpret_cast<u32 *>(ws + lay.map_v) : nullptr;
+        maps.map_k = mapped ? reinterpret_cast<u32x2 *>(ws + lay.map_k) : nullptr;
+        maps.map_v = v_mapped ? reinterpret_cast<u32x2 *>(ws + lay.map_v) : nullptr;
         maps.v_chunks = v_chunks;
         maps.k = ks;
         maps.v = vs;
@@ -854,7 +855,8 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     }
     {
         // threads per (batch, head) row: a thread keeps 32 scores in registers between the softmax passes, so
-        // rows above 8192 / 16384 tokens get 512 / 1024 threads (512 and 1024 measure level with 256 at 4096 tokens)
+        // rows above 8192 / 16384 tokens get 512 / 1024 threads (512 and 1024 measure level with 256 at 4096 tokens for 256
+        // rows; for 1024 rows of 2048 to 8192 tokens the stage takes 12.3 / 15.2 / 25.1 us with 256 / 512 / 1024)
         const int nt = R <= 8192 ? 256 : (R <= 16384 ? 512 : 1024);
         if (nt == 1024) hipLaunchKernelGGL((fused_middle_kernel<D, 1024>), dim3(B * Hq), dim3(1024), 0, st, ma);
         else if (nt == 512) hipLaunchKernelGGL((fused_middle_kernel<D, 512>), dim3(B * Hq), dim3(512), 0, st, ma);

@@ -772,8 +772,13 @@ template <int D>
 VPlan mfma_v_plan(int B, int Hkv, int n_tokens) {
     VPlan p;
     p.tuned = true;
-    int k = 1;   // macro steps of 64 tokens per wave
-    while (k < 4 && (int64_t)B * Hkv * ((n_tokens + 512 * k - 1) / (512 * k)) >= 2048) k *= 2;
+    // Macro steps of 64 tokens per wave: as many as leave a workgroup for each of the 512 slots (two per compute unit), up
+    // to the four whose probabilities a lane keeps in registers.  A workgroup's first 4 to 5 us go by before its stream
+    // runs, so fewer and longer ones win: for 256 rows of 1024 / 2048 / 3072 / 4096 / 6144 tokens the pass takes
+    // 18.1 / 30.0 / 42.8 / 56.1 / 81.6 us with one step per wave, 15.3 / 21.6 / 30.8 / 39.1 / 56.0 with two and
+    // 21.4 / 23.1 / 27.2 / 32.7 / 44.5 with four (above four the pass leaves its fast path: 41.6 us with eight at 4096).
+    int k = 1;
+    while (k < 4 && (int64_t)B * Hkv * ((n_tokens + 1024 * k - 1) / (1024 * k)) >= 512) k *= 2;
     p.iters_per_wave = k;
     p.tokens_per_wave = 64 * k;
     p.chunk_tokens = 4 * p.tokens_per_wave;

@@ -16,7 +16,8 @@ struct StepGeom {
     int kb;                                          // tokens per K plane block (64 or 256)
     int cur_len;
     const int *seq_lens;
-    const u32 *task_map;   // per-sequence lengths: workgroup -> (chunk, head index, batch) of this launch, or null
+    // per-sequence lengths: workgroup -> {(chunk, head index, batch) of this launch, the sequence's length}, or null
+    const u32x2 *task_map;
 };
 
 // Launch shape of a pass: grid (grid_x, grid_y, batch), a workgroup covers tokens_per_wg tokens of one sequence.
@@ -43,17 +44,20 @@ __device__ __forceinline__ void seq_state(const StepGeom &g, int b, int &R, int 
 // past the end of the shorter ones would be scattered between the working ones, each holding a workgroup slot for
 // a microsecond or two (measured: +22 % on the K pass with two such out of three).  The step's first kernel
 // therefore writes a map from the linear workgroup index to the tasks that exist, in the same order; what is left
-// over gathers at the end of the launch and leaves at once.
-__device__ __forceinline__ bool step_block(const StepGeom &g, int &x, int &y, int &z) {
+// over gathers at the end of the launch and leaves at once.  An entry also carries the length of its sequence, which
+// replaces the look-up in g (the kernel's own copy): one dependent read less in front of a workgroup's first requests.
+__device__ __forceinline__ bool step_block(StepGeom &g, int &x, int &y, int &z) {
     x = blockIdx.x;
     y = blockIdx.y;
     z = blockIdx.z;
     if (g.task_map != nullptr) {
-        const u32 e = g.task_map[blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)];
-        if (e == kNoTask) return false;
-        x = (int)(e & 0xfffu);
-        y = (int)((e >> 12) & 0xffu);
-        z = (int)(e >> 20);
+        const u32x2 e = g.task_map[blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z)];
+        if (e.x == kNoTask) return false;
+        x = (int)(e.x & 0xfffu);
+        y = (int)((e.x >> 12) & 0xffu);
+        z = (int)(e.x >> 20);
+        g.cur_len = (int)e.y;
+        g.seq_lens = nullptr;
     }
     return true;
 }
