@@ -585,18 +585,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
 #pragma unroll
                 for (int u = 0; u < 4; ++u) load_bytes<CPP>(tile.h[u], rH, oh + u * D);
             };
-            KTaskTile<CPP> t[4];
-#pragma unroll
-            for (int i = 0; i < 3; ++i) issue_high(t[i], t_begin + 16 * i);
-            __builtin_amdgcn_sched_barrier(0);
             // ---- the list: (token, head) pairs below level 2; every lane notes those of its head ----
             unsigned short *list = fine_tok[wave];
             int n_fine = 0;
             // all probabilities of the lane's head for the wave's tokens in one round trip (they are the operands of the
-            // loop below as well): macro step mi, step s, tokens 4 kq + 0..3 -> bit 16 mi + 4 s + u of the lane's mask
+            // loop below as well): macro step mi, step s, tokens 4 kq + 0..3 -> bit 16 mi + 4 s + u of the lane's mask.
+            // Requested in front of the first tiles: loads come back in the order they were issued, and the list waits
+            // for the probabilities only.
             u32x2 pall[LIST / MACRO][4];
 #pragma unroll
             for (int mi = 0; mi < LIST / MACRO; ++mi) load_probs(pall[mi], t_begin + mi * MACRO);
+            __builtin_amdgcn_sched_barrier(0);
+            KTaskTile<CPP> t[4];
+#pragma unroll
+            for (int i = 0; i < 3; ++i) issue_high(t[i], t_begin + 16 * i);
             __builtin_amdgcn_sched_barrier(0);
             const u16x2 a2 = threshold_operand();
             const unsigned char amin = amin_loaded;
