@@ -334,7 +334,42 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && 
                                 as_f16x4(qa & m1a, qb & m1b), as_f16x4(qa & m2a, qb & m2b), puts);
             __builtin_amdgcn_sched_barrier(0);
         }
-        // lane (j, ig): acc[s][r] = score of slot s of token set 4 ig + r for query head j
+        // lane (j, ig): acc[s][r] = score of slot s of token set 4 ig + r for query head j.  Plain stores throughout: the
+        // scores are read by the step's next kernel.
+        if constexpr (SL == 16) {
+            // A head lane (j, ig) holds the 64 scores of block 4 task + ig for its head: one 128-byte line of the head's score
+            // row.  Stored from there, an instruction scatters sixteen 16-byte pieces over sixteen lines, and the 19 MB of
+            // scores cost the pass 7 us of 54 at batch 32, 32 over 8 heads, lengths 2048 to 8192 (47.1 us with the stores
+            // dropped; written through at device scope, as they were first, 56.7).  The lines go through LDS instead
+            // -- line (ig, head) at (ig * G + j) * 128 -- and eight consecutive lanes store a whole line, 16 bytes each:
+            // 53.2 us, whatever the cache policy of the stores (a wave still ends only when its stores are through).
+            __shared__ __attribute__((aligned(16))) u32x4 lines[4][64 * 8];   // per wave: up to 4 x 16 lines of 8 pieces
+            u32x4 *mine = lines[wave];
+            if (head) {
+                const int lam = (lane >> 4) * G + j;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    u32 pk[8];
+#pragma unroll
+                    for (int sl = 0; sl < 16; sl += 2)
+                        pk[sl >> 1] = (u32)float_to_half_bits(acc[sl][r] * scale) | ((u32)float_to_half_bits(acc[sl + 1][r] * scale) << 16);
+                    mine[lam * 8 + 2 * r] = (u32x4){pk[0], pk[1], pk[2], pk[3]};
+                    mine[lam * 8 + 2 * r + 1] = (u32x4){pk[4], pk[5], pk[6], pk[7]};
+                }
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // the lines are read by other lanes of the wave
+            const int n_lines = 4 * G;
+            for (int s0 = 0; s0 * 8 < n_lines; ++s0) {
+                const int lam = s0 * 8 + (lane >> 3);
+                const int ig = lam / G, h = lam - ig * G;
+                const int out_blk = task * NBT + ig;
+                const bool store = lam < n_lines && out_blk < n_blocks;
+                const u32x4 v = mine[lam * 8 + (lane & 7)];
+                const int off = store ? (int)(((bh0 + h) * geo.row_stride + out_blk * CB) * 2) + (lane & 7) * 16 : kSkip;
+                __builtin_amdgcn_raw_buffer_store_b128(v, rS, off, 0, 0);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // (read before the next task's lines are written)
+        } else {
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int ts = 4 * (lane >> 4) + r;
@@ -345,15 +380,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && 
             for (int sl = 0; sl < SL; sl += 2)
                 pk[sl >> 1] = (u32)float_to_half_bits(acc[sl][r] * scale) | ((u32)float_to_half_bits(acc[sl + 1][r] * scale) << 16);
             const int off = store ? (int)(((bh0 + j) * geo.row_stride + out_blk * CB + (ts % PB) * SL) * 2) : kSkip;
-            // device scope: the workgroup that runs the softmax for this (batch, head) may sit on another XCD
             if constexpr (SL == 4) {
-                __builtin_amdgcn_raw_buffer_store_b64((u32x2){pk[0], pk[1]}, rS, off, 0, kDeviceScope);
+                __builtin_amdgcn_raw_buffer_store_b64((u32x2){pk[0], pk[1]}, rS, off, 0, 0);
             } else {
-                __builtin_amdgcn_raw_buffer_store_b128((u32x4){pk[0], pk[1], pk[2], pk[3]}, rS, off, 0, kDeviceScope);
-                if constexpr (SL == 16)
-                    __builtin_amdgcn_raw_buffer_store_b128((u32x4){pk[4], pk[5], pk[6], pk[7]}, rS, store ? off + 16 : kSkip, 0,
-                                                           kDeviceScope);
+                __builtin_amdgcn_raw_buffer_store_b128((u32x4){pk[0], pk[1], pk[2], pk[3]}, rS, off, 0, 0);
             }
+        }
         }
     }
 }
