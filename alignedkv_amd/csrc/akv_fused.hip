@@ -661,6 +661,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     geo.kb = kb;
     geo.cur_len = cur_len; geo.seq_lens = seq_lens;
     geo.task_map = nullptr;
+    geo.scores_through = (int64_t)B * Hq * (cur_len + 1) * 2 > ((int64_t)4 << 20) ? 1 : 0;
 
     // flushed tokens after the append: exact for uniform lengths, an upper bound for ragged ones
     const int R = (cur_len + 1) / cb * cb;

@@ -15,6 +15,7 @@ struct StepGeom {
     int cb, max_seq_len, n_max_blocks, row_stride;   // cb: tokens per flush; n_max_blocks: K plane blocks of kb tokens
     int kb;                                          // tokens per K plane block (64 or 256)
     int cur_len;
+    int scores_through;    // K pass on 256-token blocks: scores are written through to memory (see k_pass256_split_block)
     const int *seq_lens;
     // per-sequence lengths: workgroup -> {(chunk, head index, batch) of this launch, the sequence's length}, or null
     const u32x2 *task_map;
