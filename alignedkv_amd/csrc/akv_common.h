@@ -173,6 +173,13 @@ constexpr int kStream = 1 << 1;
 __device__ __forceinline__ void store_u16_device(const __amdgpu_buffer_rsrc_t r, int byte_off, unsigned short v) {
     __builtin_amdgcn_raw_buffer_store_b16((short)v, r, byte_off, 0, kDeviceScope);
 }
+// A score of the K pass, read by a later kernel.  through: written through to memory at once; otherwise it stays in L2
+// until the kernel ends (cheaper while the scores of a launch are few: the wave's store is acknowledged sooner and the
+// write-back of a few dirty lines at the kernel's end costs less than writing next to the streaming reads).
+__device__ __forceinline__ void store_score(const __amdgpu_buffer_rsrc_t r, int byte_off, unsigned short v, bool through) {
+    if (through) __builtin_amdgcn_raw_buffer_store_b16((short)v, r, byte_off, 0, kDeviceScope);
+    else __builtin_amdgcn_raw_buffer_store_b16((short)v, r, byte_off, 0, 0);
+}
 __device__ __forceinline__ void store_f32_device(const __amdgpu_buffer_rsrc_t r, int byte_off, float v) {
     __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, byte_off, 0, kDeviceScope);
 }

@@ -108,7 +108,7 @@ template <int D>
 __device__ __forceinline__ void k_score_blocks(KHalfTile<D / 32> &ta, const uint8_t *f8, const uint8_t *m4,
                                                const uint8_t *l4, int n_blocks, int first_blk, int end_blk,
                                                const float *qf, u32 need_mid, u32 need_last, unsigned short *s_row,
-                                               float scale, int blk_stride = 1) {
+                                               float scale, int blk_stride = 1, bool through = true) {
     constexpr int CB = 64;
     constexpr int NG = D / 16;
     constexpr int HG = NG / 2;
@@ -143,8 +143,7 @@ __device__ __forceinline__ void k_score_blocks(KHalfTile<D / 32> &ta, const uint
         reduce_scatter_step<8>(acc, 16);
         reduce_scatter_step<4>(acc, 8);
         reduce_scatter_step<2>(acc, 4);
-        // device scope: the workgroup that runs the softmax for this (batch, head) may sit on another XCD
-        store_u16_device(rS, (blk * CB + slot) * 2, float_to_half_bits(acc[0] * scale));
+        store_score(rS, (blk * CB + slot) * 2, float_to_half_bits(acc[0] * scale), through);
     }
 }
 
@@ -154,7 +153,7 @@ __device__ __forceinline__ void k_score_blocks(KHalfTile<D / 32> &ta, const uint
 template <int D>
 __device__ __forceinline__ void k_score_block_whole(KHalfTile<D / 16> &t, const uint8_t *m4, const uint8_t *l4, int n_blocks,
                                                     int blk, const float *qf, u32 need_mid, u32 need_last,
-                                                    unsigned short *s_row, float scale) {
+                                                    unsigned short *s_row, float scale, bool through = true) {
     constexpr int CB = 64;
     constexpr int NG = D / 16;
     const int lane = threadIdx.x & 63;
@@ -173,8 +172,7 @@ __device__ __forceinline__ void k_score_block_whole(KHalfTile<D / 16> &t, const 
     reduce_scatter_step<8>(acc, 16);
     reduce_scatter_step<4>(acc, 8);
     reduce_scatter_step<2>(acc, 4);
-    // device scope: the workgroup that runs the softmax for this (batch, head) may sit on another XCD
-    store_u16_device(rS, (blk * CB + slot) * 2, float_to_half_bits(acc[0] * scale));
+    store_score(rS, (blk * CB + slot) * 2, float_to_half_bits(acc[0] * scale), through);
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -296,7 +296,7 @@ __global__ __launch_bounds__(256) void fused_k_pass_kernel(
             levels_out[(int64_t)bh * D + g * 16 + (lane >> 2)] = (uint8_t)lv;
     }
     k_score_blocks<D>(ta, first_8 + plane_off * 2, mid_4 + plane_off, last_4 + plane_off, n_blocks, first_blk, end_blk, qf,
-                      need_mid, need_last, scores + (int64_t)bh * geo.row_stride, scale);
+                      need_mid, need_last, scores + (int64_t)bh * geo.row_stride, scale, 1, geo.scores_through != 0);
 }
 
 // K pass over planes with 256-token blocks (multi-head): one workgroup per block, its four waves take a quarter of the

@@ -67,7 +67,7 @@ __device__ __forceinline__ void k_pass64_whole_blocks(
     }
     if (blk < n_blocks)
         k_score_block_whole<D>(ta, mid_4 + plane_off, last_4 + plane_off, n_blocks, blk, qf, need_mid, need_last,
-                               scores + (int64_t)bh * geo.row_stride, scale);
+                               scores + (int64_t)bh * geo.row_stride, scale, geo.scores_through != 0);
 }
 
 // K pass over one 256-token block `blk` of the (batch, head) row `bh` of planes with 256-token blocks, by a workgroup of
@@ -164,10 +164,8 @@ __device__ __forceinline__ void k_pass256_split_block(
             // is cheaper than writing them through while the planes stream as long as they are few: 31.3 instead of 32.0 us
             // for the pass at batch 8 x 32 heads x 4096 tokens (2 MB of scores), but 149.7 instead of 146.0 at 4 x 32 x 32768
             // (8 MB), so the host picks by their volume.
-            const __amdgpu_buffer_rsrc_t rS = make_rsrc(scores + (int64_t)bh * geo.row_stride, (u32)R * 2);
-            const unsigned short s16 = float_to_half_bits(sum * scale);
-            if (geo.scores_through) store_u16_device(rS, token * 2, s16);
-            else __builtin_amdgcn_raw_buffer_store_b16((short)s16, rS, token * 2, 0, 0);
+            store_score(make_rsrc(scores + (int64_t)bh * geo.row_stride, (u32)R * 2), token * 2, float_to_half_bits(sum * scale),
+                        geo.scores_through != 0);
         }
     }
 }
