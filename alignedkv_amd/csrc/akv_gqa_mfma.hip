@@ -620,18 +620,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
             // ---- the list: (token, head) pairs below level 2; every lane notes those of its head ----
             unsigned short *list = fine_tok[wave];
             int n_fine = 0;
-            // all probabilities of the lane's head for the wave's tokens in one round trip (they are the operands of the
-            // loop below as well): macro step mi, step s, tokens 4 kq + 0..3 -> bit 16 mi + 4 s + u of the lane's mask.
-            // Requested in front of the first tiles: loads come back in the order they were issued, and the list waits
-            // for the probabilities only.
-            u32x2 pall[LIST / MACRO][4];
+            // All probabilities of the group's heads for the wave's tokens in one round trip (they are the operands of the
+            // loop below as well), requested in front of the first tiles: loads come back in the order they were issued,
+            // and the list waits for the probabilities only.  They come as whole rows -- a request of the wave covers the
+            // 256 tokens of two heads, 16 bytes a lane -- and go through LDS into the operand layout (macro step mi, step s,
+            // tokens 4 kq + 0..3 of the lane's head): sixteen 8-byte requests per lane, a quarter of the lanes active,
+            // cost the pass 7.8 us of 38 at batch 32, 32 over 8 heads, lengths 2048 to 8192.
+            constexpr int PS = LIST + 16;       // halves between two heads' rows in LDS (the step keeps the reads off each other's banks)
+            __shared__ __attribute__((aligned(16))) unsigned short wave_probs[4][16 * PS];
+            unsigned short *wp = wave_probs[wave];
+            u32x4 prow[8];
+            {
+                const int tok = t_begin + (lane & 31) * 8;
 #pragma unroll
-            for (int mi = 0; mi < LIST / MACRO; ++mi) load_probs(pall[mi], t_begin + mi * MACRO);
+                for (int i = 0; i < 8; ++i) {
+                    const int h = 2 * i + (lane >> 5);
+                    prow[i] = __builtin_amdgcn_raw_buffer_load_b128(rP, (h < G && tok < t_end) ? (int)((bh0 + h) * geo.row_stride + tok) * 2 : kSkip, 0, 0);
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
             KTaskTile<CPP> t[4];
 #pragma unroll
             for (int i = 0; i < 3; ++i) issue_high(t[i], t_begin + 16 * i);
             __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                *reinterpret_cast<u32x4 *>(wp + (2 * i + (lane >> 5)) * PS + (lane & 31) * 8) = prow[i];
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // the rows are read by other lanes of the wave
+            u32x2 pall[LIST / MACRO][4];
+#pragma unroll
+            for (int mi = 0; mi < LIST / MACRO; ++mi)
+#pragma unroll
+                for (int sidx = 0; sidx < 4; ++sidx) {
+                    const u32x2 v = *reinterpret_cast<const u32x2 *>(wp + (head ? j : 0) * PS + mi * MACRO + 16 * sidx + 4 * kq);
+                    pall[mi][sidx] = head ? v : (u32x2){0u, 0u};
+                }
             const u16x2 a2 = threshold_operand();
             const unsigned char amin = amin_loaded;
             {
@@ -692,8 +715,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void m
                         load_bytes<CPP>(ct.h[u], rH, on ? tok * D + (lane & 15) * CPP : kSkip);
                         load_bytes<CPP / 2>(ct.m[u], rM, on ? tok * (D / 2) + (lane & 15) * (CPP / 2) : kSkip);
                         load_bytes<CPP / 2>(ct.l[u], rL, last ? tok * (D / 2) + (lane & 15) * (CPP / 2) : kSkip);
-                        cp[u] = (u32)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(
-                            rP, mine ? (int)((bh0 + j) * geo.row_stride + tok) * 2 : kSkip, 0, 0);
+                        cp[u] = mine ? (u32)wp[j * PS + (int)(entry & 0xffu)] : 0u;
                         c_mid |= (on ? 1u : 0u) << u;
                         c_last |= (last ? 1u : 0u) << u;
                     }
