@@ -468,7 +468,11 @@ struct VListed {
 // PREFETCHED: the caller has requested the first half tile's high bytes (v_prefetch_first); otherwise they are requested
 // here, behind the probabilities -- loads come back in the order they were issued, so the small loads that the fetch
 // levels depend on go first where nothing else has to happen in between.
-template <int D, bool REF, int NIT, int PAUX = 0, bool PREFETCHED = true>
+// PROWS: the probabilities of the wave's tokens are requested as one row (8 bytes a lane) and spread through LDS; for
+// callers whose rows are 8-byte aligned and whose token ranges are multiples of 4 (the fused step).  Otherwise every lane
+// requests its own, two bytes at a time: a wave-wide request then brings 64 / (D / 16) probabilities, 32 requests for
+// the 256 tokens of a wave at head_dim 128.
+template <int D, bool REF, int NIT, int PAUX = 0, bool PREFETCHED = true, bool PROWS = false>
 __device__ __forceinline__ void v_accumulate(VFirstTile<D> &ft, const uint8_t *f8, const uint8_t *m4, const uint8_t *l4,
                                              int n_tokens, const unsigned short *s_row, unsigned char amin, int t_begin,
                                              int t_end, float *acc, uint8_t *levels_row) {
@@ -486,6 +490,35 @@ __device__ __forceinline__ void v_accumulate(VFirstTile<D> &ft, const uint8_t *f
     // The probabilities of all the wave's tokens first: the fetch level of a token depends on its
     // probability, and a load per batch would put a memory round trip in front of every batch.
     u32 sb[NH][HV];
+    if constexpr (PROWS) {
+        constexpr int NK = NH * HV, NTOK = NK * TPL;      // loads and tokens per wave
+        static_assert(NTOK <= 256 && NK % 2 == 0, "one 8-byte request per lane covers the wave's tokens");
+        __shared__ __attribute__((aligned(16))) unsigned short prob_rows[4][TPL * NK];   // per wave: [token row of a load][load]
+        unsigned short *wp = prob_rows[threadIdx.x >> 6];
+        const int i0 = 4 * lane, t0 = t_begin + i0;
+        const u32x2 four = __builtin_amdgcn_raw_buffer_load_b64(rS, (i0 < NTOK && t0 < t_end) ? t0 * 2 : kSkip, 0, PAUX);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (!PREFETCHED) v_prefetch_first<D>(ft, f8, n_tokens, t_begin, t_end);
+        __builtin_amdgcn_sched_barrier(0);
+        if (i0 < NTOK) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int i = i0 + e;     // token i of the wave: row i % TPL of load i / TPL
+                wp[(i % TPL) * NK + i / TPL] = (unsigned short)(((e & 2) ? four.y : four.x) >> (16 * (e & 1)));
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // read by other lanes of the wave
+        u32 pw[NK / 2];
+#pragma unroll
+        for (int w = 0; w < NK / 2; ++w) pw[w] = *reinterpret_cast<const u32 *>(wp + tl * NK + 2 * w);
+#pragma unroll
+        for (int hf = 0; hf < NH; ++hf)
+#pragma unroll
+            for (int u = 0; u < HV; ++u) {
+                const int k = hf * HV + u;
+                sb[hf][u] = (pw[k >> 1] >> (16 * (k & 1))) & 0xffffu;
+            }
+    } else {
 #pragma unroll
     for (int hf = 0; hf < NH; ++hf)
 #pragma unroll
@@ -495,6 +528,7 @@ __device__ __forceinline__ void v_accumulate(VFirstTile<D> &ft, const uint8_t *f
         }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (!PREFETCHED) v_prefetch_first<D>(ft, f8, n_tokens, t_begin, t_end);
+    }
     // Software pipeline over half tiles (see k_score_blocks): one half tile is in flight while the other is
     // multiplied; sched_barrier(0) keeps the instruction scheduler from merging the phases.
     VHalfTile<HV> &ta = ft.t;

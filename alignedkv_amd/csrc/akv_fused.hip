@@ -577,7 +577,7 @@ __global__ __launch_bounds__(256) void fused_v_pass_kernel(
     float acc[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-    v_accumulate<D, REF, NIT, 0, false>(ft, first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
+    v_accumulate<D, REF, NIT, 0, false, true>(ft, first_8 + row0 * D, mid_4 + row0 * (D / 2), last_4 + row0 * (D / 2), n_tokens,
                                         probs + (int64_t)bh * geo.row_stride, amin, t_begin, t_end, acc,
                                         levels_out != nullptr ? levels_out + (int64_t)bh * levels_stride : nullptr);
     if (!REF && amin_out != nullptr && chunk == 0 && threadIdx.x == 0) amin_out[bh] = amin;
