@@ -328,7 +328,15 @@ __global__ __launch_bounds__(64 * NWV) void fused_k_pass256_split_kernel(
 template <int D, int NT>
 __global__ __launch_bounds__(NT) void fused_middle_kernel(MiddleArgs a) {
     __shared__ MiddleShared<D, NT / 64> ms;
-    middle_body<D, NT>(a, blockIdx.x, ms);
+    // Workgroups go to the 8 XCDs round-robin by index.  The G query heads of a KV head read the same rest-buffer rows
+    // and probe the same value rows: with indices 8 apart they meet in one XCD's L2.
+    int bh = blockIdx.x;
+    const int G = a.g.G, n_groups = (int)gridDim.x / G;
+    if (G > 1 && (n_groups & 7) == 0) {
+        const int t = bh >> 3;
+        bh = ((t / G) * 8 + (bh & 7)) * G + t % G;
+    }
+    middle_body<D, NT>(a, bh, ms);
 }
 
 constexpr int tail_rows_per_cu = 2, tail_max_tokens = 8192;
