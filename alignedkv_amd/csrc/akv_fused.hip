@@ -649,7 +649,8 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
                     const uint8_t *v_new, const uint8_t *mask, int mask_stride, uint8_t *out, uint8_t *scores,
                     uint8_t *probs, int row_stride, uint8_t *ws, uint8_t *k_levels_out, uint8_t *v_levels_out,
                     uint8_t *amin_out, int B, int Hq, int Hkv, int n_max_blocks, int max_seq_len, int cb, int kb, int top_k,
-                    int cur_len, int *seq_lens, bool ref, int literal_broadcast, hipStream_t st) {
+                    int cur_len, int *seq_lens, bool ref, int flags, hipStream_t st) {
+    const int literal_broadcast = flags & AKV_STEP_LITERAL_BROADCAST;
     const StepLayout lay = step_layout(B, Hq, D, max_seq_len);
     uint8_t *toe = ws + lay.toe;
     uint8_t *amin = ws + lay.amin;
@@ -764,6 +765,7 @@ static int run_step(uint8_t *kf8, uint8_t *km4, uint8_t *kl4, uint8_t *vf8, uint
     ma.scores = s16; ma.probs = p16; ma.otail = otail;
     ma.kcm = kcm; ma.vcm = vcm; ma.toe = toe; ma.amin = amin; ma.v_first_8 = vf8;
     ma.g = geo; ma.mask_stride = mask_stride; ma.top_k = top_k; ma.persist = persist;
+    ma.record_probs = (flags & AKV_STEP_NO_PROBS_RECORD) ? 0 : 1;
     mark(0, st);
     if (n_blocks > 0 && matrix) {
         int rc = AKV_OK;
@@ -992,7 +994,8 @@ extern "C" int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t
     AKV_REQUIRE(top_max_k == 32, "decode_step: top_max_k %d not supported by the fused step (32)", top_max_k);
     AKV_REQUIRE(bsz <= 65535 && n_kv_heads <= 65535, "decode_step: bsz/heads exceed the grid limit 65535");
     AKV_REQUIRE(cur_len >= 0 && cur_len + 1 <= max_seq_len, "decode_step: cache full (%d of %d tokens)", cur_len, max_seq_len);
-    AKV_REQUIRE(!literal_broadcast || (n_q_heads == n_kv_heads && seq_lens == nullptr),
+    AKV_REQUIRE((literal_broadcast & ~(AKV_STEP_LITERAL_BROADCAST | AKV_STEP_NO_PROBS_RECORD)) == 0, "decode_step: unknown flags %d", literal_broadcast);
+    AKV_REQUIRE(!(literal_broadcast & AKV_STEP_LITERAL_BROADCAST) || (n_q_heads == n_kv_heads && seq_lens == nullptr),
                 "decode_step: literal_broadcast is defined for multi-head caches of uniform length only");
     const int flushed = (cur_len + 1) / d_block * d_block;
     AKV_REQUIRE(flushed + d_block <= 65536 * 32, "decode_step: at most %d flushed tokens (16-bit group index of the probe)",

@@ -178,6 +178,7 @@ struct MiddleArgs {
     StepGeom g;
     int mask_stride;
     int top_k;
+    int record_probs;      // 0: the form of the step that keeps the probabilities on chip does not write them to `probs`
     int persist;  // this kernel appends the token (it is not in the rest buffers / planes yet)
 };
 
@@ -337,13 +338,15 @@ __device__ __forceinline__ void middle_body(const MiddleArgs &a, const int bh, M
     const bool in_regs = MAXTOK > 0 || nvec <= NT * VPT;
     // scores of the flushed part are read at device scope: other workgroups of the same launch wrote them
     const __amdgpu_buffer_rsrc_t rScores = make_rsrc(srow, (u32)R * 2);
+    // (SPLIT: the caller reads the probabilities from LDS; their copy in memory is a record for the host)
+    const bool to_memory = !SPLIT || a.record_probs != 0;
     auto store_probs8 = [&](int i, const u32x4 o) {
         if (probs_lds != nullptr) *reinterpret_cast<u32x4 *>(probs_lds + i * 8) = o;
-        *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
+        if (to_memory) *reinterpret_cast<u32x4 *>(prow + i * 8) = o;
     };
     auto store_prob1 = [&](int t, unsigned short p) {
         if (probs_lds != nullptr) probs_lds[t] = p;
-        prow[t] = p;
+        if (to_memory) prow[t] = p;
     };
 
     // Everything that does not depend on anything else is requested first: the score vectors of the

@@ -168,8 +168,9 @@ class _AlignedKVModule:
     def decode_step(self, k_planes, v_planes, k_exp_column_max, v_exp_column_max, restk, restv, q, k_new, v_new,
                     mask, out, scores, probs, bsz, n_kv_heads, n_max_blocks, max_seq_len, head_dim, d_block,
                     top_max_k, cur_len, rest_start, rest_len, reference, literal_broadcast,
-                    k_levels_out=None, v_levels_out=None, amin_out=None):
-        """All tensors as torch.uint8 views on one device; see akv_decode_step in include/alignedkv.h."""
+                    k_levels_out=None, v_levels_out=None, amin_out=None, record_probs=True):
+        """All tensors as torch.uint8 views on one device; see akv_decode_step in include/alignedkv.h.
+        record_probs=False: AKV_STEP_NO_PROBS_RECORD (probs may be left unwritten where the step does not need it)."""
         lib = load_library()
         dev = q.device
         kplane = bsz * n_kv_heads * n_max_blocks * head_dim * d_block
@@ -209,12 +210,12 @@ class _AlignedKVModule:
                                       row_stride, _ptr(ws), ws.numel(), _ptr(k_levels_out), _ptr(v_levels_out),
                                       _ptr(amin_out), bsz, n_kv_heads, n_max_blocks, max_seq_len, head_dim, d_block,
                                       top_max_k, cur_len, rest_start, rest_len, int(bool(reference)),
-                                      int(bool(literal_broadcast)), _stream_ptr(dev)), lib)
+                                      _step_flags(literal_broadcast, record_probs), _stream_ptr(dev)), lib)
 
     def decode_step_gqa(self, k_planes, v_planes, k_exp_column_max, v_exp_column_max, restk, restv, q, k_new, v_new,
                         mask, out, scores, probs, bsz, n_q_heads, n_kv_heads, n_max_blocks, max_seq_len, head_dim,
                         d_block, top_max_k, cur_len, seq_lens, reference, k_levels_out=None, v_levels_out=None,
-                        amin_out=None, k_block=None, literal_broadcast=False):
+                        amin_out=None, k_block=None, literal_broadcast=False, record_probs=True):
         """Fused step with grouped-query heads and optional per-sequence lengths (seq_lens: int32 device tensor
         [bsz], incremented by the step; cur_len then bounds them).  See akv_decode_step_gqa in include/alignedkv.h."""
         lib = load_library()
@@ -261,7 +262,12 @@ class _AlignedKVModule:
                                           row_stride, _ptr(ws), ws.numel(), _ptr(k_levels_out), _ptr(v_levels_out),
                                           _ptr(amin_out), bsz, n_q_heads, n_kv_heads, n_max_blocks, max_seq_len,
                                           head_dim, d_block, k_block, top_max_k, cur_len, _ptr(seq_lens),
-                                          int(bool(reference)), int(bool(literal_broadcast)), _stream_ptr(dev)), lib)
+                                          int(bool(reference)), _step_flags(literal_broadcast, record_probs), _stream_ptr(dev)), lib)
+
+
+def _step_flags(literal_broadcast, record_probs) -> int:
+    """flags of the fused step: AKV_STEP_LITERAL_BROADCAST = 1, AKV_STEP_NO_PROBS_RECORD = 2 (include/alignedkv.h)"""
+    return (1 if literal_broadcast else 0) | (0 if record_probs else 2)
 
 
 class PreparedDecodeStep:
@@ -284,7 +290,7 @@ class PreparedDecodeStep:
         self._keep = keep               # the tensors behind the pointers
 
     def __call__(self, q, k_new, v_new, out, mask, mask_stride, cur_len, reference, literal_broadcast,
-                 k_levels_out=None, v_levels_out=None, amin_out=None):
+                 k_levels_out=None, v_levels_out=None, amin_out=None, record_probs=True):
         tok = self._tok
         for t in (q, k_new, v_new, out):
             if t.numel() * t.element_size() != tok or not t.is_contiguous() or t.device != self.device:
@@ -292,7 +298,7 @@ class PreparedDecodeStep:
                                    f"{tok} bytes on {self.device}")
         rc = self._fn(self._desc_ref, q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(), _ptr(mask), mask_stride,
                       out.data_ptr(), _ptr(k_levels_out), _ptr(v_levels_out), _ptr(amin_out), cur_len, None,
-                      1 if reference else 0, 1 if literal_broadcast else 0, self.stream)
+                      1 if reference else 0, (1 if literal_broadcast else 0) | (0 if record_probs else 2), self.stream)
         if rc != 0:
             check(rc, self._lib)
 

@@ -69,6 +69,9 @@ class QuantizedCache_AlignedKV(_HFCache):
         # of ops and framework kernels (K op -> mask -> softmax -> probe op -> V op), kept for A/B checks.
         self.fused = self.head_dim in (64, 128, 256)
         self.literal_broadcast = literal_broadcast
+        # False: the fused step may leave the probabilities' record in memory (`_probs`) unwritten where it keeps them on
+        # chip (AKV_STEP_NO_PROBS_RECORD); nothing of the reference's API reads them
+        self.record_probabilities = True
         self._device = device
         # fp16 scratch rows of the fused step, one pair per stream: steps issued on different streams may overlap
         # (all layers of one stream share a pair, their steps are ordered)
@@ -86,7 +89,8 @@ class QuantizedCache_AlignedKV(_HFCache):
 
     @property
     def _probs(self):
-        """fp16 probabilities [B, H, width] the fused step last wrote on the current stream (debug output)."""
+        """fp16 probabilities [B, H, width] the fused step last wrote on the current stream (debug output; with
+        record_probabilities = False a step that keeps them on chip leaves this unwritten)."""
         return self._buffers()[1]
 
     def update(self, key_states, value_states, layer_idx, cache_kwargs=None):
@@ -187,9 +191,11 @@ class QuantizedCache_AlignedKV(_HFCache):
         # (the step takes the fp16 tensors as they are: it reads their bytes)
         if q.device.index != torch.cuda.current_device():
             with torch.cuda.device(q.device):
-                step(q, k, v, out, mask2d, mask_stride, start_pos, self.reference, self.literal_broadcast, klv, vlv, amin)
+                step(q, k, v, out, mask2d, mask_stride, start_pos, self.reference, self.literal_broadcast, klv, vlv, amin,
+                     self.record_probabilities)
         else:
-            step(q, k, v, out, mask2d, mask_stride, start_pos, self.reference, self.literal_broadcast, klv, vlv, amin)
+            step(q, k, v, out, mask2d, mask_stride, start_pos, self.reference, self.literal_broadcast, klv, vlv, amin,
+                 self.record_probabilities)
         kc._advance_after_fused_step()
         vc._advance_after_fused_step()
         if klv is not None:

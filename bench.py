@@ -136,7 +136,9 @@ class StepRunner:
     """Pre-marshalled akv_decode_step_gqa call (multi-head, uniform length) for one layer at a fixed state
     (cur_len = cache_len)."""
 
-    def __init__(self, torch, lib, cache, layer, q, k_new, v_new, out, reference, record):
+    def __init__(self, torch, lib, cache, layer, q, k_new, v_new, out, reference, record, record_probs=False):
+        # record_probs False: AKV_STEP_NO_PROBS_RECORD, the probabilities are not copied to memory where the step keeps them on
+        # chip (nothing reads them; outputs, fetch levels and thresholds are what the bench checks)
         from alignedkv_amd.extension._plane_cache import column_block
         self.lib = lib
         kc, vc = cache.key_cache[layer], cache.value_cache[layer]
@@ -157,7 +159,7 @@ class StepRunner:
                      p(q), p(k_new), p(v_new), None, 0, p(out), p(self.scores), p(self.probs), width, p(self.ws),
                      self.ws.numel(), p(self.k_levels), p(self.v_levels), p(self.amin), B, H, H, kc.k_n_max_blocks,
                      cache.max_cache_len, D, column_block, kc.k_block, vc.top_max_k, kc.current_cache_len, None,
-                     int(reference), 0, torch.cuda.current_stream().cuda_stream]
+                     int(reference), 0 if record_probs else 2, torch.cuda.current_stream().cuda_stream]
 
         self.cur_len_index = len(self.args) - 5
 
@@ -265,7 +267,9 @@ def phase_times(torch, lib, runners, steps):
 def algorithmic_bytes(k_levels, v_levels, B, H, D, R, L, top_k=32):
     """Bytes one decode step has to move given the fetch levels (0: all planes, 1: no last_4, 2: high byte
     only): per plane element 1 + 1/2 [level < 2] + 1/2 [level == 0] bytes, plus the fp16 tail, q, the
-    score/probability rows and the probe rows.  Dense fp16 reads 2 bytes per K and per V element."""
+    score row written by the K side and one row of the same size read by the V side (the scores, where the
+    probabilities stay on chip; the probabilities, where a kernel of its own turns the scores into them) and the
+    probe rows.  Dense fp16 reads 2 bytes per K and per V element."""
     tail = L - R
     k_plane = float(R) * (k_levels.size + 0.5 * (k_levels < 2).sum() + 0.5 * (k_levels == 0).sum())
     v_plane = float(D) * (v_levels.size + 0.5 * (v_levels < 2).sum() + 0.5 * (v_levels == 0).sum())
@@ -748,8 +752,11 @@ def main():
         torch.cuda.synchronize()
         res["avg_us_over_64_growing_steps"] = round((time.perf_counter() - t0) / (64 * a.layers) * 1e6, 2)
     # the same steps through the reference's host API (QuantizedCache_AlignedKV.auto_compute), beside the raw C-ABI figure
+    res["probabilities_recorded"] = False      # (AKV_STEP_NO_PROBS_RECORD in every timed step: see StepRunner)
     if not a.profile_run:
+        cache.record_probabilities = False
         api_us, api_host_us = time_api_path(torch, cache, q, k_new, v_new, L, max(a.steps, 400))
+        cache.record_probabilities = True
         res["us_per_step_via_auto_compute"] = round(api_us, 2)
         res["host_us_per_auto_compute_call"] = round(api_host_us, 2)
     if not a.no_extras and not a.no_cpu and (B, H, D, L) == (8, 32, 128, 4096):

@@ -141,10 +141,15 @@ AKV_API int akv_v_cache_compute(const uint8_t *first_8, const uint8_t *mid_4, co
  * row_stride >= flushed tokens + d_block.
  * k_levels_out uint8 [bsz,heads,head_dim], v_levels_out uint8 [bsz,heads,flushed tokens], amin_out uint8
  * [bsz,heads]: optional (NULL) records of the fetch decisions.
- * literal_broadcast != 0 reproduces the reference's threshold indexing as written
- * (extension/v_cache_file.py:157-160 broadcasts [B,H,1,D] against [B,1,H,D]).
+ * flags: AKV_STEP_LITERAL_BROADCAST reproduces the reference's threshold indexing as written
+ * (extension/v_cache_file.py:157-160 broadcasts [B,H,1,D] against [B,1,H,D]); AKV_STEP_NO_PROBS_RECORD lets the step
+ * leave `probs` unwritten where no kernel of the step reads it back (the form of the step that keeps a row's
+ * probabilities on chip: 2 MB of stores, 0.7 us, at batch 8 x 32 heads x 4096 tokens) -- `probs` is still required,
+ * the other forms use it as scratch, and its contents are then unspecified.
  * Supported: head_dim 64/128/256, d_block 64, top_max_k 32; other shapes go through the five ops.
  */
+#define AKV_STEP_LITERAL_BROADCAST 1
+#define AKV_STEP_NO_PROBS_RECORD 2
 AKV_API size_t akv_decode_step_workspace_bytes(int bsz, int n_q_heads, int head_dim, int max_seq_len);
 AKV_API int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_last_4, uint8_t *v_first_8,
                             uint8_t *v_mid_4, uint8_t *v_last_4, uint8_t *k_exp_column_max,
@@ -154,7 +159,7 @@ AKV_API int akv_decode_step(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k_las
                             size_t workspace_bytes, uint8_t *k_levels_out, uint8_t *v_levels_out, uint8_t *amin_out,
                             int bsz, int n_kv_heads, int n_max_blocks, int max_seq_len, int head_dim, int d_block,
                             int top_max_k, int cur_len, int rest_start, int rest_len, int reference,
-                            int literal_broadcast, akv_stream_t stream);
+                            int flags, akv_stream_t stream);
 
 /*
  * akv_decode_step for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
@@ -179,7 +184,7 @@ AKV_API int akv_decode_step_static(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t
                                    uint8_t *k_levels_out, uint8_t *v_levels_out, uint8_t *amin_out,
                                    int bsz, int n_kv_heads, int n_max_blocks, int max_seq_len, int head_dim, int d_block,
                                    int top_max_k, int cur_len, int rest_start, int rest_len, int reference,
-                                   int literal_broadcast, akv_stream_t stream);
+                                   int flags, akv_stream_t stream);
 
 /*
  * The fused decode step for grouped-query attention and per-sequence lengths; beyond the reference, which
@@ -205,7 +210,7 @@ AKV_API int akv_decode_step_gqa(uint8_t *k_first_8, uint8_t *k_mid_4, uint8_t *k
                                 size_t workspace_bytes, uint8_t *k_levels_out, uint8_t *v_levels_out, uint8_t *amin_out,
                                 int bsz, int n_q_heads, int n_kv_heads, int n_max_blocks, int max_seq_len, int head_dim,
                                 int d_block, int k_block, int top_max_k, int cur_len, int *seq_lens, int reference,
-                                int literal_broadcast, akv_stream_t stream);
+                                int flags, akv_stream_t stream);
 
 /*
  * akv_decode_step_gqa with everything that stays the same from step to step of one layer gathered in a descriptor the
@@ -225,7 +230,7 @@ typedef struct akv_step_desc {
 AKV_API int akv_decode_step_desc(const akv_step_desc *desc, const uint8_t *q, const uint8_t *k_new, const uint8_t *v_new,
                                  const uint8_t *mask, int mask_stride, uint8_t *out, uint8_t *k_levels_out,
                                  uint8_t *v_levels_out, uint8_t *amin_out, int cur_len, int *seq_lens, int reference,
-                                 int literal_broadcast, akv_stream_t stream);
+                                 int flags, akv_stream_t stream);
 
 /*
  * Dense fp16 decode attention, the baseline of the benchmark (semantics of the reference's dense branch,

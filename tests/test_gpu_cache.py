@@ -371,6 +371,52 @@ def test_two_launch_step_matches_the_four_launch_step(monkeypatch, reference, sw
     lib.akv_reload_tuning()
 
 
+@pytest.mark.parametrize("tail", ["1", "0"])
+def test_step_without_the_record_of_the_probabilities(monkeypatch, tail):
+    """record_probabilities = False (AKV_STEP_NO_PROBS_RECORD): the two-launch form of the step keeps a row's probabilities
+    on chip and then leaves `_probs` as it was; the four-launch form needs them in memory and writes them whatever the flag
+    says.  Outputs, fetch levels, thresholds and planes are the same bits as with the record, step after step (across
+    the flush at 192 tokens)."""
+    from alignedkv_amd import load_library
+    from alignedkv_amd.model.KVCache_AlignedKV import QuantizedCache_AlignedKV
+    lib = load_library()
+    B, H, D, prefill, steps = 2, 8, 128, 150, 60
+    q, k, v = make_qkv(B, prefill + steps, H, D, seed=31)
+    rng = np.random.default_rng(5)
+    caches = []
+    for record in (True, False):
+        c = QuantizedCache_AlignedKV(cfg(H, D), B, prefill + steps + 64, "cuda", torch.half, k_block=256)
+        c.record_probabilities = record
+        c.key_cache[0].save(dev(k[:, :prefill]), 0, prefill)
+        c.value_cache[0].save(dev(v[:, :prefill]), 0, prefill)
+        c.key_cache[0].record_levels = c.value_cache[0].record_levels = True
+        caches.append(c)
+    monkeypatch.setenv("AKV_TUNE_TAIL", tail)
+    lib.akv_reload_tuning()
+    try:
+        for t in range(prefill, prefill + steps):
+            qt = dev(rng.standard_normal((B, 1, H, D)).astype(np.float16))
+            if caches[1]._probs is not None:
+                caches[1]._probs.fill_(-7.0)          # (a value no probability takes)
+            want = caches[0].auto_compute(qt, dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None)
+            got = caches[1].auto_compute(qt, dev(k[:, t:t + 1]), dev(v[:, t:t + 1]), 0, None)
+            assert torch.equal(got, want), f"token {t}"
+            assert torch.equal(caches[0].value_cache[0].last_levels, caches[1].value_cache[0].last_levels)
+            assert torch.equal(caches[0].value_cache[0].last_alignment_min, caches[1].value_cache[0].last_alignment_min)
+            assert torch.equal(caches[0].key_cache[0].last_levels, caches[1].key_cache[0].last_levels)
+            if t > prefill:
+                if tail == "1":
+                    assert (caches[1]._probs[:, :, :t + 1] == -7.0).all(), "the record was written although it was switched off"
+                else:
+                    assert torch.equal(caches[1]._probs[:, :, :t + 1], caches[0]._probs[:, :, :t + 1])
+    finally:
+        monkeypatch.delenv("AKV_TUNE_TAIL")
+        lib.akv_reload_tuning()
+    for i, j in zip(caches[0].key_cache[0].__dict__.items(), caches[1].key_cache[0].__dict__.items()):
+        if isinstance(i[1], torch.Tensor) and i[0].startswith("k_cache"):
+            assert torch.equal(i[1], j[1]), i[0]
+
+
 def _stagewise_shapes(seed, n):
     rng = np.random.default_rng(seed)
     for _ in range(n):
