@@ -342,7 +342,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(SL == 8 && 
             // scores cost the pass 7 us of 54 at batch 32, 32 over 8 heads, lengths 2048 to 8192 (47.1 us with the stores
             // dropped; written through at device scope, as they were first, 56.7).  The lines go through LDS instead
             // -- line (ig, head) at (ig * G + j) * 128 -- and eight consecutive lanes store a whole line, 16 bytes each:
-            // 53.2 us, whatever the cache policy of the stores (the 10 MB of writes cost what they cost next to the reads: 47.7 us with the stores aimed at a region that stays in L2).
+            // 53.2 us and 9.5 MiB written, whatever the cache policy of the stores.  (The rest is what 10 MB of writes
+            // cost next to the reads: 47.7 us with the same stores aimed at a region that stays in L2.)
             __shared__ __attribute__((aligned(16))) u32x4 lines[4][64 * 8];   // per wave: up to 4 x 16 lines of 8 pieces
             u32x4 *mine = lines[wave];
             if (head) {
